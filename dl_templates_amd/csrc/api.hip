@@ -1,0 +1,189 @@
+// extern "C" surface of libdlt_hip.so: argument validation and translation of the
+// reference's call signatures into the attention-core problem description.
+#include "dlt_internal.hpp"
+#include <string.h>
+
+static thread_local char g_err[512] = "";
+
+int dlt_set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+extern "C" const char* dlt_last_error(void) { return g_err; }
+extern "C" int dlt_version(void) { return 1; }
+
+namespace {
+
+__global__ void swa_neighbors_kernel(DltGeom g, uint8_t* mask) {
+  // one thread per (query tile, kv tile): the same dlt_key_range the attention kernels call
+  const int T = g.TR * g.TC;
+  const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= (int64_t)T * T) return;
+  const int qi = (int)(id / T), kj = (int)(id - (int64_t)qi * T);
+  const int qr = qi / g.TC, qc = qi - qr * g.TC;
+  const int kr = kj / g.TC, kc = kj - kr * g.TC;
+  int rlo, rhi, xlo, xhi;
+  dlt_key_range(g, qr, qc * g.S, rlo, rhi, xlo, xhi);
+  const int kx = kc * g.S;
+  mask[id] = (uint8_t)((kr >= rlo && kr <= rhi && kx >= xlo && kx < xhi) ? 1 : 0);
+}
+
+bool is_dtype(int d) { return d == DLT_BF16 || d == DLT_FP16 || d == DLT_FP32; }
+
+int check_ptrs(const char* who, const void* const* ptrs, const int64_t* const* strides, int n) {
+  for (int i = 0; i < n; i++) {
+    DLT_REQUIRE(ptrs[i] != nullptr, "%s: tensor argument %d is NULL", who, i);
+    DLT_REQUIRE(strides[i] != nullptr, "%s: stride argument %d is NULL", who, i);
+  }
+  return DLT_OK;
+}
+
+int swa_problem(const char* who, const dlt_swa_shape_t* s, const dlt_rope_t* rope, AttnProblem& p) {
+  DLT_REQUIRE(s != nullptr, "%s: shape is NULL", who);
+  DLT_REQUIRE(is_dtype(s->dtype), "%s: bad dtype %d", who, s->dtype);
+  DLT_REQUIRE(s->B > 0 && s->H > 0, "%s: B=%d H=%d must be positive", who, s->B, s->H);
+  DLT_REQUIRE(s->b_size > 0 && s->t_height > 0 && s->t_width > 0, "%s: b_size=%d t_height=%d t_width=%d must be positive",
+              who, s->b_size, s->t_height, s->t_width);
+  DLT_REQUIRE(s->row_size >= 0 && s->col_size >= 0, "%s: negative window (%d, %d)", who, s->row_size, s->col_size);
+  DLT_REQUIRE(s->dk > 0 && s->dv > 0, "%s: dk=%d dv=%d must be positive", who, s->dk, s->dv);
+  DLT_REQUIRE((int64_t)s->t_height * s->t_width * s->b_size <= 0x3fffffff, "%s: too many tokens", who);
+  p.g.mode = DLT_GEOM_SWA;
+  p.g.TR = s->t_height;
+  p.g.TC = s->t_width;
+  p.g.S = s->b_size;
+  p.g.XLq = p.g.XLk = s->t_width * s->b_size;
+  p.g.WR = dlt_imin(s->row_size, s->t_height);
+  p.g.WC = dlt_imin(s->col_size, s->t_width);
+  p.B = s->B; p.H = s->H; p.dk = s->dk; p.dv = s->dv; p.sm_scale = s->sm_scale; p.dtype = s->dtype;
+  if (rope != nullptr) {
+    int rc = dlt_validate_rope(rope, s->dk);
+    if (rc != DLT_OK) return rc;
+  }
+  p.rope = dlt_make_rope_dev(rope, 0);
+  return DLT_OK;
+}
+
+int flash_problem(const char* who, const dlt_flash_shape_t* s, AttnProblem& p) {
+  DLT_REQUIRE(s != nullptr, "%s: shape is NULL", who);
+  DLT_REQUIRE(is_dtype(s->dtype), "%s: bad dtype %d", who, s->dtype);
+  DLT_REQUIRE(s->B > 0 && s->H > 0 && s->Lq > 0 && s->Lk > 0, "%s: B=%d H=%d Lq=%d Lk=%d must be positive", who, s->B, s->H, s->Lq, s->Lk);
+  DLT_REQUIRE(s->dk > 0 && s->dv > 0, "%s: dk=%d dv=%d must be positive", who, s->dk, s->dv);
+  DLT_REQUIRE(!s->causal || s->Lq == s->Lk, "%s: causal attention needs Lq == Lk (got %d, %d)", who, s->Lq, s->Lk);
+  p.g.mode = s->causal ? DLT_GEOM_CAUSAL : DLT_GEOM_DENSE;
+  p.g.TR = 1; p.g.TC = 1; p.g.S = 1; p.g.WR = 0; p.g.WC = 0;
+  p.g.XLq = s->Lq; p.g.XLk = s->Lk;
+  p.B = s->B; p.H = s->H; p.dk = s->dk; p.dv = s->dv; p.sm_scale = s->sm_scale; p.dtype = s->dtype;
+  p.rope = dlt_make_rope_dev(nullptr, 0);
+  return DLT_OK;
+}
+
+void cp4(int64_t* d, const int64_t* s) { for (int i = 0; i < 4; i++) d[i] = s[i]; }
+void cp3(int64_t* d, const int64_t* s) { for (int i = 0; i < 3; i++) d[i] = s[i]; }
+
+int fill_fwd(const char* who, AttnTensors& t, const void* q, const int64_t* qs, const void* k, const int64_t* ks,
+             const void* v, const int64_t* vs, void* o, const int64_t* os, float* lse, const int64_t* ls) {
+  const void* const ptrs[] = {q, k, v, o, lse};
+  const int64_t* const st[] = {qs, ks, vs, os, ls};
+  int rc = check_ptrs(who, ptrs, st, 5);
+  if (rc != DLT_OK) return rc;
+  memset(&t, 0, sizeof(t));
+  t.q = q; t.k = k; t.v = v; t.out_o = o; t.lse = lse;
+  cp4(t.qs, qs); cp4(t.ks, ks); cp4(t.vs, vs); cp4(t.os, os); cp3(t.ls, ls);
+  return DLT_OK;
+}
+
+int fill_bwd(const char* who, AttnTensors& t, const void* q, const int64_t* qs, const void* k, const int64_t* ks,
+             const void* v, const int64_t* vs, const void* o, const int64_t* os, const void* d_o, const int64_t* dos,
+             const float* lse, float* delta, const int64_t* ls, void* dq, const int64_t* dqs, void* dk,
+             const int64_t* dks, void* dv, const int64_t* dvs) {
+  const void* const ptrs[] = {q, k, v, o, d_o, lse, delta, dq, dk, dv};
+  const int64_t* const st[] = {qs, ks, vs, os, dos, ls, ls, dqs, dks, dvs};
+  int rc = check_ptrs(who, ptrs, st, 10);
+  if (rc != DLT_OK) return rc;
+  memset(&t, 0, sizeof(t));
+  t.q = q; t.k = k; t.v = v; t.o = o; t.d_o = d_o; t.lse = const_cast<float*>(lse); t.delta = delta;
+  t.dq = dq; t.dk = dk; t.dv = dv;
+  cp4(t.qs, qs); cp4(t.ks, ks); cp4(t.vs, vs); cp4(t.os, os); cp4(t.dos, dos);
+  cp4(t.dqs, dqs); cp4(t.dks, dks); cp4(t.dvs, dvs); cp3(t.ls, ls);
+  return DLT_OK;
+}
+
+}  // namespace
+
+extern "C" int dlt_swa_neighbors(int32_t t_height, int32_t t_width, int32_t row_size, int32_t col_size,
+                                 uint8_t* mask, void* stream) {
+  DLT_REQUIRE(t_height > 0 && t_width > 0 && row_size >= 0 && col_size >= 0, "swa_neighbors: bad grid/window");
+  DLT_REQUIRE(mask != nullptr, "swa_neighbors: mask is NULL");
+  const int64_t T = (int64_t)t_height * t_width;
+  DLT_REQUIRE(T * T <= ((int64_t)1 << 36), "swa_neighbors: grid too large for a dense mask");
+  DltGeom g;
+  g.mode = DLT_GEOM_SWA; g.TR = t_height; g.TC = t_width; g.S = 1; g.XLq = g.XLk = t_width;
+  g.WR = dlt_imin(row_size, t_height); g.WC = dlt_imin(col_size, t_width);
+  hipLaunchKernelGGL(swa_neighbors_kernel, dim3((unsigned)((T * T + 255) / 256)), dim3(256), 0, (hipStream_t)stream, g, mask);
+  DLT_CHECK_LAUNCH("swa_neighbors launch");
+  return DLT_OK;
+}
+
+extern "C" int dlt_swa_fwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                           const void* v, const int64_t v_strides[4], void* o, const int64_t o_strides[4],
+                           float* lse2, const int64_t lse_strides[3],
+                           const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream) {
+  AttnProblem p;
+  int rc = swa_problem("swa_fwd", shape, rope, p);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  rc = fill_fwd("swa_fwd", t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, lse2, lse_strides);
+  if (rc != DLT_OK) return rc;
+  return dlt_attn_forward(p, t, (hipStream_t)stream);
+}
+
+extern "C" int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                           const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],
+                           const void* d_o, const int64_t do_strides[4],
+                           const float* lse2, float* delta, const int64_t lse_strides[3],
+                           void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                           void* dv, const int64_t dv_strides[4],
+                           const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream) {
+  AttnProblem p;
+  int rc = swa_problem("swa_bwd", shape, rope, p);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  rc = fill_bwd("swa_bwd", t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, d_o, do_strides, lse2, delta,
+                lse_strides, dq, dq_strides, dk, dk_strides, dv, dv_strides);
+  if (rc != DLT_OK) return rc;
+  return dlt_attn_backward(p, t, (hipStream_t)stream);
+}
+
+extern "C" int dlt_flash_fwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                             const void* v, const int64_t v_strides[4], void* o, const int64_t o_strides[4],
+                             float* lse2, const int64_t lse_strides[3],
+                             const dlt_flash_shape_t* shape, void* stream) {
+  AttnProblem p;
+  int rc = flash_problem("flash_fwd", shape, p);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  rc = fill_fwd("flash_fwd", t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, lse2, lse_strides);
+  if (rc != DLT_OK) return rc;
+  return dlt_attn_forward(p, t, (hipStream_t)stream);
+}
+
+extern "C" int dlt_flash_bwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                             const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],
+                             const void* d_o, const int64_t do_strides[4],
+                             const float* lse2, float* delta, const int64_t lse_strides[3],
+                             void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                             void* dv, const int64_t dv_strides[4],
+                             const dlt_flash_shape_t* shape, void* stream) {
+  AttnProblem p;
+  int rc = flash_problem("flash_bwd", shape, p);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  rc = fill_bwd("flash_bwd", t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, d_o, do_strides, lse2, delta,
+                lse_strides, dq, dq_strides, dk, dk_strides, dv, dv_strides);
+  if (rc != DLT_OK) return rc;
+  return dlt_attn_backward(p, t, (hipStream_t)stream);
+}

@@ -1,0 +1,60 @@
+// Internal declarations shared by the translation units of libdlt_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/dlt.h"
+#include "dlt_geom.h"
+
+// ---- error reporting ---------------------------------------------------------------
+int dlt_set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define DLT_REQUIRE(cond, ...)                                   \
+  do {                                                           \
+    if (!(cond)) return dlt_set_error(DLT_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+#define DLT_CHECK_LAUNCH(what)                                                              \
+  do {                                                                                      \
+    hipError_t e__ = hipGetLastError();                                                     \
+    if (e__ != hipSuccess)                                                                  \
+      return dlt_set_error(DLT_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e__));         \
+  } while (0)
+
+static inline int dlt_elem_size(int dtype) { return dtype == DLT_FP32 ? 4 : 2; }
+
+// ---- rotary operands as the kernels see them ------------------------------------------
+struct RopeDev {
+  const int32_t* idx;
+  const float* row_cs;
+  const float* col_cs;
+  int64_t rs0, cs0;
+  int32_t R, row_len, col_len;
+  int32_t inverse;
+  int32_t enabled;
+};
+
+int dlt_validate_rope(const dlt_rope_t* rope, int64_t n_dim);
+RopeDev dlt_make_rope_dev(const dlt_rope_t* rope, int inverse);
+
+// ---- attention core (attn_fwd.hip / attn_bwd.hip) -------------------------------------
+struct AttnTensors {
+  const void *q, *k, *v, *o, *d_o;
+  void *out_o, *dq, *dk, *dv;
+  float* lse;        // written by forward, read by backward
+  float* delta;      // scratch written by the backward pre-pass
+  int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+};
+
+struct AttnProblem {
+  DltGeom g;
+  int32_t B, H, dk, dv;
+  float sm_scale;
+  int32_t dtype;
+  RopeDev rope;
+};
+
+int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream);
+int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream);

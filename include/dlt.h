@@ -1,0 +1,147 @@
+/*
+ * dlt.h - C ABI of libdlt_hip.so: the MI355X (gfx950) attention hot path of dl_templates.
+ *
+ * Conventions shared by every entry point
+ *   - returns DLT_OK (0) or a DLT_ERR_* code; dlt_last_error() gives the message of the
+ *     last failing call made by the calling thread (thread-local, never NULL);
+ *   - every data pointer is a DEVICE pointer owned by the caller; the library allocates
+ *     no device memory, never synchronises and keeps no state between calls, so calls
+ *     are re-entrant (forward on the caller thread, backward on the autograd thread);
+ *   - strides are in ELEMENTS (int64), tensors are [B, H, N, D] unless said otherwise;
+ *   - `stream` is a hipStream_t (NULL = the default stream); work is only enqueued;
+ *   - arguments are validated on the host before anything is launched: a call that
+ *     returns an error has launched nothing.
+ */
+#ifndef DLT_H
+#define DLT_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DLT_OK 0
+#define DLT_ERR_INVALID 1     /* bad shape / pointer / stride / enum            */
+#define DLT_ERR_UNSUPPORTED 2 /* valid request the kernels do not cover (yet)   */
+#define DLT_ERR_LAUNCH 3      /* the HIP runtime reported an error on launch    */
+
+/* element type of q/k/v/o and their gradients; arithmetic is bf16 (fp16 for DLT_FP16)
+ * MFMA with fp32 accumulation, fp32 inputs are rounded to bf16 when staged. */
+typedef enum { DLT_BF16 = 0, DLT_FP16 = 1, DLT_FP32 = 2 } dlt_dtype_t;
+
+const char* dlt_last_error(void);
+int dlt_version(void);
+
+/* ---- 2D rotary encoding -------------------------------------------------------------
+ * Per-token packed index and the two cos/sin tables, exactly the operands of
+ * RotaryPE2D.forward (src/fused_rope2d.py:126-141): idx[n] = (row << 16) | col,
+ * an axis whose signed 16-bit value is negative is not rotated (:40-45, :215-219);
+ * tables are fp32 [len, R, 2] with (cos, sin) innermost (:22-23, :238-240) and
+ * `*_stride0` elements between table rows (cs_stride0, :29,141).  Indices are clamped
+ * to [0, len-1] instead of reading out of bounds. */
+typedef struct {
+  const int32_t* idx;
+  const float* row_cs;
+  const float* col_cs;
+  int64_t row_cs_stride0;
+  int64_t col_cs_stride0;
+  int32_t n_rdim;  /* R: dims [0,R)x[R,2R) use the row angle, [2R,3R)x[3R,4R) the column angle */
+  int32_t row_len; /* number of rows of row_cs */
+  int32_t col_len;
+} dlt_rope_t;
+
+/* In-place rotation of x[B', N, C] (any strides).  Replaces rope2d_fwd_kernel
+ * (src/fused_rope2d.py:24-72) when inverse == 0 and rope2d_bwd_kernel (:74-122, the
+ * transposed rotation applied to a gradient) when inverse != 0.  No-PE semantics follow
+ * rope2d_ref (:204-225): an unrotated axis leaves its dims bit-identical. */
+int dlt_rope2d(void* x, const int64_t x_strides[3], int64_t n_batch, int64_t n_tokens, int64_t n_dim,
+               const dlt_rope_t* rope, int inverse, int dtype, void* stream);
+
+/* The same rotation applied to two tensors (q and k of one attention call) in ONE launch;
+ * both share idx/tables, N and C.  Replaces two back-to-back RotaryPE2D launches
+ * (README.md:11 composition; src/fused_rope2d.py:197-201 called once per tensor). */
+int dlt_rope2d_pair(void* x0, const int64_t x0_strides[3], int64_t n_batch0,
+                    void* x1, const int64_t x1_strides[3], int64_t n_batch1,
+                    int64_t n_tokens, int64_t n_dim,
+                    const dlt_rope_t* rope, int inverse, int dtype, void* stream);
+
+/* Debug export: bits[n] = (row >= 0) | (col >= 0) << 1, computed by the SAME device code
+ * the rotation kernels use to decode idx (src/fused_rope2d.py:40-45). */
+int dlt_rope_pe_mask(const int32_t* idx, int64_t n_tokens, uint8_t* bits, void* stream);
+
+/* ---- tiled 2D sliding-window attention -------------------------------------------------
+ * Scalars of TiledSwa.forward (src/tiled_swa.py:604): token n = (r * t_width + c) * b_size + s;
+ * query tile (r, c) attends kv tile (r', c') iff |r-r'| <= row_size and |c-c'| <= col_size,
+ * truncated at the grid border (:701-713). */
+typedef struct {
+  int32_t B, H;
+  int32_t b_size, t_height, t_width, row_size, col_size;
+  int32_t dk, dv; /* q/k head dim, v/o head dim */
+  float sm_scale;
+  int32_t dtype;  /* dlt_dtype_t */
+} dlt_swa_shape_t;
+
+/* Forward: o = softmax_window(q k^T * sm_scale) v, lse2 = log2 sum exp2(.) in log2 units.
+ * Replaces tiled_swa_fwd_kernel / tiled_swa_fwd_large_kernel (src/tiled_swa.py:15-133,
+ * :142-244) and the launch code of TiledSwa.forward (:605-637).  lse2 is fp32 [B, H, N]
+ * (the reference stores fp16 `m`, :608).  When `rope` is not NULL the rotation of
+ * dlt_rope2d is applied to q and k as they are loaded (q, k in HBM stay untouched);
+ * the result equals RotaryPE2D on q and k followed by the plain forward. */
+int dlt_swa_fwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                const void* v, const int64_t v_strides[4], void* o, const int64_t o_strides[4],
+                float* lse2, const int64_t lse_strides[3],
+                const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream);
+
+/* Backward: replaces tiled_swa_bwd_preprocess_kernel (src/tiled_swa.py:253-282) and
+ * tiled_swa_bwd_large_kernel_decoupled_q (:407-562) plus TiledSwa.backward (:649-689).
+ * `delta` is caller-provided fp32 scratch with the strides of lse2.  dq/dk/dv are written
+ * in the element type of q/k/v (the reference accumulates dq in an fp32 tensor, :656).
+ * With `rope` the inputs q, k are the UN-rotated tensors and dq, dk are returned with
+ * respect to them (transposed rotation applied on store). */
+int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],
+                const void* d_o, const int64_t do_strides[4],
+                const float* lse2, float* delta, const int64_t lse_strides[3],
+                void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                void* dv, const int64_t dv_strides[4],
+                const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream);
+
+/* Debug export: mask[i * T + j] = 1 iff query tile i attends kv tile j (T = t_height *
+ * t_width, row-major tiles), produced on the device by the SAME window routine the
+ * attention kernels call (src/tiled_swa.py:76-79, :97-100, :212-214, :701-713). */
+int dlt_swa_neighbors(int32_t t_height, int32_t t_width, int32_t row_size, int32_t col_size,
+                      uint8_t* mask, void* stream);
+
+/* ---- flash attention with separate qk / vo head dims -----------------------------------
+ * q [B,H,Lq,dk], k [B,H,Lk,dk], v [B,H,Lk,dv], o [B,H,Lq,dv], lse2 fp32 [B,H,Lq].
+ * Replaces _attn_fwd (src/flash_attn.py:81-172) and _attention.forward (:455-490); unlike
+ * the reference (single N_CTX, :479) Lq != Lk is accepted when causal == 0. */
+typedef struct {
+  int32_t B, H, Lq, Lk;
+  int32_t dk, dv;
+  float sm_scale;
+  int32_t causal;
+  int32_t dtype;
+} dlt_flash_shape_t;
+
+int dlt_flash_fwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                  const void* v, const int64_t v_strides[4], void* o, const int64_t o_strides[4],
+                  float* lse2, const int64_t lse_strides[3],
+                  const dlt_flash_shape_t* shape, void* stream);
+
+/* Replaces _attn_bwd_preprocess / _attn_bwd (src/flash_attn.py:186-449) and
+ * _attention.backward (:493-538); no host-side pre-scaling pass over k (:509-510) and no
+ * N_CTX % 128 requirement (:512). */
+int dlt_flash_bwd(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                  const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],
+                  const void* d_o, const int64_t do_strides[4],
+                  const float* lse2, float* delta, const int64_t lse_strides[3],
+                  void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                  void* dv, const int64_t dv_strides[4],
+                  const dlt_flash_shape_t* shape, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DLT_H */
