@@ -1,0 +1,311 @@
+// Device helpers shared by the attention kernels (forward, backward dK/dV, backward dQ).
+//
+// Register layouts (wave64, v_mfma_f32_16x16x32_{bf16,f16}); lane = 16 * g + n:
+//   A operand (16 x 32): lane holds row n,   k-slots 8g .. 8g+7
+//   B operand (32 x 16): lane holds col n,   k-slots 8g .. 8g+7
+//   C result  (16 x 16): lane holds col n,   rows 4g .. 4g+3
+// A product only needs A and B to agree on which k-slot means what, so the slot order is
+// chosen per use: contiguous head-dim chunks for q.k products, and for products that
+// contract over tokens the order in which the C layout of the previous product delivers
+// them (slot 8g + 4*mb + i  <->  token 16*mb + 4g + i of a 32-token block), which makes the
+// probability tile a B operand without any cross-lane traffic.  The matching A operand
+// (a [token][dim] LDS tile read with tokens along k) comes from ds_read_b64_tr_b16.
+#pragma once
+#include "dlt_internal.hpp"
+
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef short s16x4 __attribute__((__vector_size__(8)));
+
+#define DLT_LDS __attribute__((address_space(3)))
+#define DLT_DEV __device__ __forceinline__
+
+// compute type for an I/O element type: fp16 stays fp16, bf16 and fp32 run on bf16 MFMA
+template <typename TIO> struct ComputeOf { typedef bf16_t type; };
+template <> struct ComputeOf<f16_t> { typedef f16_t type; };
+
+template <typename CT> struct Mma;
+template <> struct Mma<bf16_t> {
+  static DLT_DEV f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<f16_t> {
+  static DLT_DEV f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+template <typename CT> DLT_DEV unsigned int pack2(float lo, float hi) {
+  CT a = (CT)lo, b = (CT)hi;
+  return (unsigned int)__builtin_bit_cast(unsigned short, a) | ((unsigned int)__builtin_bit_cast(unsigned short, b) << 16);
+}
+template <typename CT> DLT_DEV float unpack_lo(unsigned int w) {
+  return (float)__builtin_bit_cast(CT, (unsigned short)(w & 0xffffu));
+}
+template <typename CT> DLT_DEV float unpack_hi(unsigned int w) {
+  return (float)__builtin_bit_cast(CT, (unsigned short)(w >> 16));
+}
+
+DLT_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+DLT_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+DLT_DEV float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
+DLT_DEV u32x4 lds_read16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
+DLT_DEV void lds_write16(char* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+
+// transpose read: within a 16-lane group lane i receives element (i % 4) of the 8-byte chunk
+// addressed by lane 4j + i/4, for j = 0..3 (the four 16-bit results)
+DLT_DEV u32x2 lds_read_tr16(const char* p) {
+  s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((DLT_LDS s16x4*)(DLT_LDS void*)(p));
+  return __builtin_bit_cast(u32x2, v);
+}
+
+// A operand with tokens along k for the 32-token block starting at LDS row `row0` of a
+// [token][dim] tile: dims dim0 .. dim0+15 become the 16 rows of the operand.
+DLT_DEV u32x4 lds_read_tokens_as_k(const char* tile, int pitch, int row0, int dim0, int n, int g) {
+  const char* p = tile + (row0 + 4 * g + (n >> 2)) * pitch + (dim0 + 4 * (n & 3)) * 2;
+  const u32x2 lo = lds_read_tr16(p);
+  const u32x2 hi = lds_read_tr16(p + 16 * pitch);
+  u32x4 r;
+  r.x = lo.x; r.y = lo.y; r.z = hi.x; r.w = hi.y;
+  return r;
+}
+
+DLT_DEV float wave_max4(float v) {  // max over the 4 lanes that share n (lane ^ 16, lane ^ 32)
+  v = fmaxf(v, __shfl_xor(v, 16));
+  v = fmaxf(v, __shfl_xor(v, 32));
+  return v;
+}
+DLT_DEV float wave_sum4(float v) {
+  v += __shfl_xor(v, 16);
+  v += __shfl_xor(v, 32);
+  return v;
+}
+
+// ---- global <-> register moves of 8 consecutive head dims -------------------------------
+template <typename TIO, typename CT> struct Io;
+
+template <typename T> struct Io<T, T> {  // 2-byte element, same compute type
+  static DLT_DEV u32x4 load8(const T* p, bool vec, int64_t sd, int nvalid) {
+    if (vec) return *reinterpret_cast<const u32x4*>(p);
+    unsigned short e[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) e[j] = j < nvalid ? __builtin_bit_cast(unsigned short, p[j * sd]) : (unsigned short)0;
+    u32x4 r;
+    r.x = e[0] | ((unsigned)e[1] << 16); r.y = e[2] | ((unsigned)e[3] << 16);
+    r.z = e[4] | ((unsigned)e[5] << 16); r.w = e[6] | ((unsigned)e[7] << 16);
+    return r;
+  }
+  static DLT_DEV void store8(T* p, const float* v, bool vec, int64_t sd, int nvalid) {
+    if (vec) {
+      u32x4 r;
+      r.x = pack2<T>(v[0], v[1]); r.y = pack2<T>(v[2], v[3]); r.z = pack2<T>(v[4], v[5]); r.w = pack2<T>(v[6], v[7]);
+      *reinterpret_cast<u32x4*>(p) = r;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j++) if (j < nvalid) p[j * sd] = (T)v[j];
+    }
+  }
+};
+
+template <> struct Io<float, bf16_t> {  // fp32 in HBM, bf16 arithmetic
+  static DLT_DEV u32x4 load8(const float* p, bool vec, int64_t sd, int nvalid) {
+    float f[8];
+    if (vec) {
+      const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
+      f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j++) f[j] = j < nvalid ? p[j * sd] : 0.f;
+    }
+    u32x4 r;
+    r.x = pack2<bf16_t>(f[0], f[1]); r.y = pack2<bf16_t>(f[2], f[3]);
+    r.z = pack2<bf16_t>(f[4], f[5]); r.w = pack2<bf16_t>(f[6], f[7]);
+    return r;
+  }
+  static DLT_DEV void store8(float* p, const float* v, bool vec, int64_t sd, int nvalid) {
+    if (vec) {
+      reinterpret_cast<float4*>(p)[0] = make_float4(v[0], v[1], v[2], v[3]);
+      reinterpret_cast<float4*>(p)[1] = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j++) if (j < nvalid) p[j * sd] = v[j];
+    }
+  }
+};
+
+template <typename CT> DLT_DEV void unpack8(u32x4 r, float* f) {
+  f[0] = unpack_lo<CT>(r.x); f[1] = unpack_hi<CT>(r.x); f[2] = unpack_lo<CT>(r.y); f[3] = unpack_hi<CT>(r.y);
+  f[4] = unpack_lo<CT>(r.z); f[5] = unpack_hi<CT>(r.z); f[6] = unpack_lo<CT>(r.w); f[7] = unpack_hi<CT>(r.w);
+}
+template <typename CT> DLT_DEV u32x4 pack8(const float* f) {
+  u32x4 r;
+  r.x = pack2<CT>(f[0], f[1]); r.y = pack2<CT>(f[2], f[3]); r.z = pack2<CT>(f[4], f[5]); r.w = pack2<CT>(f[6], f[7]);
+  return r;
+}
+
+// ---- rotary encoding applied to one 8-dim chunk -----------------------------------------
+// y = self * cos -/+ partner * sin with each product rounded before the add: the evaluation
+// order of the standalone kernel and of the eager reference (src/fused_rope2d.py:221-222).
+DLT_DEV float rope_mix(float self, float partner, float c, float s, bool is_x0) {
+#pragma clang fp contract(off)
+  const float a = self * c, b = partner * s;
+  return is_x0 ? a - b : b + a;
+}
+
+// Per-thread rotary context for a fixed 8-dim chunk index `c` (dims 8c .. 8c+7).
+struct RopeChunk {
+  int mode;      // 0: chunk not rotated, 1: whole-chunk fast path (R % 8 == 0), 2: per-element path
+  int axis;      // fast path: 0 row, 1 column
+  int is_x0;     // fast path: chunk holds the first element of each pair
+  int partner_c; // fast path: chunk index holding the pair partners
+  int tab_off;   // fast path: float offset of this chunk's (cos, sin) pairs inside a table row
+};
+
+DLT_DEV RopeChunk rope_chunk_setup(const RopeDev& r, int c, bool vec) {
+  RopeChunk rc;
+  rc.mode = 0; rc.axis = 0; rc.is_x0 = 0; rc.partner_c = 0; rc.tab_off = 0;
+  if (!r.enabled || r.R == 0 || 8 * c >= 4 * r.R) return rc;
+  if (vec && (r.R & 7) == 0) {
+    const int r8 = r.R >> 3;
+    const int region = c / r8, ci = c - region * r8;
+    rc.mode = 1;
+    rc.axis = region >> 1;
+    rc.is_x0 = (region & 1) == 0;
+    rc.partner_c = rc.is_x0 ? c + r8 : c - r8;
+    rc.tab_off = 16 * ci;
+  } else {
+    rc.mode = 2;
+  }
+  return rc;
+}
+
+DLT_DEV const float* rope_table_row(const RopeDev& r, int axis, int32_t id, bool& rotated) {
+  int pos = axis == 0 ? dlt_rope_row(id) : dlt_rope_col(id);
+  rotated = pos >= 0;
+  pos = dlt_imax(0, dlt_imin(pos, (axis == 0 ? r.row_len : r.col_len) - 1));
+  return axis == 0 ? r.row_cs + (int64_t)pos * r.rs0 : r.col_cs + (int64_t)pos * r.cs0;
+}
+
+// Rotate the 8 values `self` (dims 8c..8c+7 of one token).  `partner(d)` returns the value
+// of dim d of the same token (only called for pair partners).
+template <typename PartnerFn>
+DLT_DEV void rope_apply8(const RopeDev& r, const RopeChunk& rc, int c, int32_t id, float* self, const float* partner8,
+                         PartnerFn partner) {
+  if (rc.mode == 1) {
+    bool rotated;
+    const float* tab = rope_table_row(r, rc.axis, id, rotated) + rc.tab_off;
+    if (!rotated) return;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const float cs = tab[2 * j], sn = r.inverse ? -tab[2 * j + 1] : tab[2 * j + 1];
+      self[j] = rope_mix(self[j], partner8[j], cs, sn, rc.is_x0);
+    }
+  } else if (rc.mode == 2) {
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      const int d = 8 * c + j;
+      if (d >= 4 * r.R) continue;
+      const int region = d / r.R, i = d - region * r.R;
+      bool rotated;
+      const float* tab = rope_table_row(r, region >> 1, id, rotated) + 2 * i;
+      if (!rotated) continue;
+      const bool is_x0 = (region & 1) == 0;
+      const float pv = partner(is_x0 ? d + r.R : d - r.R);
+      const float sn = r.inverse ? -tab[1] : tab[1];
+      self[j] = rope_mix(self[j], pv, tab[0], sn, is_x0);
+    }
+  }
+}
+
+// ---- HBM -> LDS staging of `nrows` token rows of D head dims -------------------------------
+// LDS tile: row-major, `pitch` bytes per row, compute-type elements.  tok(row) gives the token
+// index inside the [N, D] slab at `base` (or -1: the row is zero-filled).  Dims >= dact are
+// zero-filled.  With `rope.enabled` rows are rotated on the way in (q and k of the fused call).
+template <typename TIO, typename CT, int D, typename TokFn>
+DLT_DEV void stage_tile(char* s, int pitch, const TIO* base, int64_t sn, int64_t sd, int dact, bool vec, int nrows,
+                        TokFn tok, const RopeDev& rope, int tid) {
+  constexpr int CH = D / 8;
+  constexpr int RSTEP = 256 / CH;
+  const int c = tid % CH;
+  const RopeChunk rc = rope_chunk_setup(rope, c, vec);
+  const int nvalid = dlt_imin(8, dact - 8 * c);
+  for (int row = tid / CH; row < nrows; row += RSTEP) {
+    const int64_t t = tok(row);
+    u32x4 val = {0u, 0u, 0u, 0u};
+    if (t >= 0 && nvalid > 0) {
+      const TIO* p = base + t * sn;
+      val = Io<TIO, CT>::load8(p + (int64_t)8 * c * sd, vec, sd, nvalid);
+      if (rc.mode != 0) {
+        float self[8], partner8[8];
+        unpack8<CT>(val, self);
+        if (rc.mode == 1) {
+          const u32x4 pr = Io<TIO, CT>::load8(p + (int64_t)8 * rc.partner_c * sd, vec, sd, 8);
+          unpack8<CT>(pr, partner8);
+        }
+        // operands are rounded to the compute type first, as the standalone op sees them
+        rope_apply8(rope, rc, c, rope.idx[t], self, partner8,
+                    [&](int d) { return (float)(CT)(float)p[(int64_t)d * sd]; });
+        val = pack8<CT>(self);
+      }
+    }
+    lds_write16(s + row * pitch + c * 16, val);
+  }
+}
+
+// ---- LDS -> HBM store of an output tile ------------------------------------------------------
+// TL: element type of the LDS tile (the output type, or float for fp32 outputs).
+template <typename TO, typename TL, int D, typename TokFn>
+DLT_DEV void store_tile(const char* s, int pitch, TO* base, int64_t sn, int64_t sd, int dact, bool vec, int nrows,
+                        TokFn tok, const RopeDev& rope, int tid) {
+  constexpr int CH = D / 8;
+  constexpr int RSTEP = 256 / CH;
+  typedef typename ComputeOf<TO>::type CT;
+  const int c = tid % CH;
+  const RopeChunk rc = rope_chunk_setup(rope, c, true);
+  const int nvalid = dlt_imin(8, dact - 8 * c);
+  if (nvalid <= 0) return;
+  for (int row = tid / CH; row < nrows; row += RSTEP) {
+    const int64_t t = tok(row);
+    if (t < 0) continue;
+    const TL* lrow = reinterpret_cast<const TL*>(s + row * pitch);
+    float v[8], partner8[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) v[j] = (float)lrow[8 * c + j];
+    if (rc.mode != 0) {
+      if (rc.mode == 1) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) partner8[j] = (float)lrow[8 * rc.partner_c + j];
+      }
+      rope_apply8(rope, rc, c, rope.idx[t], v, partner8, [&](int d) { return (float)lrow[d]; });
+    }
+    Io<TO, CT>::store8(base + t * sn + (int64_t)8 * c * sd, v, vec, sd, nvalid);
+  }
+}
+
+// LDS tile element type used for an output element type
+template <typename TO> struct TileOf { typedef TO type; };
+
+// workgroup id -> logical id such that each XCD (8 of them, workgroups are dealt round-robin)
+// walks a contiguous range of logical ids: neighbouring tiles of one head share an L2.
+DLT_DEV int xcd_remap(int bid, int nblocks) {
+  const int per = nblocks >> 3;
+  if (per == 0 || bid >= per * 8) return bid;
+  return (bid & 7) * per + (bid >> 3);
+}
+
+// Per-launch plan computed on the host (attn_plan.cpp logic lives in attn_launch.hip).
+struct AttnPlan {
+  int32_t rowfit;      // 1: a chunk holds whole halo rows, each wave walks from its own x origin
+  int32_t chunk_rows;  // halo rows per chunk (rowfit) else 1
+  int32_t chunk_x;     // tokens staged per halo row (LDS row pitch in tokens)
+  int32_t nblk_x;      // workgroups per grid row on the own side
+  int32_t off_a, off_b, off_c, off_d;  // LDS byte offsets of the halo buffers
+  int32_t lds_bytes;
+};

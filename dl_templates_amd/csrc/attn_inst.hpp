@@ -1,0 +1,36 @@
+// Included by attn_inst_<DK>_<DV>.hip with DLT_DK / DLT_DV defined: instantiates the kernels
+// for one pair of (padded) head dims and exports their launchers.
+#include "attn_fwd_kernel.hpp"
+
+#define DLT_CAT3_(a, b, c) a##b##_##c
+#define DLT_CAT3(a, b, c) DLT_CAT3_(a, b, c)
+
+namespace {
+template <typename KernT>
+int set_lds_limit(KernT kern, int bytes) {
+  // dynamic LDS above the default limit must be opted into once per kernel
+  if (bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
+  }
+  return DLT_OK;
+}
+
+template <typename TIO, int NP>
+int launch_fwd_t(const FwdArgs& a, int grid, hipStream_t stream) {
+  auto kern = attn_fwd_kernel<TIO, DLT_DK, DLT_DV, NP>;
+  int rc = set_lds_limit(kern, a.plan.lds_bytes);
+  if (rc != DLT_OK) return rc;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), a.plan.lds_bytes, stream, a);
+  DLT_CHECK_LAUNCH("attention forward launch");
+  return DLT_OK;
+}
+}  // namespace
+
+int DLT_CAT3(dlt_launch_fwd_, DLT_DK, DLT_DV)(const FwdArgs& a, int np, int grid, hipStream_t stream) {
+  switch (a.p.dtype) {
+    case DLT_BF16: return np == 1 ? launch_fwd_t<bf16_t, 1>(a, grid, stream) : launch_fwd_t<bf16_t, 2>(a, grid, stream);
+    case DLT_FP16: return np == 1 ? launch_fwd_t<f16_t, 1>(a, grid, stream) : launch_fwd_t<f16_t, 2>(a, grid, stream);
+    default: return np == 1 ? launch_fwd_t<float, 1>(a, grid, stream) : launch_fwd_t<float, 2>(a, grid, stream);
+  }
+}

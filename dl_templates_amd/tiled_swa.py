@@ -1,0 +1,123 @@
+"""Tiled 2D sliding-window flash attention (drop-in for src/tiled_swa.py).
+
+``TiledSwa`` keeps the reference's autograd contract (src/tiled_swa.py:602-689): positional
+arguments ``(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)`` and a
+backward that returns ``(dq, dk, dv, None * 6)``.  ``tiled_swa_fwd`` (:564-600) is the no-grad
+forward.  Deliberate differences from the reference, all documented in the C header:
+outputs have the dtype and device of ``q`` (the reference hard-codes fp16 and the default
+device, :608-609), the saved log-sum-exp is fp32, and tiles smaller than 16 tokens have a
+backward (the reference raises, :660-661).
+
+``TiledSwaRope`` is the fused RoPE-2D + attention op: it equals ``RotaryPE2D`` applied to
+q and k followed by ``TiledSwa`` (the composition of README.md:11) without writing the
+rotated q / k to HBM; its backward returns gradients for the un-rotated q and k.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+
+def _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale) -> _lib.SwaShape:
+    B, H, N, KEY_DIM = q.shape
+    HEAD_DIM = v.shape[-1]
+    assert N == t_height * t_width * b_size, "seqlen should match image size"
+    assert k.shape == (B, H, N, KEY_DIM) and v.shape[:3] == (B, H, N)
+    assert q.dtype == k.dtype == v.dtype
+    return _lib.SwaShape(B, H, b_size, t_height, t_width, row_size, col_size, KEY_DIM, HEAD_DIM, float(sm_scale),
+                         _lib.dtype_code(q))
+
+
+def _forward(q, k, v, shape, rope):
+    _lib.require_cuda(q, k, v)
+    lib = _lib.load()
+    B, H, N, _ = q.shape
+    o = torch.empty((B, H, N, v.shape[-1]), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+    desc, keep = (None, None) if rope is None else _lib.rope_desc(*rope)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.dlt_swa_fwd(_lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v),
+                                   _lib.strides(v), _lib.ptr(o), _lib.strides(o), _lib.ptr(lse), _lib.strides(lse),
+                                   shape, desc, _lib.stream_of(q)))
+    del keep
+    return o, lse
+
+
+def _backward(q, k, v, o, lse, do, shape, rope):
+    lib = _lib.load()
+    _lib.require_cuda(q, k, v, o, lse, do)
+    dq = torch.empty_like(q)
+    dk = torch.empty_like(k)
+    dv = torch.empty_like(v)
+    delta = torch.empty_like(lse)
+    desc, keep = (None, None) if rope is None else _lib.rope_desc(*rope)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.dlt_swa_bwd(_lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v),
+                                   _lib.strides(v), _lib.ptr(o), _lib.strides(o), _lib.ptr(do), _lib.strides(do),
+                                   _lib.ptr(lse), _lib.ptr(delta), _lib.strides(lse),
+                                   _lib.ptr(dq), _lib.strides(dq), _lib.ptr(dk), _lib.strides(dk),
+                                   _lib.ptr(dv), _lib.strides(dv), shape, desc, _lib.stream_of(q)))
+    del keep
+    return dq, dk, dv
+
+
+def tiled_swa_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_size: int, t_height: int, t_width: int,
+                  row_size: int, col_size: int, sm_scale: float = 1.0):
+    shape = _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)
+    return _forward(q, k, v, shape, None)[0]
+
+
+class TiledSwa(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_size: int, t_height: int, t_width: int,
+                row_size: int, col_size: int, sm_scale: float):
+        shape = _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)
+        o, m = _forward(q, k, v, shape, None)
+        ctx.save_for_backward(q, k, v, m, o)
+        ctx.b_size = b_size
+        ctx.t_height = t_height
+        ctx.t_width = t_width
+        ctx.row_size = row_size
+        ctx.col_size = col_size
+        ctx.sm_scale = sm_scale
+        return o
+
+    @staticmethod
+    def backward(ctx, do: torch.Tensor):
+        q, k, v, m, o = ctx.saved_tensors
+        shape = _shape(q, k, v, ctx.b_size, ctx.t_height, ctx.t_width, ctx.row_size, ctx.col_size, ctx.sm_scale)
+        dq, dk, dv = _backward(q, k, v, o, m, do, shape, None)
+        return dq, dk, dv, None, None, None, None, None, None,
+
+
+class TiledSwaRope(torch.autograd.Function):
+    """o = TiledSwa(rope(q), rope(k), v) with the rotation fused into the q / k tile loads."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, idx, row_cs_buffer, col_cs_buffer, b_size, t_height, t_width, row_size, col_size,
+                sm_scale):
+        shape = _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)
+        assert row_cs_buffer.shape[1] == col_cs_buffer.shape[1]
+        assert idx.shape[0] == q.shape[2]
+        o, m = _forward(q, k, v, shape, (idx, row_cs_buffer, col_cs_buffer))
+        ctx.save_for_backward(q, k, v, m, o, idx, row_cs_buffer, col_cs_buffer)
+        ctx.scalars = (b_size, t_height, t_width, row_size, col_size, sm_scale)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, m, o, idx, row_cs_buffer, col_cs_buffer = ctx.saved_tensors
+        shape = _shape(q, k, v, *ctx.scalars)
+        dq, dk, dv = _backward(q, k, v, o, m, do, shape, (idx, row_cs_buffer, col_cs_buffer))
+        return (dq, dk, dv) + (None,) * 9
+
+
+def swa_neighbors(t_height: int, t_width: int, row_size: int, col_size: int, device="cuda") -> torch.Tensor:
+    """bool [T, T] neighbour mask computed on the device by the kernels' own window routine."""
+    T = t_height * t_width
+    out = torch.empty((T, T), dtype=torch.uint8, device=device)
+    with torch.cuda.device(out.device):
+        _lib.check(_lib.load().dlt_swa_neighbors(t_height, t_width, row_size, col_size, _lib.ptr(out),
+                                                 _lib.stream_of(out)))
+    return out.bool()

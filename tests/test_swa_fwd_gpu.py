@@ -1,0 +1,127 @@
+"""GPU parity of the SWA forward (dlt_swa_fwd) against the CPU oracle.
+
+Bar (fp32 oracle on the same seeded inputs): neighbour sets bit-exact; forward max-abs
+error <= 2e-2 (bf16/fp16/fp32 I/O, bf16 or fp16 MFMA with fp32 accumulation).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+FWD_TOL = 2e-2
+
+
+def _swa():
+    from dl_templates_amd import tiled_swa
+    return tiled_swa
+
+
+@pytest.mark.parametrize("th,tw,wr,wc", [(16, 16, 3, 3), (5, 7, 2, 1), (1, 9, 0, 4), (12, 3, 20, 0), (4, 4, 4, 4)])
+def test_neighbor_sets_bit_exact(th, tw, wr, wc):
+    got = _swa().swa_neighbors(th, tw, wr, wc).cpu().numpy()
+    assert np.array_equal(got, orc.neighbor_mask(th, tw, wr, wc))
+
+
+def _run(seed, B, H, b_size, th, tw, wr, wc, dk, dv, dtype, scale=None, check_lse=True):
+    N = b_size * th * tw
+    q, k, v, _ = orc.make_qkv(seed, B, H, N, N, dk, dv, dtype)
+    scale = 1.0 / math.sqrt(dk) if scale is None else scale
+    want, lse_w = orc.tiled_swa_explicit(q.float(), k.float(), v.float(), b_size, th, tw, wr, wc, scale, return_lse2=True)
+    got = _swa().tiled_swa_fwd(q.cuda(), k.cuda(), v.cuda(), b_size, th, tw, wr, wc, scale)
+    assert got.dtype == dtype and got.shape == want.shape
+    err = (got.float().cpu() - want).abs().max().item()
+    assert err <= FWD_TOL, f"max abs err {err}"
+    return err
+
+
+def test_c1_tiny_fp32_and_golden():
+    # BASELINE config 1 + the committed fixture
+    import os
+    f = np.load(os.path.join(os.path.dirname(__file__), "golden", "c1_swa_fwd.npz"))
+    q, k, v, _ = orc.make_qkv(int(f["seed"]), 1, 2, 256, 256, 32, 32)
+    got = _swa().tiled_swa_fwd(q.cuda(), k.cuda(), v.cuda(), 1, 16, 16, 3, 3, 1 / math.sqrt(32)).cpu()
+    assert (got - torch.from_numpy(f["o"])).abs().max().item() <= FWD_TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_small_grid_dtypes(dtype):
+    _run(1, 2, 2, 1, 16, 16, 3, 3, 32, 32, dtype)
+
+
+@pytest.mark.parametrize("th,tw,wr,wc", [(7, 9, 2, 3), (3, 70, 1, 6), (20, 5, 6, 1), (1, 1, 0, 0), (9, 130, 3, 10), (6, 6, 8, 8)])
+def test_ragged_and_boundary_grids(th, tw, wr, wc):
+    _run(2, 1, 3, 1, th, tw, wr, wc, 64, 64, torch.bfloat16)
+
+
+@pytest.mark.parametrize("b_size,th,tw,wr,wc", [(16, 8, 8, 1, 1), (4, 6, 5, 1, 2), (3, 5, 4, 2, 1), (32, 3, 4, 1, 1), (2, 9, 9, 6, 6), (100, 2, 3, 1, 1)])
+def test_tiles_with_several_tokens(b_size, th, tw, wr, wc):
+    _run(3, 1, 2, b_size, th, tw, wr, wc, 32, 32, torch.bfloat16, scale=0.25)
+
+
+@pytest.mark.parametrize("dk,dv", [(64, 64), (128, 128), (64, 128), (16, 32), (40, 24), (128, 64)])
+def test_head_dims(dk, dv):
+    _run(4, 1, 2, 1, 12, 12, 3, 3, dk, dv, torch.bfloat16)
+
+
+def test_c3_shape_fwd():
+    # BASELINE config 3 shape (unfused): B=2, H=8, 64x64, d=64, 13x13
+    err = _run(5, 2, 8, 1, 64, 64, 6, 6, 64, 64, torch.bfloat16)
+    print("c3 fwd max abs err", err)
+
+
+def test_strided_inputs():
+    sw = _swa()
+    B, H, th, tw, d = 2, 3, 8, 8, 64
+    N = th * tw
+    q, k, v, _ = orc.make_qkv(6, B, H, N, N, d, d, torch.bfloat16)
+    want = orc.tiled_swa_explicit(q.float(), k.float(), v.float(), 1, th, tw, 2, 2, 0.125)
+    # [B, N, H, D] storage viewed as [B, H, N, D]; and a last-dim-strided q
+    qg = q.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)
+    kg = k.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)
+    vg = torch.stack([v, v], -1).cuda()[..., 0]
+    got = sw.tiled_swa_fwd(qg, kg, vg, 1, th, tw, 2, 2, 0.125)
+    assert (got.float().cpu() - want).abs().max().item() <= FWD_TOL
+
+
+def test_constant_v_and_determinism():
+    sw = _swa()
+    q, k, v, _ = orc.make_qkv(7, 1, 2, 400, 400, 64, 64, torch.bfloat16)
+    v = torch.ones_like(v) * 0.5
+    a = sw.tiled_swa_fwd(q.cuda(), k.cuda(), v.cuda(), 1, 20, 20, 4, 4, 0.125)
+    b = sw.tiled_swa_fwd(q.cuda(), k.cuda(), v.cuda(), 1, 20, 20, 4, 4, 0.125)
+    assert torch.equal(a, b)
+    assert (a.float() - 0.5).abs().max().item() <= 4e-3
+
+
+def test_fused_rope_forward_equals_composition():
+    from dl_templates_amd import fused_rope2d as fr
+    sw = _swa()
+    B, H, th, tw, d = 2, 2, 16, 16, 64
+    N = th * tw
+    q, k, v, _ = orc.make_qkv(8, B, H, N, N, d, d, torch.bfloat16)
+    idx = orc.make_rope_idx(9, th, tw, 0.05)
+    rcs, ccs = orc.rope_tables(8, th), orc.rope_tables(8, tw)
+    want = orc.rope_swa_ref(q.float(), k.float(), v.float(), idx, rcs, ccs, 1, th, tw, 3, 3, 0.125)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    got = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, 3, 3, 0.125)
+    assert torch.equal(qg.cpu(), q) and torch.equal(kg.cpu(), k), "fused op must not modify q / k"
+    assert (got.float().cpu() - want).abs().max().item() <= FWD_TOL
+    # bit-identical to running the standalone rotation first
+    q2, k2 = fr.rope2d_qk_(q.cuda().clone(), k.cuda().clone(), idx.cuda(), rcs.cuda(), ccs.cuda())
+    comp = sw.tiled_swa_fwd(q2, k2, vg, 1, th, tw, 3, 3, 0.125)
+    assert torch.equal(comp, got)
+
+
+def test_bad_arguments_raise():
+    sw = _swa()
+    q = torch.randn(1, 1, 16, 64, dtype=torch.bfloat16).cuda()
+    with pytest.raises(AssertionError):
+        sw.tiled_swa_fwd(q, q, q, 1, 4, 5, 1, 1, 1.0)
+    big = torch.randn(1, 1, 16, 256, dtype=torch.bfloat16).cuda()
+    from dl_templates_amd._lib import DltError
+    with pytest.raises(DltError):
+        sw.tiled_swa_fwd(big, big, big, 1, 4, 4, 1, 1, 1.0)
