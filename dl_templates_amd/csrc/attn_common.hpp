@@ -300,7 +300,7 @@ DLT_DEV int xcd_remap(int bid, int nblocks) {
   return (bid & 7) * per + (bid >> 3);
 }
 
-// Per-launch plan computed on the host (attn_plan.cpp logic lives in attn_launch.hip).
+// Per-launch plan computed on the host (attn_launch.hip).
 struct AttnPlan {
   int32_t rowfit;      // 1: a chunk holds whole halo rows, each wave walks from its own x origin
   int32_t chunk_rows;  // halo rows per chunk (rowfit) else 1
@@ -308,4 +308,74 @@ struct AttnPlan {
   int32_t nblk_x;      // workgroups per grid row on the own side
   int32_t off_a, off_b, off_c, off_d;  // LDS byte offsets of the halo buffers
   int32_t lds_bytes;
+};
+
+// Which tokens a workgroup / wave / lane owns and which tokens of the other side they touch.
+// "Own" tokens are queries for the forward and dQ kernels and keys for the dK/dV kernel
+// (TRANSPOSE); the "halo" is the set of tokens of the other side inside the window of any
+// own token: grid rows [rlo, rhi] (the same for the whole workgroup, which owns tokens of a
+// single grid row) and x in [X0, X1).  Per lane the window of own token n is the x interval
+// [xlo, xlo + span); per 16-token patch and per wave the union / intersection of those
+// intervals are wave-uniform and steer which 32-token blocks are visited and whether a
+// block needs the element mask at all.
+template <int NP, bool TRANSPOSE>
+struct TileCtx {
+  int b, h, r_own, x0, xlast;
+  int rlo, rhi, X0, X1;
+  int wfirst, wxlo, wxhi;
+  int xlo[NP], span[NP];
+  int pxlo[NP], pxhi[NP], pin_lo[NP], pin_hi[NP];
+  int64_t own_tok0;
+  int XL_own, XL_halo;
+
+  static DLT_DEV void range(const DltGeom& G, int r, int x, int& rl, int& rh, int& xl, int& xh) {
+    if (TRANSPOSE) dlt_query_range(G, r, x, rl, rh, xl, xh);
+    else dlt_key_range(G, r, x, rl, rh, xl, xh);
+  }
+
+  DLT_DEV void init(const DltGeom& G, const AttnPlan& plan, int H, int wave, int n) {
+    constexpr int OWN = 64 * NP;
+    XL_own = TRANSPOSE ? G.XLk : G.XLq;
+    XL_halo = TRANSPOSE ? G.XLq : G.XLk;
+    const int lin = xcd_remap(blockIdx.x, gridDim.x);
+    const int per_bh = G.TR * plan.nblk_x;
+    const int bh = lin / per_bh;
+    const int rem = lin - bh * per_bh;
+    r_own = rem / plan.nblk_x;
+    x0 = (rem - r_own * plan.nblk_x) * OWN;
+    b = bh / H;
+    h = bh - b * H;
+    xlast = dlt_imin(x0 + OWN, XL_own) - 1;
+    own_tok0 = (int64_t)r_own * XL_own + x0;
+    int t0, t1;
+    range(G, r_own, x0, rlo, rhi, X0, t0);
+    range(G, r_own, xlast, t0, t1, t0, X1);
+    wfirst = x0 + wave * 16 * NP;
+    wxlo = wxhi = 0;
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      const int xq = wfirst + 16 * p + n;
+      int a0, a1, lo = 0, hi = 0;
+      if (xq <= xlast) range(G, r_own, xq, a0, a1, lo, hi);
+      xlo[p] = lo; span[p] = hi - lo;
+      const int pf = wfirst + 16 * p, pl = dlt_imin(pf + 15, xlast);
+      pxlo[p] = pxhi[p] = 0; pin_lo[p] = 0x7fffffff; pin_hi[p] = 0;
+      if (pf <= xlast) {
+        int l0, h0, l1, h1;
+        range(G, r_own, pf, a0, a1, l0, h0);
+        range(G, r_own, pl, a0, a1, l1, h1);
+        pxlo[p] = l0; pxhi[p] = h1;
+        if (pl == pf + 15) { pin_lo[p] = l1; pin_hi[p] = h0; }
+        if (p == 0) wxlo = l0;
+        wxhi = h1;
+      }
+    }
+  }
+  DLT_DEV int64_t own_token(int row) const { return x0 + row <= xlast ? own_tok0 + row : (int64_t)-1; }
+  DLT_DEV bool patch_skips(int p, int kx0) const { return kx0 >= pxhi[p] || kx0 + 32 <= pxlo[p]; }
+  DLT_DEV bool patch_needs_mask(int p, int kx0) const { return !(kx0 >= pin_lo[p] && kx0 + 32 <= pin_hi[p]); }
+  // element (mb, i) of a 32-token block at kx0, held by lane group g: token x = kx0 + 16 mb + 4 g + i
+  DLT_DEV bool valid(int p, int kx0, int g, int mb, int i) const {
+    return (unsigned)(kx0 + 16 * mb + 4 * g + i - xlo[p]) < (unsigned)span[p];
+  }
 };

@@ -39,19 +39,10 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const DltGeom& G = a.p.g;
 
-  // ---- which tile is ours
-  const int lin = xcd_remap(blockIdx.x, gridDim.x);
-  const int per_bh = G.TR * a.plan.nblk_x;
-  const int bh = lin / per_bh;
-  const int rem = lin - bh * per_bh;
-  const int r_own = rem / a.plan.nblk_x;
-  const int x0 = (rem - r_own * a.plan.nblk_x) * OWN;
-  const int b = bh / a.p.H, h = bh - b * a.p.H;
-  const int xlast = dlt_imin(x0 + OWN, G.XLq) - 1;
-
-  int rlo, rhi, X0, X1, t0, t1;
-  dlt_key_range(G, r_own, x0, rlo, rhi, X0, t0);
-  dlt_key_range(G, r_own, xlast, t0, t1, t0, X1);
+  TileCtx<NP, false> T;
+  T.init(G, a.plan, a.p.H, wave, n);
+  const int b = T.b, h = T.h, r_own = T.r_own, xlast = T.xlast;
+  const int rlo = T.rlo, rhi = T.rhi, X0 = T.X0, X1 = T.X1, wxlo = T.wxlo, wxhi = T.wxhi, wfirst = T.wfirst;
 
   char* sQ = smem;
   char* sK = smem + a.plan.off_a;
@@ -65,39 +56,14 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   no_rope.enabled = 0;
 
   // ---- own queries -> LDS -> B-operand fragments
-  const int64_t own_tok0 = (int64_t)r_own * G.XLq + x0;
   stage_tile<TIO, CT, DK>(sQ, PQ, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, OWN,
-                          [&](int row) { return x0 + row <= xlast ? own_tok0 + row : (int64_t)-1; }, a.p.rope, tid);
+                          [&](int row) { return T.own_token(row); }, a.p.rope, tid);
   __syncthreads();
   u32x4 qf[NP][KC];
 #pragma unroll
   for (int p = 0; p < NP; p++)
 #pragma unroll
     for (int c = 0; c < KC; c++) qf[p][c] = lds_read16(sQ + (wave * 16 * NP + 16 * p + n) * PQ + (32 * c + 8 * g) * 2);
-
-  // ---- per-lane key intervals, per-patch and per-wave bounds (wave-uniform)
-  int xlo[NP], span[NP];
-  int pxlo[NP], pxhi[NP], pin_lo[NP], pin_hi[NP];
-  const int wfirst = x0 + wave * 16 * NP;
-  int wxlo = 0, wxhi = 0;
-#pragma unroll
-  for (int p = 0; p < NP; p++) {
-    const int xq = wfirst + 16 * p + n;
-    int a0, a1, lo = 0, hi = 0;
-    if (xq <= xlast) dlt_key_range(G, r_own, xq, a0, a1, lo, hi);
-    xlo[p] = lo; span[p] = hi - lo;
-    const int pf = wfirst + 16 * p, pl = dlt_imin(pf + 15, xlast);
-    pxlo[p] = pxhi[p] = 0; pin_lo[p] = 0x7fffffff; pin_hi[p] = 0;
-    if (pf <= xlast) {
-      int l0, h0, l1, h1;
-      dlt_key_range(G, r_own, pf, a0, a1, l0, h0);
-      dlt_key_range(G, r_own, pl, a0, a1, l1, h1);
-      pxlo[p] = l0; pxhi[p] = h1;
-      if (pl == pf + 15) { pin_lo[p] = l1; pin_hi[p] = h0; }
-      if (p == 0) wxlo = l0;
-      wxhi = h1;
-    }
-  }
 
   float m_run[NP], l_run[NP];
   f32x4 acc[NP][VB];
@@ -145,7 +111,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
 
 #pragma unroll
           for (int p = 0; p < NP; p++) {
-            if (kx0 >= pxhi[p] || kx0 + 32 <= pxlo[p]) continue;
+            if (T.patch_skips(p, kx0)) continue;
             f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < KC; c++) {
@@ -153,13 +119,11 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
               s1 = Mma<CT>::mfma(ka[1][c], qf[p][c], s1);
             }
             float t[8];
-            const bool need_mask = !(kx0 >= pin_lo[p] && kx0 + 32 <= pin_hi[p]);
-            if (need_mask) {
-              const int base = kx0 + 4 * g - xlo[p];
+            if (T.patch_needs_mask(p, kx0)) {
 #pragma unroll
               for (int i = 0; i < 4; i++) {
-                t[i] = (unsigned)(base + i) < (unsigned)span[p] ? s0[i] * scale : -INFINITY;
-                t[4 + i] = (unsigned)(base + 16 + i) < (unsigned)span[p] ? s1[i] * scale : -INFINITY;
+                t[i] = T.valid(p, kx0, g, 0, i) ? s0[i] * scale : -INFINITY;
+                t[4 + i] = T.valid(p, kx0, g, 1, i) ? s1[i] * scale : -INFINITY;
               }
             } else {
 #pragma unroll
@@ -207,5 +171,5 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   }
   __syncthreads();
   store_tile<TIO, TL, DV>(sO, PO, ob, a.os[2], a.os[3], a.p.dv, a.o_vec != 0, OWN,
-                          [&](int row) { return x0 + row <= xlast ? own_tok0 + row : (int64_t)-1; }, no_rope, tid);
+                          [&](int row) { return T.own_token(row); }, no_rope, tid);
 }

@@ -1,6 +1,7 @@
 // Included by attn_inst_<DK>_<DV>.hip with DLT_DK / DLT_DV defined: instantiates the kernels
 // for one pair of (padded) head dims and exports their launchers.
 #include "attn_fwd_kernel.hpp"
+#include "attn_bwd_kernel.hpp"
 
 #define DLT_CAT3_(a, b, c) a##b##_##c
 #define DLT_CAT3(a, b, c) DLT_CAT3_(a, b, c)
@@ -25,7 +26,41 @@ int launch_fwd_t(const FwdArgs& a, int grid, hipStream_t stream) {
   DLT_CHECK_LAUNCH("attention forward launch");
   return DLT_OK;
 }
+
+template <typename TIO, int NP>
+int launch_bwd_t(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q, hipStream_t stream) {
+  {
+    constexpr int CH = DLT_DV / 8;
+    const int64_t threads = (int64_t)aq.p.B * aq.p.H * aq.n_tokens_q * CH;
+    hipLaunchKernelGGL((attn_delta_kernel<TIO, DLT_DV>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, aq);
+    DLT_CHECK_LAUNCH("attention delta launch");
+  }
+  {
+    auto kern = attn_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP>;
+    int rc = set_lds_limit(kern, akv.plan.lds_bytes);
+    if (rc != DLT_OK) return rc;
+    hipLaunchKernelGGL(kern, dim3(grid_kv), dim3(256), akv.plan.lds_bytes, stream, akv);
+    DLT_CHECK_LAUNCH("attention dK/dV launch");
+  }
+  {
+    auto kern = attn_bwd_q_kernel<TIO, DLT_DK, DLT_DV, NP>;
+    int rc = set_lds_limit(kern, aq.plan.lds_bytes);
+    if (rc != DLT_OK) return rc;
+    hipLaunchKernelGGL(kern, dim3(grid_q), dim3(256), aq.plan.lds_bytes, stream, aq);
+    DLT_CHECK_LAUNCH("attention dQ launch");
+  }
+  return DLT_OK;
+}
 }  // namespace
+
+int DLT_CAT3(dlt_launch_bwd_, DLT_DK, DLT_DV)(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q, int np,
+                                              hipStream_t stream) {
+  switch (aq.p.dtype) {
+    case DLT_BF16: return np == 1 ? launch_bwd_t<bf16_t, 1>(akv, grid_kv, aq, grid_q, stream) : launch_bwd_t<bf16_t, 2>(akv, grid_kv, aq, grid_q, stream);
+    case DLT_FP16: return np == 1 ? launch_bwd_t<f16_t, 1>(akv, grid_kv, aq, grid_q, stream) : launch_bwd_t<f16_t, 2>(akv, grid_kv, aq, grid_q, stream);
+    default: return np == 1 ? launch_bwd_t<float, 1>(akv, grid_kv, aq, grid_q, stream) : launch_bwd_t<float, 2>(akv, grid_kv, aq, grid_q, stream);
+  }
+}
 
 int DLT_CAT3(dlt_launch_fwd_, DLT_DK, DLT_DV)(const FwdArgs& a, int np, int grid, hipStream_t stream) {
   switch (a.p.dtype) {

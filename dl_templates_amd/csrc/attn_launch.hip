@@ -1,10 +1,15 @@
 // Host side of the attention core: validation that depends on the kernels' limits, the
 // per-launch LDS / chunking plan, and dispatch to the instantiation for the padded head dims.
 #include "attn_fwd_kernel.hpp"
+#include "attn_bwd_kernel.hpp"
 
 int dlt_launch_fwd_64_64(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_128_128(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_64_128(const FwdArgs&, int, int, hipStream_t);
+
+int dlt_launch_bwd_64_64(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
+int dlt_launch_bwd_128_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
+int dlt_launch_bwd_64_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 
 namespace {
 
@@ -96,6 +101,62 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
   }
 }
 
-int dlt_attn_backward(const AttnProblem&, const AttnTensors&, hipStream_t) {
-  return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward not built");
+int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
+  DimClass dc;
+  int rc = pick_dims(p, dc);
+  if (rc != DLT_OK) return rc;
+  const int es = dlt_elem_size(p.dtype);
+  const int np = 1;
+  const int own = 64 * np;
+  const int PQ = dc.DK * 2 + 16, PV = dc.DV * 2 + 16;
+  const int tile_k = dc.DK * es + 16, tile_v = dc.DV * es + 16;
+  int own_bytes = own * (PQ + PV);
+  if (own * tile_k > own_bytes) own_bytes = own * tile_k;
+  if (own * tile_v > own_bytes) own_bytes = own * tile_v;
+
+  BwdArgs a;
+  a.p = p;
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.o; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
+  for (int i = 0; i < 4; i++) {
+    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; a.dos[i] = t.dos[i];
+    a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
+  }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.q_vec = vec_ok(t.q, t.qs, 4, p.dk, es);
+  a.k_vec = vec_ok(t.k, t.ks, 4, p.dk, es);
+  a.v_vec = vec_ok(t.v, t.vs, 4, p.dv, es);
+  a.o_vec = vec_ok(t.o, t.os, 4, p.dv, es);
+  a.do_vec = vec_ok(t.d_o, t.dos, 4, p.dv, es);
+  a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, es);
+  a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, es);
+  a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, es);
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  a.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
+
+  // dK/dV: keys are the own side, queries (Q, dO, lse2, delta) are streamed
+  BwdArgs akv = a;
+  rc = make_plan(p, own, own_bytes, PQ + PV + 8, p.g.XLk, p.g.XLq, akv.plan);
+  if (rc != DLT_OK) return rc;
+  {
+    const int toks = akv.plan.chunk_rows * akv.plan.chunk_x;
+    akv.plan.off_b = akv.plan.off_a + toks * PQ;
+    akv.plan.off_c = akv.plan.off_b + toks * PV;
+    akv.plan.off_d = akv.plan.off_c + toks * 4;
+  }
+  // dQ: queries are the own side, K and V are streamed
+  BwdArgs aq = a;
+  rc = make_plan(p, own, own_bytes, PQ + PV, p.g.XLq, p.g.XLk, aq.plan);
+  if (rc != DLT_OK) return rc;
+  aq.plan.off_b = aq.plan.off_a + aq.plan.chunk_rows * aq.plan.chunk_x * PQ;
+  aq.plan.off_c = aq.plan.off_d = 0;
+
+  const int64_t grid_kv = (int64_t)p.B * p.H * p.g.TR * akv.plan.nblk_x;
+  const int64_t grid_q = (int64_t)p.B * p.H * p.g.TR * aq.plan.nblk_x;
+  if (grid_kv > 0x7fffffff || grid_q > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward: grid too large");
+  switch (dc.id) {
+    case 0: return dlt_launch_bwd_64_64(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
+    case 1: return dlt_launch_bwd_128_128(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
+    default: return dlt_launch_bwd_64_128(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
+  }
 }

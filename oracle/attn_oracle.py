@@ -86,7 +86,7 @@ def tiled_swa_ref(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_sca
     B, H, N, _ = q.shape
     n_tiles = t_height * t_width
     assert N == n_tiles * b_size, "seqlen should match image size"
-    allowed = torch.from_numpy(token_mask(b_size, t_height, t_width, row_size, col_size))
+    allowed = torch.from_numpy(token_mask(b_size, t_height, t_width, row_size, col_size).copy())
     attn_mask = torch.where(allowed, 0.0, MASK_VALUE).to(q.dtype)
     return F.scaled_dot_product_attention(q, k, v, attn_mask=attn_mask, scale=sm_scale)
 
@@ -94,7 +94,7 @@ def tiled_swa_ref(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_sca
 def tiled_swa_explicit(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale=1.0,
                        return_lse2: bool = False):
     """Same operator written out: softmax over the allowed set only (-inf fill)."""
-    allowed = torch.from_numpy(token_mask(b_size, t_height, t_width, row_size, col_size))
+    allowed = torch.from_numpy(token_mask(b_size, t_height, t_width, row_size, col_size).copy())
     s = torch.matmul(q, k.transpose(-1, -2)) * sm_scale
     s = s.masked_fill(~allowed, float("-inf"))
     p = torch.softmax(s, dim=-1)

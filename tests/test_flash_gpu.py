@@ -1,0 +1,100 @@
+"""GPU parity of flash attention (dlt_flash_fwd / dlt_flash_bwd) against SDPA on the CPU.
+
+Follows the reference's own check (src/flash_attn.py:616-659: q, k L2-normalised, loss =
+o.sum(), allclose(1e-2, 1e-2) on o, dq, dk, dv, Z=4, H in {4,8}, N in {512,2048},
+dv in {16,32}, dk in {16,64}) with seeded inputs, plus Lq != Lk, odd lengths, bf16 and the
+BASELINE tolerances (forward max-abs <= 2e-2, gradients relative <= 5e-2).
+"""
+import itertools
+import math
+
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+
+def _fa():
+    from dl_templates_amd import flash_attn
+    return flash_attn
+
+
+def _l2(x):
+    return x / torch.linalg.norm(x, dim=-1, keepdims=True)
+
+
+def _rel(got, want):
+    return ((got.float().cpu() - want).abs().max() / want.abs().max().clamp_min(1e-3)).item()
+
+
+SWEEP = list(itertools.product([False, True], [4, 8], [512, 2048], [16, 32], [16, 64]))
+
+
+@pytest.mark.parametrize("causal,head,n_ctx,h_dim,k_dim", SWEEP[::3] + [SWEEP[-1]])
+def test_reference_correctness_sweep(causal, head, n_ctx, h_dim, k_dim):
+    Z = 2 if n_ctx == 2048 else 4
+    g = torch.Generator().manual_seed(n_ctx + head + h_dim + k_dim)
+    q = _l2(torch.randn((Z, head, n_ctx, k_dim), generator=g)).half()
+    k = _l2(torch.randn((Z, head, n_ctx, k_dim), generator=g)).half()
+    v = torch.randn((Z, head, n_ctx, h_dim), generator=g).half()
+    do = torch.ones((Z, head, n_ctx, h_dim))
+    o_std, dq, dk, dv = orc.flash_grads(q.float(), k.float(), v.float(), do, causal, 1.0)
+    q2, k2, v2 = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(q2, k2, v2, causal, 1.0)
+    o.flatten().sum().backward()
+    assert torch.allclose(o.float().cpu(), o_std, atol=1e-2, rtol=1e-2)
+    assert torch.allclose(q2.grad.float().cpu(), dq, atol=1e-2, rtol=1e-2)
+    assert torch.allclose(k2.grad.float().cpu(), dk, atol=1e-2, rtol=1e-2)
+    assert torch.allclose(v2.grad.float().cpu(), dv, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("Lq,Lk,dk,dv,dtype", [
+    (256, 512, 64, 128, torch.bfloat16), (100, 333, 64, 128, torch.bfloat16), (1, 1, 16, 16, torch.bfloat16),
+    (129, 31, 32, 64, torch.float16), (64, 1000, 128, 128, torch.bfloat16), (300, 300, 64, 64, torch.float32),
+    (17, 257, 48, 80, torch.bfloat16)])
+def test_cross_attention_distinct_dims_and_lengths(Lq, Lk, dk, dv, dtype):
+    q, k, v, do = orc.make_qkv(Lq * 7 + Lk, 2, 3, Lq, Lk, dk, dv, dtype)
+    scale = 1 / math.sqrt(dk)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), False, scale)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(qg, kg, vg, False, scale)
+    o.backward(do.cuda())
+    assert o.shape == (2, 3, Lq, dv) and o.dtype == dtype
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert max(errs) <= 5e-2, errs
+
+
+def test_c5_shape_reduced_batch():
+    # BASELINE config 5 shape with B=1, H=2 (CPU oracle time): Lq=4096, Lk=8192, 64/128
+    q, k, v, do = orc.make_qkv(55, 1, 2, 4096, 8192, 64, 128, torch.bfloat16)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), False, 0.125)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(qg, kg, vg, False, 0.125)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    print("c5 rel errs", errs)
+    assert max(errs) <= 5e-2, errs
+
+
+def test_causal_matches_sdpa_bf16():
+    q, k, v, do = orc.make_qkv(56, 1, 2, 777, 777, 64, 64, torch.bfloat16)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), True, 0.125)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(qg, kg, vg, True, 0.125)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    assert max(_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w)) <= 5e-2
+
+
+def test_bad_arguments_raise():
+    from dl_templates_amd._lib import DltError
+    q = torch.randn(1, 1, 64, 64, dtype=torch.bfloat16).cuda()
+    k = torch.randn(1, 1, 128, 64, dtype=torch.bfloat16).cuda()
+    with pytest.raises(DltError):
+        _fa().attention(q, k, k, True, 1.0)  # causal needs Lq == Lk
+    with pytest.raises(AssertionError):
+        _fa().attention(q, k[..., :32], k, False, 1.0)

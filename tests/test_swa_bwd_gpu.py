@@ -1,0 +1,132 @@
+"""GPU parity of the SWA backward (dlt_swa_bwd through TiledSwa / TiledSwaRope autograd) against
+autograd through the fp32 CPU oracle on the same seeded inputs.
+
+Bar: max|g - g_ref| / max|g_ref| <= 5e-2 for dQ, dK, dV (bf16/fp16 MFMA, fp32 accumulation);
+gradients are bit-reproducible run to run (no atomics).
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+GRAD_TOL = 5e-2
+FWD_TOL = 2e-2
+
+
+def _swa():
+    from dl_templates_amd import tiled_swa
+    return tiled_swa
+
+
+def _rel(got, want):
+    return ((got.float().cpu() - want).abs().max() / want.abs().max().clamp_min(1e-3)).item()
+
+
+def _run(seed, B, H, b_size, th, tw, wr, wc, dk, dv, dtype, scale=None):
+    N = b_size * th * tw
+    q, k, v, do = orc.make_qkv(seed, B, H, N, N, dk, dv, dtype)
+    scale = 1.0 / math.sqrt(dk) if scale is None else scale
+    o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), b_size, th, tw, wr, wc, scale,
+                                                fn=orc.tiled_swa_explicit)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _swa().TiledSwa.apply(qg, kg, vg, b_size, th, tw, wr, wc, scale)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert qg.grad.dtype == dtype and kg.grad.dtype == dtype and vg.grad.dtype == dtype
+    assert max(errs) <= GRAD_TOL, f"rel errs dq/dk/dv = {errs}"
+    return errs
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_small_grid_dtypes(dtype):
+    _run(1, 2, 2, 1, 16, 16, 3, 3, 32, 32, dtype)
+
+
+@pytest.mark.parametrize("th,tw,wr,wc", [(7, 9, 2, 3), (3, 70, 1, 6), (20, 5, 6, 1), (1, 1, 0, 0), (9, 130, 3, 10), (6, 6, 8, 8)])
+def test_ragged_and_boundary_grids(th, tw, wr, wc):
+    _run(2, 1, 3, 1, th, tw, wr, wc, 64, 64, torch.bfloat16)
+
+
+def test_reference_demo_shape_b16():
+    # src/tiled_swa.py:736-750: S=16 (4x4 px), 16x16 tiles, W=1, d=32, scale 0.25; B, H reduced
+    _run(3, 1, 2, 16, 16, 16, 1, 1, 32, 32, torch.float16, scale=0.25)
+
+
+@pytest.mark.parametrize("b_size,th,tw,wr,wc", [(4, 6, 5, 1, 2), (3, 5, 4, 2, 1), (32, 3, 4, 1, 1), (2, 9, 9, 6, 6), (100, 2, 3, 1, 1)])
+def test_tiles_with_several_tokens(b_size, th, tw, wr, wc):
+    _run(4, 1, 2, b_size, th, tw, wr, wc, 32, 32, torch.bfloat16, scale=0.25)
+
+
+@pytest.mark.parametrize("dk,dv", [(64, 64), (128, 128), (64, 128), (16, 32), (40, 24), (128, 64)])
+def test_head_dims(dk, dv):
+    _run(5, 1, 2, 1, 12, 12, 3, 3, dk, dv, torch.bfloat16)
+
+
+def test_c3_shape_unfused_one_batch():
+    # BASELINE config 3 shape with B=1 (CPU oracle time), 64x64, d=64, 13x13
+    errs = _run(6, 1, 8, 1, 64, 64, 6, 6, 64, 64, torch.bfloat16)
+    print("c3 rel errs", errs)
+
+
+def test_backward_signature_and_determinism():
+    sw = _swa()
+    q, k, v, do = orc.make_qkv(7, 1, 2, 400, 400, 64, 64, torch.bfloat16)
+    outs = []
+    for _ in range(2):
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        o = sw.TiledSwa.apply(qg, kg, vg, 1, 20, 20, 4, 4, 0.125)
+        o.backward(do.cuda())
+        outs.append((qg.grad.clone(), kg.grad.clone(), vg.grad.clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    # softmax logits are invariant to scaling q up and k down: sum(dq*q) == sum(dk*k) per head
+    a = (outs[0][0].float() * q.cuda().float()).sum((-1, -2))
+    b = (outs[0][1].float() * k.cuda().float()).sum((-1, -2))
+    assert torch.allclose(a, b, atol=0.5, rtol=5e-2)
+
+
+def test_strided_grad_and_inputs():
+    sw = _swa()
+    B, H, th, tw, d = 2, 3, 8, 8, 64
+    N = th * tw
+    q, k, v, do = orc.make_qkv(8, B, H, N, N, d, d, torch.bfloat16)
+    _, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), 1, th, tw, 2, 2, 0.125)
+    qg = q.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3).requires_grad_(True)
+    kg = k.cuda().requires_grad_(True)
+    vg = v.cuda().requires_grad_(True)
+    o = sw.TiledSwa.apply(qg, kg, vg, 1, th, tw, 2, 2, 0.125)
+    dog = do.permute(0, 2, 1, 3).contiguous().cuda().permute(0, 2, 1, 3)
+    o.backward(dog)
+    assert max(_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w)) <= GRAD_TOL
+
+
+@pytest.mark.parametrize("R", [8, 4, 3])
+def test_fused_rope_backward(R):
+    sw = _swa()
+    B, H, th, tw, d = 1, 2, 16, 16, 64
+    N = th * tw
+    q, k, v, do = orc.make_qkv(9, B, H, N, N, d, d, torch.bfloat16)
+    idx = orc.make_rope_idx(10, th, tw, 0.05)
+    idx[7] = (3 << 16) | 0xFFFF
+    rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+    o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, 3, 3, 0.125)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, 3, 3, 0.125)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert max(errs) <= GRAD_TOL, errs
+    if R == 8:
+        # equals the unfused composition: rope (autograd) -> TiledSwa
+        from dl_templates_amd import fused_rope2d as fr
+        q2, k2, v2 = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        qr = fr.RotaryPE2D.apply(q2.clone().view(-1, N, d), idx.cuda(), rcs.cuda(), ccs.cuda()).view(q.shape)
+        kr = fr.RotaryPE2D.apply(k2.clone().view(-1, N, d), idx.cuda(), rcs.cuda(), ccs.cuda()).view(k.shape)
+        o2 = sw.TiledSwa.apply(qr, kr, v2, 1, th, tw, 3, 3, 0.125)
+        o2.backward(do.cuda())
+        assert torch.equal(o2, o)
+        assert torch.equal(q2.grad, qg.grad) and torch.equal(k2.grad, kg.grad) and torch.equal(v2.grad, vg.grad)
