@@ -1,0 +1,368 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+One "step" is one forward + backward pass of the fused RoPE-2D + tiled 2D sliding-window
+attention over one synthetic batch of BASELINE config 3 (bf16, B=2, H=8, 64x64 token grid,
+d=64, 13x13 window), inputs resident in HBM.  `value` is the effective TFLOP/s of that
+step (in-window FLOPs only: fwd 2*pairs*(dk+dv), bwd 2*pairs*(3dk+2dv)).  The JSON line also
+carries the roofline of the dominant kernel (per-kernel HIP-event durations taken inside the
+timed steps), the standalone RoPE-2D bandwidth (config 2), configs 4 / 5 as extras, and a CPU
+baseline: the eager-PyTorch oracle of the same step timed on the host cores.
+
+Only one GPU is used; --gpus N with N > 1 exits with a message.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+PEAK_HBM_GBPS = 8000.0     # MI355X HBM3E, published
+
+
+def axis_count(t, w):
+    w = min(w, t - 1)
+    return t * (2 * w + 1) - w * (w + 1)
+
+
+def swa_pairs(B, H, S, th, tw, wr, wc):
+    return B * H * S * S * axis_count(th, wr) * axis_count(tw, wc)
+
+
+def make_inputs(seed, B, H, Nq, Nk, dk, dv, dtype, device):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((B, H, Nq, dk), generator=g)
+    k = torch.randn((B, H, Nk, dk), generator=g)
+    v = torch.randn((B, H, Nk, dv), generator=g)
+    do = torch.randn((B, H, Nq, dv), generator=g)
+    return [t.to(dtype).to(device) for t in (q, k, v, do)]
+
+
+class Timer:
+    """K back-to-back repetitions between two events on torch's current stream (the stream the
+    library launches on)."""
+
+    @staticmethod
+    def run(fn, steps, warmup):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3 / steps
+        return e0.elapsed_time(e1) / steps, wall
+
+
+def kernel_breakdown(fn, steps):
+    """Average per-kernel duration (ms) over `steps` eager repetitions, from HIP events recorded
+    around every launch on the launch stream."""
+    from dl_templates_amd import _lib
+    torch.cuda.synchronize()
+    _lib.timing_enable(True)
+    try:
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        rec = _lib.timing_collect()
+    finally:
+        _lib.timing_enable(False)
+    acc = {}
+    for name, ms in rec:
+        s = acc.setdefault(name, [0.0, 0])
+        s[0] += ms
+        s[1] += 1
+    return {k: {"avg_ms": v[0] / v[1], "launches_per_step": v[1] / steps} for k, v in acc.items()}
+
+
+def try_graph(wl, steps, warmup):
+    """Replay `len(wl.calls)` steps (one per input set) from a captured HIP graph, so that host
+    launch cost is out of the picture; returns ms per step or None if capture fails.  The
+    library launches on the stream it is handed, so the capture stream is passed explicitly."""
+    try:
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        nsets = len(wl.calls)
+        with torch.cuda.graph(g, stream=s):
+            wl.stream.value = torch.cuda.current_stream().cuda_stream
+            for _ in range(nsets):
+                wl.step()
+        wl.stream.value = torch.cuda.current_stream().cuda_stream
+        reps = max(steps // nsets, 1)
+        ms, _ = Timer.run(g.replay, reps, max(warmup // nsets, 1))
+        return ms / nsets
+    except Exception as exc:  # pragma: no cover - depends on the runtime
+        wl.stream.value = torch.cuda.current_stream().cuda_stream
+        print(f"[bench] graph capture unavailable: {exc}", file=sys.stderr)
+        return None
+
+
+# ------------------------------------------------------------------------------------------ SWA
+class SwaWorkload:
+    def __init__(self, name, B, H, th, tw, W, d, fused_rope, nsets, seed=0, dtype=torch.bfloat16):
+        from dl_templates_amd import _lib, tiled_swa
+        from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
+        from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as Rope
+        self.name, self.B, self.H, self.th, self.tw, self.W, self.d = name, B, H, th, tw, W, d
+        dev = torch.device("cuda:0")
+        N = th * tw
+        self.sets = []
+        for i in range(nsets):
+            q, k, v, do = make_inputs(seed + i, B, H, N, N, d, d, dtype, dev)
+            o = torch.empty_like(v)
+            lse = torch.empty((B, H, N), dtype=torch.float32, device=dev)
+            delta = torch.empty_like(lse)
+            dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+            self.sets.append((q, k, v, do, o, lse, delta, dq, dk, dv))
+        self.shape = _lib.SwaShape(B, H, 1, th, tw, W, W, d, d, 1.0 / math.sqrt(d), _lib.dtype_code(self.sets[0][0]))
+        self.rope = None
+        if fused_rope:
+            g = torch.Generator().manual_seed(seed + 1000)
+            idx = Rope.encode_idx(th, tw).clone()
+            idx[torch.rand(N, generator=g) < 0.05] = -1
+            self.idx = idx.to(dev)
+            self.rcs = Ctx(16, th).cs_components.to(dev)
+            self.ccs = Ctx(16, tw).cs_components.to(dev)
+            self.rope, self._keep = _lib.rope_desc(self.idx, self.rcs, self.ccs)
+        self.lib = _lib.load()
+        self._lib = _lib
+        self.stream = _lib.stream_of(self.sets[0][0])
+        self.calls = [self._build_calls(s) for s in self.sets]
+        self.i = 0
+        self.pairs = swa_pairs(B, H, 1, th, tw, W, W)
+        self.flops_fwd = 2 * self.pairs * (d + d)
+        self.flops_bwd = 2 * self.pairs * (3 * d + 2 * d)
+
+    def _build_calls(self, s):
+        L = self._lib
+        q, k, v, do, o, lse, delta, dq, dk, dv = s
+        fwd = (L.ptr(q), L.strides(q), L.ptr(k), L.strides(k), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
+               L.ptr(lse), L.strides(lse), self.shape, self.rope, self.stream)
+        bwd = (L.ptr(q), L.strides(q), L.ptr(k), L.strides(k), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
+               L.ptr(do), L.strides(do), L.ptr(lse), L.ptr(delta), L.strides(lse), L.ptr(dq), L.strides(dq),
+               L.ptr(dk), L.strides(dk), L.ptr(dv), L.strides(dv), self.shape, self.rope, self.stream)
+        return fwd, bwd
+
+    def step(self):
+        fwd, bwd = self.calls[self.i % len(self.calls)]
+        self.i += 1
+        rc = self.lib.dlt_swa_fwd(*fwd)
+        rc = rc or self.lib.dlt_swa_bwd(*bwd)
+        if rc:
+            self._lib.check(rc)
+
+    def fwd_only(self):
+        fwd, _ = self.calls[self.i % len(self.calls)]
+        self.i += 1
+        rc = self.lib.dlt_swa_fwd(*fwd)
+        if rc:
+            self._lib.check(rc)
+
+    def kernel_flops(self):
+        d = self.d
+        return {"attn_fwd": self.flops_fwd, "attn_bwd_kv": 2 * self.pairs * (2 * d + 2 * d), "attn_bwd_q": 2 * self.pairs * d}
+
+
+class FlashWorkload:
+    def __init__(self, B, H, Lq, Lk, dk, dv, seed=0, dtype=torch.bfloat16):
+        from dl_templates_amd import _lib
+        dev = torch.device("cuda:0")
+        q, k, v, do = make_inputs(seed, B, H, Lq, Lk, dk, dv, dtype, dev)
+        o = torch.empty((B, H, Lq, dv), dtype=dtype, device=dev)
+        lse = torch.empty((B, H, Lq), dtype=torch.float32, device=dev)
+        delta = torch.empty_like(lse)
+        dq, dkk, dvv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        self.keep = (q, k, v, do, o, lse, delta, dq, dkk, dvv)
+        L = _lib
+        shape = L.FlashShape(B, H, Lq, Lk, dk, dv, 1.0 / math.sqrt(dk), 0, L.dtype_code(q))
+        st = L.stream_of(q)
+        self.fwd = (L.ptr(q), L.strides(q), L.ptr(k), L.strides(k), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
+                    L.ptr(lse), L.strides(lse), shape, st)
+        self.bwd = (L.ptr(q), L.strides(q), L.ptr(k), L.strides(k), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
+                    L.ptr(do), L.strides(do), L.ptr(lse), L.ptr(delta), L.strides(lse), L.ptr(dq), L.strides(dq),
+                    L.ptr(dkk), L.strides(dkk), L.ptr(dvv), L.strides(dvv), shape, st)
+        self.lib, self._lib = L.load(), L
+        pairs = B * H * Lq * Lk
+        self.flops_fwd = 2 * pairs * (dk + dv)
+        self.flops_bwd = 2 * pairs * (3 * dk + 2 * dv)
+
+    def step(self):
+        rc = self.lib.dlt_flash_fwd(*self.fwd) or self.lib.dlt_flash_bwd(*self.bwd)
+        if rc:
+            self._lib.check(rc)
+
+
+# ------------------------------------------------------------------------------------------ RoPE
+def bench_rope(steps, warmup):
+    """Config 2: B=4, H=8, 64x64, d=64, first 32 dims rotated, 5% no-PE, q and k in one launch.
+    `cold` cycles through > 512 MB of distinct (q, k) pairs so that the 256 MB infinity cache
+    cannot hold the working set; `hot` reuses one pair."""
+    from dl_templates_amd import _lib
+    from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
+    from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as Rope
+    dev = torch.device("cuda:0")
+    B, H, N, C, R = 4, 8, 4096, 64, 8
+    g = torch.Generator().manual_seed(2)
+    idx = Rope.encode_idx(64, 64).clone()
+    idx[torch.rand(N, generator=g) < 0.05] = -1
+    n_pe = int((idx >= 0).sum())
+    idx = idx.to(dev)
+    rcs, ccs = Ctx(16, 64).cs_components.to(dev), Ctx(16, 64).cs_components.to(dev)
+    desc, keep = _lib.rope_desc(idx, rcs, ccs)
+    lib = _lib.load()
+    nbuf = 17  # 17 * 2 * 16.8 MB = 570 MB
+    bufs = [(torch.randn(B * H, N, C, generator=g).to(torch.bfloat16).to(dev),
+             torch.randn(B * H, N, C, generator=g).to(torch.bfloat16).to(dev)) for _ in range(nbuf)]
+    st = _lib.stream_of(idx)
+    calls = [(_lib.ptr(q), _lib.strides(q), B * H, _lib.ptr(k), _lib.strides(k), B * H, N, C, desc, 0, _lib.DLT_BF16, st)
+             for q, k in bufs]
+    state = {"i": 0}
+
+    def cold():
+        rc = lib.dlt_rope2d_pair(*calls[state["i"] % nbuf])
+        state["i"] += 1
+        if rc:
+            _lib.check(rc)
+
+    def hot():
+        rc = lib.dlt_rope2d_pair(*calls[0])
+        if rc:
+            _lib.check(rc)
+
+    # algorithmic bytes: read + write of the 4R rotated dims of tokens with a rotated axis, idx once, x2 tensors
+    alg_bytes = 2 * (2 * 2 * (B * H) * n_pe * 4 * R) + 4 * N
+    out = {"alg_bytes": alg_bytes, "n_pe_tokens": n_pe}
+    for name, fn in (("cold", cold), ("hot", hot)):
+        ms_ev, _ = Timer.run(fn, steps * 5, warmup * 5)
+        kb = kernel_breakdown(fn, steps * 5)
+        kms = kb["rope2d"]["avg_ms"]
+        out[name] = {"us_per_launch_back_to_back": ms_ev * 1e3, "us_kernel_events": kms * 1e3,
+                     "gbps": alg_bytes / (kms * 1e-3) / 1e9, "frac_of_hbm_peak": alg_bytes / (kms * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+    del keep
+    return out
+
+
+# ------------------------------------------------------------------------------------------ CPU baseline
+def cpu_baseline_c3():
+    """The oracle (eager PyTorch, fp32) of the same fused step on the host cores: one repetition of
+    the whole config-3 step after one warm-up on a quarter of the heads."""
+    from oracle import attn_oracle as orc
+    B, H, th, tw, W, d = 2, 8, 64, 64, 6, 64
+    N = th * tw
+    q, k, v, do = orc.make_qkv(0, B, H, N, N, d, d, torch.float32)
+    idx = orc.make_rope_idx(1000, th, tw, 0.05)
+    rcs, ccs = orc.rope_tables(8, th), orc.rope_tables(8, tw)
+    args = (idx, rcs, ccs, 1, th, tw, W, W, 1.0 / math.sqrt(d))
+    orc.rope_swa_grads(q[:, :2], k[:, :2], v[:, :2], do[:, :2], *args)
+    t0 = time.perf_counter()
+    orc.rope_swa_grads(q, k, v, do, *args)
+    dt = time.perf_counter() - t0
+    pairs = swa_pairs(B, H, 1, th, tw, W, W)
+    flops = 2 * pairs * (d + d) + 2 * pairs * (5 * d)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"whole config-3 step (B=2,H=8,64x64,d=64,13x13, fp32 eager masked SDPA + autograd), 1 repetition, {dt * 1e3:.0f} ms",
+            "ms_per_step": dt * 1e3, "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--quick", action="store_true", help="skip the extra configs and the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the hot path shards over batch*heads with no exchange); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    torch.cuda.set_device(0)
+    K, W = args.steps, args.warmup
+
+    # ---- main workload: config 3, fused RoPE, 4 input sets cycled (about 400 MB touched per cycle)
+    wl = SwaWorkload("C3", 2, 8, 64, 64, 6, 64, fused_rope=True, nsets=4)
+    ms_eager, wall_eager = Timer.run(wl.step, K, W)
+    kb = kernel_breakdown(wl.step, K)
+    ms_graph = try_graph(wl, K, W)
+    ms_step = ms_graph if ms_graph is not None else ms_eager
+    flops_step = wl.flops_fwd + wl.flops_bwd
+    value = flops_step / (ms_step * 1e-3) / 1e12
+
+    kflops = wl.kernel_flops()
+    dom = max((k for k in kb if k in kflops), key=lambda k: kb[k]["avg_ms"])
+    ach = kflops[dom] / (kb[dom]["avg_ms"] * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None,
+                "avg_launch_ms": kb[dom]["avg_ms"], "alg_flops_per_launch": kflops[dom]}
+    kernels = {}
+    for k_, v_ in kb.items():
+        kernels[k_] = {"avg_ms": v_["avg_ms"]}
+        if k_ in kflops:
+            kernels[k_]["eff_tflops"] = kflops[k_] / (v_["avg_ms"] * 1e-3) / 1e12
+            kernels[k_]["frac_mfma_peak"] = kernels[k_]["eff_tflops"] / PEAK_BF16_TFLOPS
+
+    extra = {"ms_per_step_eager_events": ms_eager, "ms_per_step_eager_wall": wall_eager, "ms_per_step_graph": ms_graph,
+             "step_source": "hip graph replay" if ms_graph is not None else "eager launches",
+             "frac_mfma_peak_effective": value / PEAK_BF16_TFLOPS, "kernels": kernels,
+             "hbm_floor_ms": 101e6 / (PEAK_HBM_GBPS * 1e9) * 1e3}
+
+    rope = bench_rope(K, W)
+    extra["rope2d_c2"] = rope
+
+    if not args.quick:
+        for name, (B, H, th, tw, Wn, d) in {"C4_128x128": (1, 16, 128, 128, 10, 128), "C4_96x160": (1, 16, 96, 160, 10, 128)}.items():
+            w4 = SwaWorkload(name, B, H, th, tw, Wn, d, fused_rope=False, nsets=1)
+            ms4, _ = Timer.run(w4.step, max(K // 5, 3), 2)
+            kb4 = kernel_breakdown(w4.step, 3)
+            f4 = w4.flops_fwd + w4.flops_bwd
+            extra[name] = {"ms_per_step": ms4, "eff_tflops": f4 / (ms4 * 1e-3) / 1e12,
+                           "frac_mfma_peak": f4 / (ms4 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                           "kernels_ms": {k_: v_["avg_ms"] for k_, v_ in kb4.items()}}
+            del w4
+        w5 = FlashWorkload(2, 16, 4096, 8192, 64, 128)
+        ms5, _ = Timer.run(w5.step, max(K // 5, 3), 2)
+        kb5 = kernel_breakdown(w5.step, 3)
+        f5 = w5.flops_fwd + w5.flops_bwd
+        extra["C5_flash"] = {"ms_per_step": ms5, "eff_tflops": f5 / (ms5 * 1e-3) / 1e12,
+                             "frac_mfma_peak": f5 / (ms5 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                             "kernels_ms": {k_: v_["avg_ms"] for k_, v_ in kb5.items()}}
+        del w5
+
+    cpu = None if args.quick else cpu_baseline_c3()
+
+    line = {
+        "metric": "swa2d_fwd_bwd_effective_tflops", "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C3: fused RoPE-2D + tiled 2D SWA fwd+bwd, B=2 H=8 64x64 grid b_size=1 d=64 13x13 window, "
+                               "bf16, 5% no-PE tokens, 4 input sets cycled",
+                   "peak_bf16_tflops": PEAK_BF16_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS},
+        "roofline": roofline, "cpu_baseline": cpu,
+        "rope2d_gbps": rope["cold"]["gbps"], "rope2d_frac_hbm": rope["cold"]["frac_of_hbm_peak"],
+        "extra": extra,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -25,7 +25,9 @@ _DTYPES = {torch.bfloat16: DLT_BF16, torch.float16: DLT_FP16, torch.float32: DLT
 EXPORTS = (
     "dlt_last_error", "dlt_version", "dlt_rope2d", "dlt_rope2d_pair", "dlt_rope_pe_mask",
     "dlt_swa_fwd", "dlt_swa_bwd", "dlt_swa_neighbors", "dlt_flash_fwd", "dlt_flash_bwd",
+    "dlt_timing_enable", "dlt_timing_collect",
 )
+KERNEL_NAMES = ("rope2d", "attn_fwd", "attn_delta", "attn_bwd_kv", "attn_bwd_q")
 
 
 class DltError(RuntimeError):
@@ -42,6 +44,10 @@ class RopeDesc(Structure):
         ("row_cs_stride0", c_int64), ("col_cs_stride0", c_int64),
         ("n_rdim", c_int32), ("row_len", c_int32), ("col_len", c_int32),
     ]
+
+
+class KernelTime(Structure):
+    _fields_ = [("kernel", c_int32), ("ms", c_float)]
 
 
 class SwaShape(Structure):
@@ -99,6 +105,10 @@ def _declare(lib) -> None:
     lib.dlt_flash_fwd.argtypes = fwd + [POINTER(FlashShape), c_void_p]
     lib.dlt_flash_bwd.restype = c_int
     lib.dlt_flash_bwd.argtypes = bwd + [POINTER(FlashShape), c_void_p]
+    lib.dlt_timing_enable.restype = c_int
+    lib.dlt_timing_enable.argtypes = [c_int]
+    lib.dlt_timing_collect.restype = c_int
+    lib.dlt_timing_collect.argtypes = [POINTER(KernelTime), c_int, POINTER(c_int)]
 
 
 def load():
@@ -120,6 +130,18 @@ def load():
 def check(rc: int) -> None:
     if rc != 0:
         raise DltError(rc, load().dlt_last_error().decode("utf-8", "replace"))
+
+
+def timing_enable(on: bool) -> None:
+    check(load().dlt_timing_enable(int(on)))
+
+
+def timing_collect(max_records: int = 1 << 16):
+    """[(kernel name, milliseconds)] for every launch since the last collect, in launch order."""
+    buf = (KernelTime * max_records)()
+    n = c_int(0)
+    check(load().dlt_timing_collect(buf, max_records, ctypes.byref(n)))
+    return [(KERNEL_NAMES[buf[i].kernel], float(buf[i].ms)) for i in range(min(n.value, max_records))]
 
 
 def dtype_code(t: torch.Tensor) -> int:

@@ -13,6 +13,66 @@ int dlt_set_error(int code, const char* fmt, ...) {
   return code;
 }
 
+// ---- per-kernel timing ------------------------------------------------------------------
+#include <vector>
+namespace {
+struct TimedLaunch { int kernel; hipEvent_t e0, e1; };
+thread_local bool g_timing = false;
+thread_local std::vector<TimedLaunch> g_launches;
+thread_local std::vector<hipEvent_t> g_event_pool;
+
+hipEvent_t take_event() {
+  if (!g_event_pool.empty()) {
+    hipEvent_t e = g_event_pool.back();
+    g_event_pool.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) return nullptr;
+  return e;
+}
+}  // namespace
+
+void dlt_timing_before(int kernel_id, hipStream_t stream) {
+  if (!g_timing) return;
+  TimedLaunch t{kernel_id, take_event(), take_event()};
+  if (t.e0 == nullptr || t.e1 == nullptr) return;
+  (void)hipEventRecord(t.e0, stream);
+  g_launches.push_back(t);
+}
+
+void dlt_timing_after(hipStream_t stream) {
+  if (!g_timing || g_launches.empty()) return;
+  (void)hipEventRecord(g_launches.back().e1, stream);
+}
+
+extern "C" int dlt_timing_enable(int on) {
+  g_timing = on != 0;
+  return DLT_OK;
+}
+
+extern "C" int dlt_timing_collect(dlt_kernel_time_t* out, int max, int* n) {
+  DLT_REQUIRE(n != nullptr, "timing_collect: n is NULL");
+  DLT_REQUIRE(out != nullptr || max == 0, "timing_collect: out is NULL");
+  *n = (int)g_launches.size();
+  int i = 0;
+  for (const TimedLaunch& t : g_launches) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(t.e1);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, t.e0, t.e1);
+    if (e != hipSuccess) {
+      g_launches.clear();
+      return dlt_set_error(DLT_ERR_LAUNCH, "timing_collect: %s", hipGetErrorString(e));
+    }
+    if (i < max) { out[i].kernel = t.kernel; out[i].ms = ms; }
+    i++;
+    g_event_pool.push_back(t.e0);
+    g_event_pool.push_back(t.e1);
+  }
+  g_launches.clear();
+  return DLT_OK;
+}
+
 extern "C" const char* dlt_last_error(void) { return g_err; }
 extern "C" int dlt_version(void) { return 1; }
 

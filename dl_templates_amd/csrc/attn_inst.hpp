@@ -22,7 +22,9 @@ int launch_fwd_t(const FwdArgs& a, int grid, hipStream_t stream) {
   auto kern = attn_fwd_kernel<TIO, DLT_DK, DLT_DV, NP>;
   int rc = set_lds_limit(kern, a.plan.lds_bytes);
   if (rc != DLT_OK) return rc;
+  dlt_timing_before(DLT_K_FWD, stream);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), a.plan.lds_bytes, stream, a);
+  dlt_timing_after(stream);
   DLT_CHECK_LAUNCH("attention forward launch");
   return DLT_OK;
 }
@@ -32,21 +34,27 @@ int launch_bwd_t(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q,
   {
     constexpr int CH = DLT_DV / 8;
     const int64_t threads = (int64_t)aq.p.B * aq.p.H * aq.n_tokens_q * CH;
+    dlt_timing_before(DLT_K_DELTA, stream);
     hipLaunchKernelGGL((attn_delta_kernel<TIO, DLT_DV>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, aq);
+    dlt_timing_after(stream);
     DLT_CHECK_LAUNCH("attention delta launch");
   }
   {
     auto kern = attn_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP>;
     int rc = set_lds_limit(kern, akv.plan.lds_bytes);
     if (rc != DLT_OK) return rc;
+    dlt_timing_before(DLT_K_BWD_KV, stream);
     hipLaunchKernelGGL(kern, dim3(grid_kv), dim3(256), akv.plan.lds_bytes, stream, akv);
+    dlt_timing_after(stream);
     DLT_CHECK_LAUNCH("attention dK/dV launch");
   }
   {
     auto kern = attn_bwd_q_kernel<TIO, DLT_DK, DLT_DV, NP>;
     int rc = set_lds_limit(kern, aq.plan.lds_bytes);
     if (rc != DLT_OK) return rc;
+    dlt_timing_before(DLT_K_BWD_Q, stream);
     hipLaunchKernelGGL(kern, dim3(grid_q), dim3(256), aq.plan.lds_bytes, stream, aq);
+    dlt_timing_after(stream);
     DLT_CHECK_LAUNCH("attention dQ launch");
   }
   return DLT_OK;

@@ -23,6 +23,10 @@ int dlt_set_error(int code, const char* fmt, ...) __attribute__((format(printf, 
       return dlt_set_error(DLT_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e__));         \
   } while (0)
 
+// per-kernel timing hooks (no-ops unless dlt_timing_enable(1) was called on this thread)
+void dlt_timing_before(int kernel_id, hipStream_t stream);
+void dlt_timing_after(hipStream_t stream);
+
 static inline int dlt_elem_size(int dtype) { return dtype == DLT_FP32 ? 4 : 2; }
 
 // ---- rotary operands as the kernels see them ------------------------------------------

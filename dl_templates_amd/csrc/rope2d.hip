@@ -147,8 +147,10 @@ int launch_rope(const RopeKArgs& a, bool vec, hipStream_t stream, int ntens) {
   if (gx > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "rope2d: too many tokens (%lld)", (long long)a.N);
   const int maxb = dlt_imax(a.nb[0], ntens > 1 ? a.nb[1] : 0);
   dim3 grid((unsigned)gx, (unsigned)((maxb + a.bb - 1) / a.bb), (unsigned)ntens);
+  dlt_timing_before(DLT_K_ROPE, stream);
   if (vec) hipLaunchKernelGGL(rope2d_vec_kernel<T>, grid, dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(rope2d_generic_kernel<T>, grid, dim3(256), 0, stream, a);
+  dlt_timing_after(stream);
   DLT_CHECK_LAUNCH("rope2d launch");
   return DLT_OK;
 }

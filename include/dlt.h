@@ -141,6 +141,21 @@ int dlt_flash_bwd(const void* q, const int64_t q_strides[4], const void* k, cons
                   void* dv, const int64_t dv_strides[4],
                   const dlt_flash_shape_t* shape, void* stream);
 
+/* ---- per-kernel timing (measurement aid) ---------------------------------------------------
+ * Counterpart of the reference's triton.testing.do_bench calls (src/tiled_swa.py:765-774,
+ * src/flash_attn.py:592,606), at kernel granularity.  While enabled for the calling thread,
+ * every kernel the library launches is bracketed by a pair of hipEvents recorded on the
+ * launch stream.  dlt_timing_collect waits for the recorded events, writes up to `max`
+ * records in launch order, stores the number available in *n and clears the list.
+ * Enabling creates events lazily (host-side handles only, no device allocation). */
+enum { DLT_K_ROPE = 0, DLT_K_FWD = 1, DLT_K_DELTA = 2, DLT_K_BWD_KV = 3, DLT_K_BWD_Q = 4, DLT_K_COUNT = 5 };
+typedef struct {
+  int32_t kernel; /* DLT_K_* */
+  float ms;
+} dlt_kernel_time_t;
+int dlt_timing_enable(int on);
+int dlt_timing_collect(dlt_kernel_time_t* out, int max, int* n);
+
 #ifdef __cplusplus
 }
 #endif
