@@ -29,15 +29,22 @@ int launch_fwd_t(const FwdArgs& a, int grid, hipStream_t stream) {
   return DLT_OK;
 }
 
+template <typename TIO>
+int launch_delta_t(const BwdArgs& aq, hipStream_t stream) {
+  constexpr int CH = DLT_DV / 8;
+  const int64_t threads = (int64_t)aq.p.B * aq.p.H * aq.n_tokens_q * CH;
+  dlt_timing_before(DLT_K_DELTA, stream);
+  hipLaunchKernelGGL((attn_delta_kernel<TIO, DLT_DV>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, aq);
+  dlt_timing_after(stream);
+  DLT_CHECK_LAUNCH("attention delta launch");
+  return DLT_OK;
+}
+
 template <typename TIO, int NP>
 int launch_bwd_t(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q, hipStream_t stream) {
   {
-    constexpr int CH = DLT_DV / 8;
-    const int64_t threads = (int64_t)aq.p.B * aq.p.H * aq.n_tokens_q * CH;
-    dlt_timing_before(DLT_K_DELTA, stream);
-    hipLaunchKernelGGL((attn_delta_kernel<TIO, DLT_DV>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, aq);
-    dlt_timing_after(stream);
-    DLT_CHECK_LAUNCH("attention delta launch");
+    int rc = launch_delta_t<TIO>(aq, stream);
+    if (rc != DLT_OK) return rc;
   }
   {
     auto kern = attn_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP>;
@@ -60,6 +67,14 @@ int launch_bwd_t(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q,
   return DLT_OK;
 }
 }  // namespace
+
+int DLT_CAT3(dlt_launch_delta_, DLT_DK, DLT_DV)(const BwdArgs& a, hipStream_t stream) {
+  switch (a.p.dtype) {
+    case DLT_BF16: return launch_delta_t<bf16_t>(a, stream);
+    case DLT_FP16: return launch_delta_t<f16_t>(a, stream);
+    default: return launch_delta_t<float>(a, stream);
+  }
+}
 
 int DLT_CAT3(dlt_launch_bwd_, DLT_DK, DLT_DV)(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q, int np,
                                               hipStream_t stream) {

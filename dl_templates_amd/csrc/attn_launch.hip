@@ -2,6 +2,8 @@
 // per-launch LDS / chunking plan, and dispatch to the instantiation for the padded head dims.
 #include "attn_fwd_kernel.hpp"
 #include "attn_bwd_kernel.hpp"
+#include "swa1_fwd_kernel.hpp"
+#include "swa1_bwd_kernel.hpp"
 
 int dlt_launch_fwd_64_64(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_128_128(const FwdArgs&, int, int, hipStream_t);
@@ -10,6 +12,13 @@ int dlt_launch_fwd_64_128(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_64_64(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_128_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_64_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
+
+int dlt_launch_delta_64_64(const BwdArgs&, hipStream_t);
+int dlt_launch_delta_128_128(const BwdArgs&, hipStream_t);
+int dlt_swa1_launch_bwd_64(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
+int dlt_swa1_launch_bwd_128(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
+int dlt_swa1_launch_fwd_64(const Swa1FwdArgs&, int, int, hipStream_t);
+int dlt_swa1_launch_fwd_128(const Swa1FwdArgs&, int, int, hipStream_t);
 
 namespace {
 
@@ -68,6 +77,106 @@ int make_plan(const AttnProblem& p, int own, int own_bytes, int per_tok, int XL_
   return DLT_OK;
 }
 
+// ---- token-grid (b_size == 1) fast path ----------------------------------------------------
+struct Swa1Class { int D, wclass, pbit; };
+
+// Can the token-grid kernels take this problem?  They need 16-byte vector access to the
+// streamed tensors, both head dims in one padded class, a window of at most 21 columns and,
+// with rotation, rotary partners a power-of-two number of 8-dim chunks apart.
+bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streamed, Swa1Class& c) {
+  if (p.g.mode != DLT_GEOM_SWA || p.g.S != 1) return false;
+  if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
+  if (p.dk <= 64 && p.dv <= 64) c.D = 64;
+  else if (p.dk <= 128 && p.dv <= 128 && p.dk > 64 && p.dv > 64) c.D = 128;
+  else return false;
+  for (int i = 0; i < n_streamed; i++)
+    if (!streamed_vec[i]) return false;
+  if ((int64_t)p.g.TR * p.g.TC >= ((int64_t)1 << 31) / 1024) return false;  // 32-bit element offsets inside a slab
+  const int ncg = (4 + 2 * p.g.WC + 3) / 4;
+  if (ncg > 6) return false;
+  c.wclass = ncg <= 4 ? 0 : 1;
+  c.pbit = 1;
+  if (p.rope.enabled && p.rope.R > 0) {
+    const int r8 = p.rope.R / 8;
+    if (p.rope.R % 8 != 0 || (r8 & (r8 - 1)) != 0 || 4 * p.rope.R > c.D) return false;
+    if ((uintptr_t)p.rope.row_cs % 4 != 0) return false;
+    c.pbit = r8;
+  }
+  return true;
+}
+
+// n_regions: [8 rows x HCW tokens] LDS regions the kernel keeps resident
+void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int extra_bytes, Swa1Plan& plan) {
+  plan.ncg = (4 + 2 * p.g.WC + 3) / 4;
+  const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
+  plan.HRP = roundup(4 + 2 * p.g.WR, 8);
+  plan.nblk_r = (p.g.TR + 3) / 4;
+  plan.nblk_c = (p.g.TC + 15) / 16;
+  plan.lds_bytes = n_regions * 8 * hcw * (c.D * 2 + 16) + extra_bytes;
+}
+
+// the token-grid kernels index a [N, D] slab with 32-bit element offsets
+bool swa1_strides_fit(const AttnTensors& t) {
+  const int64_t lim = (int64_t)1 << 20;
+  return t.qs[2] < lim && t.ks[2] < lim && t.vs[2] < lim && (t.d_o == nullptr || t.dos[2] < lim);
+}
+
+int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c, hipStream_t stream) {
+  const int es = dlt_elem_size(p.dtype);
+  // delta pre-pass (shared with the generic path)
+  BwdArgs d;
+  d.p = p;
+  d.o = t.o; d.d_o = t.d_o; d.delta = t.delta;
+  for (int i = 0; i < 4; i++) { d.os[i] = t.os[i]; d.dos[i] = t.dos[i]; }
+  for (int i = 0; i < 3; i++) d.ls[i] = t.ls[i];
+  d.o_vec = vec_ok(t.o, t.os, 4, p.dv, es);
+  d.do_vec = vec_ok(t.d_o, t.dos, 4, p.dv, es);
+  d.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
+  int rc = c.D == 64 ? dlt_launch_delta_64_64(d, stream) : dlt_launch_delta_128_128(d, stream);
+  if (rc != DLT_OK) return rc;
+
+  Swa1BwdArgs a;
+  a.p = p;
+  swa1_make_plan(p, c, 2, 0, a.plan);
+  const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
+  const int lds_q = a.plan.lds_bytes, lds_kv = a.plan.lds_bytes + 2 * 8 * hcw * 4;
+  a.q = t.q; a.k = t.k; a.v = t.v; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
+  for (int i = 0; i < 4; i++) {
+    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.dos[i] = t.dos[i];
+    a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
+  }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.q_vec = 1; a.k_vec = 1; a.v_vec = 1; a.do_vec = 1;
+  a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, es);
+  a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, es);
+  a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, es);
+  a.rope_pbit = c.pbit;
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
+  if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward: grid too large");
+  return c.D == 64 ? dlt_swa1_launch_bwd_64(a, c.wclass, (int)grid, lds_kv, lds_q, stream)
+                   : dlt_swa1_launch_bwd_128(a, c.wclass, (int)grid, lds_kv, lds_q, stream);
+}
+
+int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c, hipStream_t stream) {
+  const int es = dlt_elem_size(p.dtype);
+  Swa1FwdArgs a;
+  a.p = p;
+  swa1_make_plan(p, c, 2, 0, a.plan);
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
+  for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.q_vec = vec_ok(t.q, t.qs, 4, p.dk, es);
+  a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, es);
+  a.rope_pbit = c.pbit;
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
+  if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: grid too large");
+  return c.D == 64 ? dlt_swa1_launch_fwd_64(a, c.wclass, (int)grid, stream)
+                   : dlt_swa1_launch_fwd_128(a, c.wclass, (int)grid, stream);
+}
+
 }  // namespace
 
 int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
@@ -75,6 +184,14 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
   int rc = pick_dims(p, dc);
   if (rc != DLT_OK) return rc;
   const int es = dlt_elem_size(p.dtype);
+  {
+    const bool streamed[2] = {vec_ok(t.k, t.ks, 4, p.dk, es), vec_ok(t.v, t.vs, 4, p.dv, es)};
+    Swa1Class c;
+    if (swa1_eligible(p, streamed, 2, c) && swa1_strides_fit(t)) {
+      rc = swa1_forward(p, t, c, stream);
+      if (rc != -1) return rc;
+    }
+  }
   const int np = p.g.mode == DLT_GEOM_SWA ? 1 : 2;
   const int own = 64 * np;
   const int PQ = dc.DK * 2 + 16, PK = dc.DK * 2 + 16, PV = dc.DV * 2 + 16, PO = dc.DV * es + 16;
@@ -106,6 +223,12 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
   int rc = pick_dims(p, dc);
   if (rc != DLT_OK) return rc;
   const int es = dlt_elem_size(p.dtype);
+  {
+    const bool streamed[4] = {vec_ok(t.q, t.qs, 4, p.dk, es), vec_ok(t.k, t.ks, 4, p.dk, es),
+                              vec_ok(t.v, t.vs, 4, p.dv, es), vec_ok(t.d_o, t.dos, 4, p.dv, es)};
+    Swa1Class c;
+    if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(t)) return swa1_backward(p, t, c, stream);
+  }
   const int np = 1;
   const int own = 64 * np;
   const int PQ = dc.DK * 2 + 16, PV = dc.DV * 2 + 16;

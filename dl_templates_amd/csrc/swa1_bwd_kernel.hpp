@@ -1,0 +1,367 @@
+// Backward kernels for token grids (b_size == 1): the decoupled dK/dV and dQ passes of
+// tiled_swa_bwd_large_kernel_decoupled_q (src/tiled_swa.py:407-562) on the 2D-patch / shared
+// halo structure of the token-grid forward kernel.  The reference has no backward for tiles of
+// fewer than 16 tokens (src/tiled_swa.py:660-661).
+//
+//   dK/dV: a wave owns a 4x4 patch of keys; the queries that can see them (their halo, by the
+//          symmetry of the window) stream through LDS in chunks of 8 rows: Q (rotated when
+//          the rotary encoding is fused), dO, lse2 and delta.
+//   dQ   : a wave owns a 4x4 patch of queries; K (rotated) and V stream through LDS.
+// Both recompute P = exp2(s * scale - lse2) per block; tokens of the streamed side are the MFMA
+// rows, so P / dS leave the first products in the layout the second products take as B operand.
+#pragma once
+#include "swa1_common.hpp"
+
+struct Swa1BwdArgs {
+  AttnProblem p;
+  Swa1Plan plan;
+  const void *q, *k, *v, *d_o;
+  const float *lse, *delta;
+  void *dq, *dk, *dv;
+  int64_t qs[4], ks[4], vs[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int32_t q_vec, k_vec, v_vec, do_vec, dq_vec, dk_vec, dv_vec;
+  int32_t rope_pbit;
+  float scale_log2;
+};
+
+// per-token fp32 values (lse2 / delta) of halo rows [cr0, cr0 + 8): 8 * HCW values over 256 threads
+template <int HCW>
+struct ScalarRegs { float v[(8 * HCW + 255) / 256]; };
+
+template <int HCW>
+DLT_DEV void swa1_issue_scalar(ScalarRegs<HCW>& sr, const float* base, int64_t stride, const Swa1Geom& G, int cr0, int tid) {
+#pragma unroll
+  for (int it = 0; it < (8 * HCW + 255) / 256; it++) {
+    const int idx = tid + 256 * it;
+    sr.v[it] = 0.f;
+    if (idx < 8 * HCW) {
+      const int hr = idx / HCW, hc = idx - hr * HCW;
+      const int r = G.r0 - G.WR + cr0 + hr, c = G.c0 - G.WC + hc;
+      if ((unsigned)r < (unsigned)G.TR && (unsigned)c < (unsigned)G.TC) sr.v[it] = base[(int64_t)(r * G.TC + c) * stride];
+    }
+  }
+}
+
+template <int HCW>
+DLT_DEV void swa1_commit_scalar(const ScalarRegs<HCW>& sr, float* s, int tid) {
+#pragma unroll
+  for (int it = 0; it < (8 * HCW + 255) / 256; it++) {
+    const int idx = tid + 256 * it;
+    if (idx < 8 * HCW) s[idx] = sr.v[it];
+  }
+}
+
+// shared prologue: workgroup -> band, lane -> window biases
+template <int NCGMAX>
+struct Swa1Lane {
+  Swa1Geom G;
+  int b, h;
+  int rlo, rhi;
+  float cbias[NCGMAX][4];
+  bool cg_edge[NCGMAX];
+  int wcol_lo, wcol_hi;
+  bool wave_ok;
+  int ch_first, ch_last;
+
+  DLT_DEV void init(const AttnProblem& p, const Swa1Plan& P, int wave, int n) {
+    const int lin = xcd_remap(blockIdx.x, gridDim.x);
+    const int per_bh = P.nblk_r * P.nblk_c;
+    const int bh = lin / per_bh;
+    const int rem = lin - bh * per_bh;
+    const int br = rem / P.nblk_c;
+    b = bh / p.H;
+    h = bh - b * p.H;
+    G.r0 = 4 * br; G.c0 = 16 * (rem - br * P.nblk_c);
+    G.TR = p.g.TR; G.TC = p.g.TC; G.WR = p.g.WR; G.WC = p.g.WC;
+    const int qr_l = n >> 2, qc_l = n & 3;
+    const int cw = G.c0 + 4 * wave;
+    const bool q_ok = (G.r0 + qr_l < G.TR) && (cw + qc_l < G.TC);
+    rlo = dlt_imax(qr_l, G.WR - G.r0);
+    rhi = dlt_imin(qr_l + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
+    const int clo = dlt_imax(qc_l, G.WC - cw), chi = dlt_imin(qc_l + 2 * G.WC, G.TC - 1 - cw + G.WC);
+#pragma unroll
+    for (int cg = 0; cg < NCGMAX; cg++) {
+#pragma unroll
+      for (int i = 0; i < 4; i++) cbias[cg][i] = (q_ok && 4 * cg + i >= clo && 4 * cg + i <= chi) ? 0.f : -INFINITY;
+      cg_edge[cg] = __builtin_amdgcn_ballot_w64(cbias[cg][0] != 0.f || cbias[cg][1] != 0.f || cbias[cg][2] != 0.f ||
+                                                cbias[cg][3] != 0.f) != 0;
+    }
+    wcol_lo = dlt_imax(0, G.WC - cw);
+    wcol_hi = G.TC - 1 - cw + G.WC;
+    wave_ok = cw < G.TC;
+    const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(P.HRP - 1, G.TR - 1 - G.r0 + G.WR);
+    ch_first = wrow_lo >> 3;
+    ch_last = wrow_hi >> 3;
+  }
+  DLT_DEV int64_t own_token(int row) const {
+    const int r = G.r0 + ((row & 15) >> 2), c = G.c0 + 4 * (row >> 4) + (row & 3);
+    return (r < G.TR && c < G.TC) ? (int64_t)r * G.TC + c : (int64_t)-1;
+  }
+  DLT_DEV bool block_on(const Swa1Plan& P, int cg) const {
+    return wave_ok && cg < P.ncg && 4 * cg <= wcol_hi && 4 * cg + 3 >= wcol_lo;
+  }
+};
+
+// accumulators (C layout, [dim][own token]) -> LDS tile [own token][dim] -> HBM rows
+template <typename TIO, int D, typename LaneT>
+DLT_DEV void swa1_write_grad(char* sT, f32x4 (&acc)[D / 16], float mul, TIO* base, int64_t sn, int64_t sd, int dact, bool vec,
+                             const LaneT& L, const RopeDev& rope, int wave, int n, int g, int tid) {
+  typedef typename TileOf<TIO>::type TL;
+  constexpr int PT = D * (int)sizeof(TL) + 16;
+  TL* row = reinterpret_cast<TL*>(sT + (16 * wave + n) * PT);
+#pragma unroll
+  for (int d = 0; d < D / 16; d++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) row[16 * d + 4 * g + i] = (TL)(acc[d][i] * mul);
+  __syncthreads();
+  store_tile<TIO, TL, D>(sT, PT, base, sn, sd, dact, vec, 64, [&](int r) { return L.own_token(r); }, rope, tid);
+  __syncthreads();
+}
+
+// =============================================================================================
+template <typename TIO, int D, int NCGMAX>
+__global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
+  typedef typename ComputeOf<TIO>::type CT;
+  extern __shared__ __align__(16) char smem[];
+  constexpr int PITCH = D * 2 + 16;
+  constexpr int KC = D / 32, DB = D / 16;
+  constexpr int HCW = swa1_hcw(NCGMAX);
+  constexpr int REGION = 8 * HCW * PITCH;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const Swa1Plan& P = a.plan;
+  char* sQ = smem;
+  char* sDO = smem + REGION;
+  float* sLse = reinterpret_cast<float*>(smem + 2 * REGION);
+  float* sDel = sLse + 8 * HCW;
+
+  Swa1Lane<NCGMAX> L;
+  L.init(a.p, P, wave, n);
+  const Swa1Geom& G = L.G;
+  const int b = L.b, h = L.h;
+
+  const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
+  const TIO* kb_ = reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1];
+  const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
+  const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
+  const float* lseb = a.lse + b * a.ls[0] + h * a.ls[1];
+  const float* delb = a.delta + b * a.ls[0] + h * a.ls[1];
+  RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
+  RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
+  RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
+  const bool use_rope = a.p.rope.enabled != 0;
+  const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
+  auto own_token = [&](int row) { return L.own_token(row); };
+
+  StageRegs<swa1_items(D, HCW)> srq, srd;
+  swa1_issue<TIO, D, HCW>(srq, qb, (int)a.qs[2], a.p.dk, G, 8 * L.ch_first, rope_idx, tid);
+  swa1_issue<TIO, D, HCW>(srd, dob, (int)a.dos[2], a.p.dv, G, 8 * L.ch_first, nullptr, tid);
+  ScalarRegs<HCW> r_lse, r_del;
+  swa1_issue_scalar<HCW>(r_lse, lseb, a.ls[2], G, 8 * L.ch_first, tid);
+  swa1_issue_scalar<HCW>(r_del, delb, a.ls[2], G, 8 * L.ch_first, tid);
+
+  // own keys / values -> B-operand fragments
+  stage_tile<TIO, CT, D>(sQ, PITCH, kb_, a.ks[2], a.ks[3], a.p.dk, a.k_vec != 0, 64, own_token, fwd_rope, tid);
+  stage_tile<TIO, CT, D>(sDO, PITCH, vb_, a.vs[2], a.vs[3], a.p.dv, a.v_vec != 0, 64, own_token, no_rope, tid);
+  __syncthreads();
+  u32x4 kf[KC], vf[KC];
+#pragma unroll
+  for (int c = 0; c < KC; c++) {
+    kf[c] = lds_read16(sQ + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
+    vf[c] = lds_read16(sDO + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
+  }
+  __syncthreads();
+
+  f32x4 dk_acc[DB], dv_acc[DB];
+#pragma unroll
+  for (int d = 0; d < DB; d++) { dk_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; dv_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+  const float scale = a.scale_log2;
+
+  swa1_commit<CT, D, HCW>(srq, sQ, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
+  swa1_commit<CT, D, HCW>(srd, sDO, PITCH, 1, no_rope, false, tid);
+  swa1_commit_scalar<HCW>(r_lse, sLse, tid);
+  swa1_commit_scalar<HCW>(r_del, sDel, tid);
+  __syncthreads();
+
+  for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
+    const int cr0 = 8 * ch;
+    if (ch < L.ch_last) {
+      swa1_issue<TIO, D, HCW>(srq, qb, (int)a.qs[2], a.p.dk, G, cr0 + 8, rope_idx, tid);
+      swa1_issue<TIO, D, HCW>(srd, dob, (int)a.dos[2], a.p.dv, G, cr0 + 8, nullptr, tid);
+      swa1_issue_scalar<HCW>(r_lse, lseb, a.ls[2], G, cr0 + 8, tid);
+      swa1_issue_scalar<HCW>(r_del, delb, a.ls[2], G, cr0 + 8, tid);
+    }
+    float rbias[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++) {
+      const int hrow = cr0 + 4 * mb + g;
+      rbias[mb] = (hrow >= L.rlo && hrow <= L.rhi) ? 0.f : -INFINITY;
+    }
+#pragma unroll
+    for (int cg = 0; cg < NCGMAX; cg++) {
+      if (!L.block_on(P, cg)) continue;
+      const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg + (n & 3);   // A-operand row of this lane
+      const int tok0 = g * HCW + 4 * wave + 4 * cg;                     // first of the 4 result columns
+      f32x4 s[2], dp[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+        s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+          s[mb] = Mma<CT>::mfma(lds_read16(sQ + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), kf[c], s[mb]);
+          dp[mb] = Mma<CT>::mfma(lds_read16(sDO + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), vf[c], dp[mb]);
+        }
+      }
+      float pr[8], ds[8];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+        const f32x4 lq = *reinterpret_cast<const f32x4*>(sLse + tok0 + 4 * mb * HCW);
+        const f32x4 dq_ = *reinterpret_cast<const f32x4*>(sDel + tok0 + 4 * mb * HCW);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const float nl = (L.cbias[cg][i] + rbias[mb]) - lq[i];
+          const float pv = fast_exp2(fmaf(s[mb][i], scale, nl));
+          pr[4 * mb + i] = pv;
+          ds[4 * mb + i] = pv * (dp[mb][i] - dq_[i]);
+        }
+      }
+      const u32x4 pb = pack8<CT>(pr), dsb = pack8<CT>(ds);
+      const int kt0 = 4 * wave + 4 * cg;
+#pragma unroll
+      for (int d = 0; d < DB; d++) {
+        dv_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sDO, PITCH, HCW, kt0, 16 * d, n, g), pb, dv_acc[d]);
+        dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PITCH, HCW, kt0, 16 * d, n, g), dsb, dk_acc[d]);
+      }
+    }
+    __syncthreads();
+    if (ch < L.ch_last) {
+      swa1_commit<CT, D, HCW>(srq, sQ, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
+      swa1_commit<CT, D, HCW>(srd, sDO, PITCH, 1, no_rope, false, tid);
+      swa1_commit_scalar<HCW>(r_lse, sLse, tid);
+  swa1_commit_scalar<HCW>(r_del, sDel, tid);
+      __syncthreads();
+    }
+  }
+
+  TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
+  TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
+  swa1_write_grad<TIO, D>(smem, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.dks[3], a.p.dk, a.dk_vec != 0, L, inv_rope, wave, n, g, tid);
+  swa1_write_grad<TIO, D>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.p.dv, a.dv_vec != 0, L, no_rope, wave, n, g, tid);
+}
+
+// =============================================================================================
+template <typename TIO, int D, int NCGMAX>
+__global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
+  typedef typename ComputeOf<TIO>::type CT;
+  extern __shared__ __align__(16) char smem[];
+  constexpr int PITCH = D * 2 + 16;
+  constexpr int KC = D / 32, DB = D / 16;
+  constexpr int HCW = swa1_hcw(NCGMAX);
+  constexpr int REGION = 8 * HCW * PITCH;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const Swa1Plan& P = a.plan;
+  char* sK = smem;
+  char* sV = smem + REGION;
+
+  Swa1Lane<NCGMAX> L;
+  L.init(a.p, P, wave, n);
+  const Swa1Geom& G = L.G;
+  const int b = L.b, h = L.h;
+
+  const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
+  const TIO* kb_ = reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1];
+  const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
+  const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
+  RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
+  RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
+  RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
+  const bool use_rope = a.p.rope.enabled != 0;
+  const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
+  auto own_token = [&](int row) { return L.own_token(row); };
+
+  StageRegs<swa1_items(D, HCW)> srk, srv;
+  swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, 8 * L.ch_first, rope_idx, tid);
+  swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, 8 * L.ch_first, nullptr, tid);
+
+  stage_tile<TIO, CT, D>(sK, PITCH, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, 64, own_token, fwd_rope, tid);
+  stage_tile<TIO, CT, D>(sV, PITCH, dob, a.dos[2], a.dos[3], a.p.dv, a.do_vec != 0, 64, own_token, no_rope, tid);
+  __syncthreads();
+  u32x4 qf[KC], dof[KC];
+#pragma unroll
+  for (int c = 0; c < KC; c++) {
+    qf[c] = lds_read16(sK + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
+    dof[c] = lds_read16(sV + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
+  }
+  const int64_t tq = L.own_token(16 * wave + n);
+  const int64_t loff = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
+  const float lse_n = tq >= 0 ? a.lse[loff] : 0.f;
+  const float del_n = tq >= 0 ? a.delta[loff] : 0.f;
+  __syncthreads();
+
+  f32x4 dq_acc[DB];
+#pragma unroll
+  for (int d = 0; d < DB; d++) dq_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float scale = a.scale_log2;
+
+  swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
+  swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, no_rope, false, tid);
+  __syncthreads();
+
+  for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
+    const int cr0 = 8 * ch;
+    if (ch < L.ch_last) {
+      swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, cr0 + 8, rope_idx, tid);
+      swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, cr0 + 8, nullptr, tid);
+    }
+    float rbias[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++) {
+      const int hrow = cr0 + 4 * mb + g;
+      rbias[mb] = ((hrow >= L.rlo && hrow <= L.rhi) ? 0.f : -INFINITY) - lse_n;
+    }
+#pragma unroll
+    for (int cg = 0; cg < NCGMAX; cg++) {
+      if (!L.block_on(P, cg)) continue;
+      const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg + (n & 3);
+      f32x4 s[2], dp[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+        s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+          s[mb] = Mma<CT>::mfma(lds_read16(sK + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), qf[c], s[mb]);
+          dp[mb] = Mma<CT>::mfma(lds_read16(sV + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), dof[c], dp[mb]);
+        }
+      }
+      float ds[8];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const float pv = fast_exp2(fmaf(s[mb][i], scale, L.cbias[cg][i] + rbias[mb]));
+          ds[4 * mb + i] = pv * (dp[mb][i] - del_n);
+        }
+      const u32x4 dsb = pack8<CT>(ds);
+      const int kt0 = 4 * wave + 4 * cg;
+#pragma unroll
+      for (int d = 0; d < DB; d++)
+        dq_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sK, PITCH, HCW, kt0, 16 * d, n, g), dsb, dq_acc[d]);
+    }
+    __syncthreads();
+    if (ch < L.ch_last) {
+      swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
+      swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, no_rope, false, tid);
+      __syncthreads();
+    }
+  }
+
+  TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
+  swa1_write_grad<TIO, D>(smem, dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.dqs[3], a.p.dk, a.dq_vec != 0, L, inv_rope, wave, n, g, tid);
+}

@@ -1,0 +1,216 @@
+// Forward kernel for token grids (b_size == 1, the shape of every SWA config of the benchmark).
+//
+// Replaces tiled_swa_fwd_kernel (src/tiled_swa.py:15-133), whose idea it generalises: a 2D
+// block of queries shares one K/V halo.  The halo is streamed through LDS in chunks of 8 rows
+// (K and V side by side); while a chunk is being consumed the next one is already in flight
+// from HBM into registers.  Per chunk a wave (one 4x4 query patch)
+//   1. computes S^T = K Q^T for its NCG blocks of 8x4 keys,
+//   2. scales and masks with additive per-column / per-row biases (the window test costs no
+//      compare in the inner loop) and runs ONE online-softmax update for the whole chunk,
+//   3. accumulates O^T += V^T P^T.
+#pragma once
+#include "swa1_common.hpp"
+
+struct Swa1FwdArgs {
+  AttnProblem p;
+  Swa1Plan plan;
+  const void *q, *k, *v;
+  void* o;
+  float* lse;
+  int64_t qs[4], ks[4], vs[4], os[4], ls[3];
+  int32_t q_vec, o_vec;
+  int32_t rope_pbit;  // chunk distance between rotary partners (R / 8), 1 without rotation
+  float scale_log2;
+};
+
+template <typename TIO, int D, int NCGMAX>
+__global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const Swa1FwdArgs a) {
+  typedef typename ComputeOf<TIO>::type CT;
+  extern __shared__ __align__(16) char smem[];
+  constexpr int PITCH = D * 2 + 16;
+  constexpr int KC = D / 32, VB = D / 16;
+  constexpr int HCW = swa1_hcw(NCGMAX);
+  constexpr int REGION = 8 * HCW * PITCH;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const Swa1Plan& P = a.plan;
+  char* sK = smem;
+  char* sV = smem + REGION;
+
+  const int lin = xcd_remap(blockIdx.x, gridDim.x);
+  const int per_bh = P.nblk_r * P.nblk_c;
+  const int bh = lin / per_bh;
+  const int rem = lin - bh * per_bh;
+  const int br = rem / P.nblk_c;
+  const int b = bh / a.p.H, h = bh - b * a.p.H;
+  Swa1Geom G;
+  G.r0 = 4 * br; G.c0 = 16 * (rem - br * P.nblk_c);
+  G.TR = a.p.g.TR; G.TC = a.p.g.TC; G.WR = a.p.g.WR; G.WC = a.p.g.WC;
+
+  const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
+  const TIO* kb_ = reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1];
+  const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
+  TIO* ob = reinterpret_cast<TIO*>(a.o) + b * a.os[0] + h * a.os[1];
+  RopeDev no_rope = a.p.rope;
+  no_rope.enabled = 0;
+  const bool use_rope = a.p.rope.enabled != 0;
+  const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
+
+  // own queries: LDS row 16 w + n <-> grid (r0 + (n >> 2), c0 + 4 w + (n & 3))
+  auto own_token = [&](int row) -> int64_t {
+    const int r = G.r0 + ((row & 15) >> 2), c = G.c0 + 4 * (row >> 4) + (row & 3);
+    return (r < G.TR && c < G.TC) ? (int64_t)r * G.TC + c : (int64_t)-1;
+  };
+
+  // halo rows that hold at least one grid row; chunks outside are skipped by the whole workgroup
+  const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(P.HRP - 1, G.TR - 1 - G.r0 + G.WR);
+  const int ch_first = wrow_lo >> 3, ch_last = wrow_hi >> 3;
+
+  StageRegs<swa1_items(D, HCW)> srk, srv;
+  swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, 8 * ch_first, rope_idx, tid);
+  swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, 8 * ch_first, nullptr, tid);
+
+  stage_tile<TIO, CT, D>(sK, PITCH, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, 64, own_token, a.p.rope, tid);
+  __syncthreads();
+  u32x4 qf[KC];
+#pragma unroll
+  for (int c = 0; c < KC; c++) qf[c] = lds_read16(sK + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
+  __syncthreads();
+
+  // ---- window of this lane's query in halo coordinates -> additive biases
+  const int qr_l = n >> 2, qc_l = n & 3;
+  const int cw = G.c0 + 4 * wave;
+  const bool q_ok = (G.r0 + qr_l < G.TR) && (cw + qc_l < G.TC);
+  const int rlo = dlt_imax(qr_l, G.WR - G.r0), rhi = dlt_imin(qr_l + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
+  const int clo = dlt_imax(qc_l, G.WC - cw), chi = dlt_imin(qc_l + 2 * G.WC, G.TC - 1 - cw + G.WC);
+  float cbias[NCGMAX][4];
+#pragma unroll
+  for (int cg = 0; cg < NCGMAX; cg++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) cbias[cg][i] = (q_ok && 4 * cg + i >= clo && 4 * cg + i <= chi) ? 0.f : -INFINITY;
+  // window columns of this wave that hold at least one grid column
+  const int wcol_lo = dlt_imax(0, G.WC - cw), wcol_hi = G.TC - 1 - cw + G.WC;
+  const bool wave_ok = cw < G.TC;
+
+  // which column groups need the per-element bias at all (wave-uniform)
+  bool cg_edge[NCGMAX];
+#pragma unroll
+  for (int cg = 0; cg < NCGMAX; cg++)
+    cg_edge[cg] = __builtin_amdgcn_ballot_w64(cbias[cg][0] != 0.f || cbias[cg][1] != 0.f || cbias[cg][2] != 0.f ||
+                                              cbias[cg][3] != 0.f) != 0;
+
+  // running max of the RAW scores (sm_scale > 0 keeps the order), sum in acc_l through an
+  // extra MFMA whose A operand is a row of ones: row 0 of the result is sum_k P[k][query]
+  float m_run = -INFINITY;
+  f32x4 acc[VB], acc_l = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int d = 0; d < VB; d++) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float scale = a.scale_log2;
+  const unsigned one2 = pack2<CT>(1.f, 1.f);
+  const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
+
+  swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, a.p.rope, use_rope, tid);
+  swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, a.p.rope, false, tid);
+  __syncthreads();
+
+  for (int ch = ch_first; ch <= ch_last; ch++) {
+    const int cr0 = 8 * ch;
+    if (ch < ch_last) {  // next chunk: HBM -> registers while this one is consumed
+      swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, cr0 + 8, rope_idx, tid);
+      swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, cr0 + 8, nullptr, tid);
+    }
+
+    float t[NCGMAX][8];
+    float mloc = -INFINITY;
+    float rbias[2];
+#pragma unroll
+    for (int mb = 0; mb < 2; mb++) {
+      const int hrow = cr0 + 4 * mb + g;
+      rbias[mb] = (hrow >= rlo && hrow <= rhi) ? 0.f : -INFINITY;
+    }
+    const bool row_edge = __builtin_amdgcn_ballot_w64(rbias[0] != 0.f || rbias[1] != 0.f) != 0;
+#pragma unroll
+    for (int cg = 0; cg < NCGMAX; cg++) {
+      const bool on = wave_ok && cg < P.ncg && 4 * cg <= wcol_hi && 4 * cg + 3 >= wcol_lo;
+      if (on) {
+        const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg + (n & 3);
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; c++) {
+          const u32x4 k0 = lds_read16(sK + key0 * PITCH + (32 * c + 8 * g) * 2);
+          const u32x4 k1 = lds_read16(sK + (key0 + 4 * HCW) * PITCH + (32 * c + 8 * g) * 2);
+          s0 = Mma<CT>::mfma(k0, qf[c], s0);
+          s1 = Mma<CT>::mfma(k1, qf[c], s1);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) { t[cg][i] = s0[i]; t[cg][4 + i] = s1[i]; }
+        if (cg_edge[cg]) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) { t[cg][i] += cbias[cg][i]; t[cg][4 + i] += cbias[cg][i]; }
+        }
+        if (row_edge) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) { t[cg][i] += rbias[0]; t[cg][4 + i] += rbias[1]; }
+        }
+        mloc = fmaxf(mloc, fmaxf(fmaxf(fmaxf(t[cg][0], t[cg][1]), fmaxf(t[cg][2], t[cg][3])),
+                                 fmaxf(fmaxf(t[cg][4], t[cg][5]), fmaxf(t[cg][6], t[cg][7]))));
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) t[cg][i] = -INFINITY;
+      }
+    }
+    // one online-softmax update per chunk: p = exp2(s * scale - m * scale)
+    mloc = wave_max4(mloc);
+    const float m_new = fmaxf(m_run, mloc);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = fast_exp2((m_run - m_use) * scale);
+    const float neg_m2 = -m_use * scale;
+    m_run = m_new;
+    u32x4 pb[NCGMAX];
+#pragma unroll
+    for (int cg = 0; cg < NCGMAX; cg++) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) t[cg][i] = fast_exp2(fmaf(t[cg][i], scale, neg_m2));
+      pb[cg] = pack8<CT>(t[cg]);
+    }
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+#pragma unroll
+      for (int d = 0; d < VB; d++) acc[d] *= alpha;
+      acc_l *= alpha;
+    }
+#pragma unroll
+    for (int cg = 0; cg < NCGMAX; cg++) {
+      const bool on = wave_ok && cg < P.ncg && 4 * cg <= wcol_hi && 4 * cg + 3 >= wcol_lo;
+      if (on) {
+        const int key0 = 4 * wave + 4 * cg;
+#pragma unroll
+        for (int d = 0; d < VB; d++)
+          acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PITCH, HCW, key0, 16 * d, n, g), pb[cg], acc[d]);
+        acc_l = Mma<CT>::mfma(ones, pb[cg], acc_l);
+      }
+    }
+    __syncthreads();  // every wave is done with this chunk
+    if (ch < ch_last) {
+      swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, a.p.rope, use_rope, tid);
+      swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, a.p.rope, false, tid);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue
+  typedef typename TileOf<TIO>::type TL;
+  constexpr int PO = D * (int)sizeof(TL) + 16;
+  const float lt = __shfl(acc_l[0], n);  // row 0 of the ones product lives in lane group 0
+  const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
+  TL* orow = reinterpret_cast<TL*>(smem + (16 * wave + n) * PO);
+#pragma unroll
+  for (int d = 0; d < VB; d++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[d][i] * inv);
+  const int64_t tq = own_token(16 * wave + n);
+  if (g == 0 && tq >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq * a.ls[2]] = m_run * scale + fast_log2(lt);
+  __syncthreads();
+  store_tile<TIO, TL, D>(smem, PO, ob, a.os[2], a.os[3], a.p.dv, a.o_vec != 0, 64, own_token, no_rope, tid);
+}
