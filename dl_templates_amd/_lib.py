@@ -25,7 +25,7 @@ _DTYPES = {torch.bfloat16: DLT_BF16, torch.float16: DLT_FP16, torch.float32: DLT
 EXPORTS = (
     "dlt_last_error", "dlt_version", "dlt_rope2d", "dlt_rope2d_pair", "dlt_rope_pe_mask",
     "dlt_swa_fwd", "dlt_swa_bwd", "dlt_swa_neighbors", "dlt_flash_fwd", "dlt_flash_bwd",
-    "dlt_timing_enable", "dlt_timing_collect",
+    "dlt_timing_enable", "dlt_timing_collect", "dlt_debug_copy",
 )
 KERNEL_NAMES = ("rope2d", "attn_fwd", "attn_delta", "attn_bwd_kv", "attn_bwd_q")
 
@@ -105,6 +105,8 @@ def _declare(lib) -> None:
     lib.dlt_flash_fwd.argtypes = fwd + [POINTER(FlashShape), c_void_p]
     lib.dlt_flash_bwd.restype = c_int
     lib.dlt_flash_bwd.argtypes = bwd + [POINTER(FlashShape), c_void_p]
+    lib.dlt_debug_copy.restype = c_int
+    lib.dlt_debug_copy.argtypes = [c_void_p, c_void_p, c_int64, c_void_p]
     lib.dlt_timing_enable.restype = c_int
     lib.dlt_timing_enable.argtypes = [c_int]
     lib.dlt_timing_collect.restype = c_int

@@ -174,6 +174,29 @@ int fill_bwd(const char* who, AttnTensors& t, const void* q, const int64_t* qs, 
 
 }  // namespace
 
+namespace {
+__global__ __launch_bounds__(256) void debug_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, int64_t n) {
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (; i < n; i += stride) dst[i] = src[i];
+}
+
+}  // namespace
+
+extern "C" int dlt_debug_copy(void* dst, const void* src, int64_t bytes, void* stream) {
+  DLT_REQUIRE(bytes >= 0 && bytes % 16 == 0, "debug_copy: size must be a multiple of 16");
+  DLT_REQUIRE(((uintptr_t)dst | (uintptr_t)src) % 16 == 0, "debug_copy: pointers must be 16-byte aligned");
+  if (bytes == 0) return DLT_OK;
+  DLT_REQUIRE(dst != nullptr && src != nullptr, "debug_copy: NULL pointer");
+  const int64_t n = bytes / 16;
+  int64_t blocks = (n + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(debug_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     reinterpret_cast<const uint4*>(src), reinterpret_cast<uint4*>(dst), n);
+  DLT_CHECK_LAUNCH("debug_copy launch");
+  return DLT_OK;
+}
+
 extern "C" int dlt_swa_neighbors(int32_t t_height, int32_t t_width, int32_t row_size, int32_t col_size,
                                  uint8_t* mask, void* stream) {
   DLT_REQUIRE(t_height > 0 && t_width > 0 && row_size >= 0 && col_size >= 0, "swa_neighbors: bad grid/window");

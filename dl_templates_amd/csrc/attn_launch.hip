@@ -86,6 +86,7 @@ struct Swa1Class { int D, wclass, pbit; };
 bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streamed, Swa1Class& c) {
   if (p.g.mode != DLT_GEOM_SWA || p.g.S != 1) return false;
   if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
+  if (p.dk % 32 != 0 || p.dv % 32 != 0) return false;  // 64-byte staging pieces
   if (p.dk <= 64 && p.dv <= 64) c.D = 64;
   else if (p.dk <= 128 && p.dv <= 128 && p.dk > 64 && p.dv > 64) c.D = 128;
   else return false;

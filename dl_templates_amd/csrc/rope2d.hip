@@ -10,6 +10,7 @@
 // keeps its 8 (cos, sin) pairs in registers while it walks over the batch rows, so the
 // table is read once per thread and the x traffic is 16-byte vector loads/stores.
 #include "dlt_internal.hpp"
+#include <stdlib.h>
 
 namespace {
 
@@ -53,9 +54,25 @@ __global__ __launch_bounds__(256) void rope2d_vec_kernel(RopeKArgs a) {
   const int pc = (int)(gid - n * items);
   const int ax = pc / cpa, ci = pc - ax * cpa;
 
+  // The x loads do not depend on idx: they are issued first so that the idx -> table chain and
+  // the first batch of data travel together (tokens with an unrotated axis cost a read only).
   const int32_t id = a.r.idx[n];
+  const int d0 = ax * 2 * a.r.R + 8 * ci, d1 = d0 + a.r.R;
+  T* xb = reinterpret_cast<T*>(a.x[z]) + n * a.s[z][1];
+  const int64_t sb = a.s[z][0];
+  const int b_begin = blockIdx.y * a.bb;
+  const int b_end = dlt_imin(b_begin + a.bb, a.nb[z]);
+  Vec8<T> v0[UNR], v1[UNR];
+#pragma unroll
+  for (int u = 0; u < UNR; u++) {
+    if (b_begin + u < b_end) {
+      T* px = xb + (int64_t)(b_begin + u) * sb;
+      v0[u] = *reinterpret_cast<const Vec8<T>*>(px + d0);
+      v1[u] = *reinterpret_cast<const Vec8<T>*>(px + d1);
+    }
+  }
   int p = ax == 0 ? dlt_rope_row(id) : dlt_rope_col(id);
-  if (p < 0) return;  // this axis is not rotated for this token: no traffic at all
+  if (p < 0) return;  // this axis is not rotated for this token: nothing is written
   p = dlt_imin(p, (ax == 0 ? a.r.row_len : a.r.col_len) - 1);
   const float* tab = (ax == 0 ? a.r.row_cs + (int64_t)p * a.r.rs0 : a.r.col_cs + (int64_t)p * a.r.cs0) + 16 * ci;
   float cs[16];
@@ -68,19 +85,15 @@ __global__ __launch_bounds__(256) void rope2d_vec_kernel(RopeKArgs a) {
 #pragma unroll
     for (int j = 0; j < 8; j++) cs[2 * j + 1] = -cs[2 * j + 1];
   }
-  const int d0 = ax * 2 * a.r.R + 8 * ci, d1 = d0 + a.r.R;
-  T* xb = reinterpret_cast<T*>(a.x[z]) + n * a.s[z][1];
-  const int64_t sb = a.s[z][0];
-  const int b_begin = blockIdx.y * a.bb;
-  const int b_end = dlt_imin(b_begin + a.bb, a.nb[z]);
   for (int b0 = b_begin; b0 < b_end; b0 += UNR) {
-    Vec8<T> v0[UNR], v1[UNR];
+    if (b0 != b_begin) {
 #pragma unroll
-    for (int u = 0; u < UNR; u++) {
-      if (b0 + u < b_end) {
-        T* px = xb + (int64_t)(b0 + u) * sb;
-        v0[u] = *reinterpret_cast<const Vec8<T>*>(px + d0);
-        v1[u] = *reinterpret_cast<const Vec8<T>*>(px + d1);
+      for (int u = 0; u < UNR; u++) {
+        if (b0 + u < b_end) {
+          T* px = xb + (int64_t)(b0 + u) * sb;
+          v0[u] = *reinterpret_cast<const Vec8<T>*>(px + d0);
+          v1[u] = *reinterpret_cast<const Vec8<T>*>(px + d1);
+        }
       }
     }
 #pragma unroll
@@ -189,6 +202,7 @@ int rope_impl(void* const x[2], const int64_t* const st[2], const int64_t nb[2],
   int bb = (int)maxb;
   while (bb > UNR && bx * ((maxb + bb - 1) / bb) * ntens < 2048) bb = (bb + 1) / 2;
   a.bb = bb < 1 ? 1 : bb;
+  if (const char* e = getenv("DLT_ROPE_BB")) { const int v = atoi(e); if (v > 0) a.bb = v; }
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case DLT_BF16: return launch_rope<bf16_t>(a, vec, s, ntens);

@@ -35,9 +35,11 @@ DLT_DEV void swa1_issue_scalar(ScalarRegs<HCW>& sr, const float* base, int64_t s
     const int idx = tid + 256 * it;
     sr.v[it] = 0.f;
     if (idx < 8 * HCW) {
+      // clamped like the tile staging: out-of-grid halo positions are masked by the window bias
       const int hr = idx / HCW, hc = idx - hr * HCW;
-      const int r = G.r0 - G.WR + cr0 + hr, c = G.c0 - G.WC + hc;
-      if ((unsigned)r < (unsigned)G.TR && (unsigned)c < (unsigned)G.TC) sr.v[it] = base[(int64_t)(r * G.TC + c) * stride];
+      const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + cr0 + hr, G.TR - 1));
+      const int c = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));
+      sr.v[it] = base[(int64_t)(r * G.TC + c) * stride];
     }
   }
 }
@@ -155,32 +157,35 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  StageRegs<swa1_items(D, HCW)> srq, srd;
-  swa1_issue<TIO, D, HCW>(srq, qb, (int)a.qs[2], a.p.dk, G, 8 * L.ch_first, rope_idx, tid);
-  swa1_issue<TIO, D, HCW>(srd, dob, (int)a.dos[2], a.p.dv, G, 8 * L.ch_first, nullptr, tid);
+  constexpr int NI = swa1_items(D, HCW);
+  StagePlan<NI> sp;
+  swa1_plan_init<D, HCW>(sp, G, PITCH, tid);
+  const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
+  const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
+  StageRegs<NI> srq, srd;
+  swa1_regs_zero(srq);
+  swa1_regs_zero(srd);
+  swa1_issue(srq, sp, on_k, qb, sn2q, G, 8 * L.ch_first, rope_idx);
+  swa1_issue(srd, sp, on_v, dob, sn2d, G, 8 * L.ch_first, nullptr);
   ScalarRegs<HCW> r_lse, r_del;
   swa1_issue_scalar<HCW>(r_lse, lseb, a.ls[2], G, 8 * L.ch_first, tid);
   swa1_issue_scalar<HCW>(r_del, delb, a.ls[2], G, 8 * L.ch_first, tid);
 
-  // own keys / values -> B-operand fragments
-  stage_tile<TIO, CT, D>(sQ, PITCH, kb_, a.ks[2], a.ks[3], a.p.dk, a.k_vec != 0, 64, own_token, fwd_rope, tid);
-  stage_tile<TIO, CT, D>(sDO, PITCH, vb_, a.vs[2], a.vs[3], a.p.dv, a.v_vec != 0, 64, own_token, no_rope, tid);
-  __syncthreads();
+  // own keys / values straight into B-operand fragments
   u32x4 kf[KC], vf[KC];
-#pragma unroll
-  for (int c = 0; c < KC; c++) {
-    kf[c] = lds_read16(sQ + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
-    vf[c] = lds_read16(sDO + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
+  {
+    const int64_t tk = L.own_token(16 * wave + n);
+    swa1_load_own<TIO, CT, D>(kf, kb_, a.ks[2], a.p.dk, tk, g, fwd_rope, use_rope);
+    swa1_load_own<TIO, CT, D>(vf, vb_, a.vs[2], a.p.dv, tk, g, no_rope, false);
   }
-  __syncthreads();
 
   f32x4 dk_acc[DB], dv_acc[DB];
 #pragma unroll
   for (int d = 0; d < DB; d++) { dk_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; dv_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
   const float scale = a.scale_log2;
 
-  swa1_commit<CT, D, HCW>(srq, sQ, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
-  swa1_commit<CT, D, HCW>(srd, sDO, PITCH, 1, no_rope, false, tid);
+  swa1_commit<CT>(srq, sp, sQ, a.rope_pbit, fwd_rope, use_rope && on_k);
+  swa1_commit<CT>(srd, sp, sDO, 1, no_rope, false);
   swa1_commit_scalar<HCW>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW>(r_del, sDel, tid);
   __syncthreads();
@@ -188,8 +193,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
   for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
     const int cr0 = 8 * ch;
     if (ch < L.ch_last) {
-      swa1_issue<TIO, D, HCW>(srq, qb, (int)a.qs[2], a.p.dk, G, cr0 + 8, rope_idx, tid);
-      swa1_issue<TIO, D, HCW>(srd, dob, (int)a.dos[2], a.p.dv, G, cr0 + 8, nullptr, tid);
+      swa1_issue(srq, sp, on_k, qb, sn2q, G, cr0 + 8, rope_idx);
+      swa1_issue(srd, sp, on_v, dob, sn2d, G, cr0 + 8, nullptr);
       swa1_issue_scalar<HCW>(r_lse, lseb, a.ls[2], G, cr0 + 8, tid);
       swa1_issue_scalar<HCW>(r_del, delb, a.ls[2], G, cr0 + 8, tid);
     }
@@ -238,8 +243,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
     }
     __syncthreads();
     if (ch < L.ch_last) {
-      swa1_commit<CT, D, HCW>(srq, sQ, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
-      swa1_commit<CT, D, HCW>(srd, sDO, PITCH, 1, no_rope, false, tid);
+      swa1_commit<CT>(srq, sp, sQ, a.rope_pbit, fwd_rope, use_rope && on_k);
+      swa1_commit<CT>(srd, sp, sDO, 1, no_rope, false);
       swa1_commit_scalar<HCW>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW>(r_del, sDel, tid);
       __syncthreads();
@@ -285,39 +290,40 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(cons
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  StageRegs<swa1_items(D, HCW)> srk, srv;
-  swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, 8 * L.ch_first, rope_idx, tid);
-  swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, 8 * L.ch_first, nullptr, tid);
+  constexpr int NI = swa1_items(D, HCW);
+  StagePlan<NI> sp;
+  swa1_plan_init<D, HCW>(sp, G, PITCH, tid);
+  const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
+  const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
+  StageRegs<NI> srk, srv;
+  swa1_regs_zero(srk);
+  swa1_regs_zero(srv);
+  swa1_issue(srk, sp, on_k, kb_, sn2k, G, 8 * L.ch_first, rope_idx);
+  swa1_issue(srv, sp, on_v, vb_, sn2v, G, 8 * L.ch_first, nullptr);
 
-  stage_tile<TIO, CT, D>(sK, PITCH, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, 64, own_token, fwd_rope, tid);
-  stage_tile<TIO, CT, D>(sV, PITCH, dob, a.dos[2], a.dos[3], a.p.dv, a.do_vec != 0, 64, own_token, no_rope, tid);
-  __syncthreads();
+  // own queries / output gradients straight into B-operand fragments
   u32x4 qf[KC], dof[KC];
-#pragma unroll
-  for (int c = 0; c < KC; c++) {
-    qf[c] = lds_read16(sK + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
-    dof[c] = lds_read16(sV + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
-  }
   const int64_t tq = L.own_token(16 * wave + n);
+  swa1_load_own<TIO, CT, D>(qf, qb, a.qs[2], a.p.dk, tq, g, fwd_rope, use_rope);
+  swa1_load_own<TIO, CT, D>(dof, dob, a.dos[2], a.p.dv, tq, g, no_rope, false);
   const int64_t loff = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
   const float lse_n = tq >= 0 ? a.lse[loff] : 0.f;
   const float del_n = tq >= 0 ? a.delta[loff] : 0.f;
-  __syncthreads();
 
   f32x4 dq_acc[DB];
 #pragma unroll
   for (int d = 0; d < DB; d++) dq_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float scale = a.scale_log2;
 
-  swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
-  swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, no_rope, false, tid);
+  swa1_commit<CT>(srk, sp, sK, a.rope_pbit, fwd_rope, use_rope && on_k);
+  swa1_commit<CT>(srv, sp, sV, 1, no_rope, false);
   __syncthreads();
 
   for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
     const int cr0 = 8 * ch;
     if (ch < L.ch_last) {
-      swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, cr0 + 8, rope_idx, tid);
-      swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, cr0 + 8, nullptr, tid);
+      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + 8, rope_idx);
+      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + 8, nullptr);
     }
     float rbias[2];
 #pragma unroll
@@ -356,8 +362,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(cons
     }
     __syncthreads();
     if (ch < L.ch_last) {
-      swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, fwd_rope, use_rope, tid);
-      swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, no_rope, false, tid);
+      swa1_commit<CT>(srk, sp, sK, a.rope_pbit, fwd_rope, use_rope && on_k);
+      swa1_commit<CT>(srv, sp, sV, 1, no_rope, false);
       __syncthreads();
     }
   }

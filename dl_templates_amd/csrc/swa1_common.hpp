@@ -25,100 +25,152 @@ constexpr int swa1_hcw(int ncgmax) { return 12 + 4 * ncgmax; }
 // 64-byte items (4 chunks of 8 dims of one token) a thread stages per 8-row chunk of one tensor
 constexpr int swa1_items(int d, int hcw) { return (8 * hcw * (d / 32) + 255) / 256; }
 
-// One thread's share of a halo chunk in flight between HBM and LDS.  An item is 64 contiguous
-// bytes of one token; rotary partners (8 or 16 dims apart) live in the same item, so the
-// rotation needs no second load.
-template <int NI>
-struct StageRegs {
-  u32x4 v[NI][4];
-  int32_t id[NI];  // packed rotary index of the token (-1: no rotation / outside the grid)
-};
-
 struct Swa1Geom {
   int r0, c0;      // first grid row / column of the workgroup's band
   int TR, TC, WR, WC;
 };
 
-// Issue the global loads of halo rows [cr0, cr0 + 8) into registers (zeros outside the grid).
-// Offsets are 32-bit element offsets from `base` (the host checks that a [N, D] slab fits).
-template <typename TIO, int D, int HCW>
-DLT_DEV void swa1_issue(StageRegs<swa1_items(D, HCW)>& sr, const TIO* base, int sn, int dact, const Swa1Geom& G,
-                        int cr0, const int32_t* rope_idx, int tid) {
+// Chunk-invariant part of a thread's staging work.  Item `it` of a thread is the 64-byte piece
+// `qd` of halo token (hr[it], column cc[it]); halo positions outside the grid are CLAMPED onto
+// the nearest grid token instead of being zero-filled: such positions are always masked by the
+// -inf window bias, so their (finite) values never reach a result, and the loads need neither
+// a branch nor a zero fill.
+template <int NI>
+struct StagePlan {
+  int hr[NI];    // halo row inside the chunk (0..7)
+  int cc[NI];    // grid column, clamped
+  int loff[NI];  // byte offset inside the LDS chunk, -1: no such item
+  int qoff;      // byte offset of the thread's 64-byte piece inside a token row
+};
+
+template <int D, int HCW>
+DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW)>& sp, const Swa1Geom& G, int pitch, int tid) {
   constexpr int QUADS = D / 32;
-  constexpr int TOTAL = 8 * HCW * QUADS;
-  const int rbase = G.r0 - G.WR + cr0, cbase = G.c0 - G.WC;
+  const int qd = tid % QUADS, key0 = tid / QUADS;
 #pragma unroll
   for (int it = 0; it < swa1_items(D, HCW); it++) {
-    const int idx = tid + 256 * it;
+    const int key = key0 + it * (256 / QUADS);
+    const bool live = key < 8 * HCW;
+    const int k = live ? key : 0;
+    const int hr = k / HCW, hc = k - hr * HCW;
+    sp.hr[it] = hr;
+    sp.cc[it] = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));
+    sp.loff[it] = live ? k * pitch + 64 * qd : -1;
+  }
+  sp.qoff = 64 * qd;
+}
+
+// One thread's share of a halo chunk in flight between HBM and LDS (rotary partners, 8 or 16
+// dims apart, live in the same 64-byte item, so the rotation needs no second load).
+template <int NI>
+struct StageRegs {
+  u32x4 v[NI][4];
+  int32_t id[NI];  // packed rotary index of the token
+};
+
+template <int NI>
+DLT_DEV void swa1_regs_zero(StageRegs<NI>& sr) {
+#pragma unroll
+  for (int it = 0; it < NI; it++) {
 #pragma unroll
     for (int j = 0; j < 4; j++) sr.v[it][j] = u32x4{0u, 0u, 0u, 0u};
     sr.id[it] = -1;
-    if (TOTAL % 256 == 0 || it + 1 < swa1_items(D, HCW) || idx < TOTAL) {
-      const int key = idx / QUADS, qd = idx % QUADS;
-      const int hr = key / HCW, hc = key - hr * HCW;
-      const int r = rbase + hr, c = cbase + hc;
-      if ((unsigned)r < (unsigned)G.TR && (unsigned)c < (unsigned)G.TC) {
-        const int tok = r * G.TC + c;
-        const TIO* p = base + (tok * sn + 32 * qd);
+  }
+}
+
+// Issue the global loads of halo rows [cr0, cr0 + 8) into registers.  `sn2` is the token stride
+// in BYTES; offsets are 32-bit (the host checks that a [N, D] slab stays below 2 GiB).  `on`:
+// the thread's 64-byte piece lies below the actual head dim (pieces above it stay zero).
+template <int NI>
+DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, const void* base, int sn2, const Swa1Geom& G,
+                        int cr0, const int32_t* rope_idx) {
+  const int rbase = G.r0 - G.WR + cr0;
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-          if (32 * qd + 8 * j < dact) sr.v[it][j] = *reinterpret_cast<const u32x4*>(p + 8 * j);
-        if (rope_idx != nullptr) sr.id[it] = rope_idx[tok];
-      }
+  for (int it = 0; it < NI; it++) {
+    const int r = dlt_imax(0, dlt_imin(rbase + sp.hr[it], G.TR - 1));
+    const int tok = r * G.TC + sp.cc[it];
+    if (on) {
+      const char* p = reinterpret_cast<const char*>(base) + (uint32_t)(tok * sn2 + sp.qoff);
+#pragma unroll
+      for (int j = 0; j < 4; j++) sr.v[it][j] = *reinterpret_cast<const u32x4*>(p + 16 * j);
     }
+    if (rope_idx != nullptr) sr.id[it] = rope_idx[tok];
   }
 }
 
 // Rotate (K / Q side only) and write the staged registers into an LDS chunk.
 // pbit: chunk distance between rotary partners (1 or 2).
-template <typename CT, int D, int HCW>
-DLT_DEV void swa1_commit(StageRegs<swa1_items(D, HCW)>& sr, char* s, int pitch, int pbit, const RopeDev& rope,
-                         bool use_rope, int tid) {
-  constexpr int QUADS = D / 32;
-  constexpr int TOTAL = 8 * HCW * QUADS;
+template <typename CT, int NI>
+DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, int pbit, const RopeDev& rope, bool use_rope) {
 #pragma unroll
-  for (int it = 0; it < swa1_items(D, HCW); it++) {
-    const int idx = tid + 256 * it;
-    if (TOTAL % 256 == 0 || it + 1 < swa1_items(D, HCW) || idx < TOTAL) {
-      const int key = idx / QUADS, qd = idx % QUADS;
-      if (use_rope && sr.id[it] != -1 && 32 * qd < 4 * rope.R) {
-        const int r8 = rope.R >> 3;
+  for (int it = 0; it < NI; it++) {
+    if (sp.loff[it] < 0) continue;
+    if (use_rope && sp.qoff < 8 * rope.R) {
+      const int r8 = rope.R >> 3;
+      const int qd4 = sp.qoff >> 4;  // first chunk of this piece
 #pragma unroll
-        for (int pr = 0; pr < 2; pr++) {
-          // pbit 1: pairs (0,1), (2,3); pbit 2: pairs (0,2), (1,3)
-          const int ja = pbit == 1 ? 2 * pr : pr, jb = ja + pbit;
-          const int c0 = 4 * qd + ja;
-          if (8 * c0 < 4 * rope.R) {
-            const int region = c0 / r8, ci = c0 - region * r8;
-            bool rotated;
-            const float* tab = rope_table_row(rope, region >> 1, sr.id[it], rotated) + 16 * ci;
-            if (rotated) {
-              u32x4 lo = pbit == 1 ? (pr == 0 ? sr.v[it][0] : sr.v[it][2]) : (pr == 0 ? sr.v[it][0] : sr.v[it][1]);
-              u32x4 hi = pbit == 1 ? (pr == 0 ? sr.v[it][1] : sr.v[it][3]) : (pr == 0 ? sr.v[it][2] : sr.v[it][3]);
-              float x0[8], x1[8];
-              unpack8<CT>(lo, x0);
-              unpack8<CT>(hi, x1);
+      for (int pr = 0; pr < 2; pr++) {
+        // pbit 1: pairs (0,1), (2,3); pbit 2: pairs (0,2), (1,3)
+        const int ja = pbit == 1 ? 2 * pr : pr;
+        const int c0 = qd4 + ja;
+        if (8 * c0 < 4 * rope.R) {
+          const int region = c0 / r8, ci = c0 - region * r8;
+          bool rotated;
+          const float* tab = rope_table_row(rope, region >> 1, sr.id[it], rotated) + 16 * ci;
+          if (rotated) {
+            u32x4 lo = pbit == 1 ? (pr == 0 ? sr.v[it][0] : sr.v[it][2]) : (pr == 0 ? sr.v[it][0] : sr.v[it][1]);
+            u32x4 hi = pbit == 1 ? (pr == 0 ? sr.v[it][1] : sr.v[it][3]) : (pr == 0 ? sr.v[it][2] : sr.v[it][3]);
+            float x0[8], x1[8];
+            unpack8<CT>(lo, x0);
+            unpack8<CT>(hi, x1);
 #pragma unroll
-              for (int j = 0; j < 8; j++) {
-                const float cs = tab[2 * j], sn = tab[2 * j + 1];
-                const float y0 = rope_mix(x0[j], x1[j], cs, sn, true);
-                const float y1 = rope_mix(x1[j], x0[j], cs, sn, false);
-                x0[j] = y0; x1[j] = y1;
-              }
-              lo = pack8<CT>(x0);
-              hi = pack8<CT>(x1);
-              if (pbit == 1) {
-                if (pr == 0) { sr.v[it][0] = lo; sr.v[it][1] = hi; } else { sr.v[it][2] = lo; sr.v[it][3] = hi; }
-              } else {
-                if (pr == 0) { sr.v[it][0] = lo; sr.v[it][2] = hi; } else { sr.v[it][1] = lo; sr.v[it][3] = hi; }
-              }
+            for (int j = 0; j < 8; j++) {
+              const float cs = tab[2 * j], sn = tab[2 * j + 1];
+              const float y0 = rope_mix(x0[j], x1[j], cs, sn, true);
+              const float y1 = rope_mix(x1[j], x0[j], cs, sn, false);
+              x0[j] = y0; x1[j] = y1;
+            }
+            lo = pack8<CT>(x0);
+            hi = pack8<CT>(x1);
+            if (pbit == 1) {
+              if (pr == 0) { sr.v[it][0] = lo; sr.v[it][1] = hi; } else { sr.v[it][2] = lo; sr.v[it][3] = hi; }
+            } else {
+              if (pr == 0) { sr.v[it][0] = lo; sr.v[it][2] = hi; } else { sr.v[it][1] = lo; sr.v[it][3] = hi; }
             }
           }
         }
       }
-      char* row = s + key * pitch + 64 * qd;
+    }
+    char* row = s + sp.loff[it];
 #pragma unroll
-      for (int j = 0; j < 4; j++) lds_write16(row + 16 * j, sr.v[it][j]);
+    for (int j = 0; j < 4; j++) lds_write16(row + 16 * j, sr.v[it][j]);
+  }
+}
+
+// B-operand fragments of one OWN token (head dim along k) straight from HBM: lane group g
+// holds dims 32c + 8g .. +7 of chunk c.  Rotated on the way in when `use_rope`.
+template <typename TIO, typename CT, int D>
+DLT_DEV void swa1_load_own(u32x4 (&f)[D / 32], const TIO* base, int64_t sn, int dact, int64_t tok, int g,
+                           const RopeDev& rope, bool use_rope) {
+#pragma unroll
+  for (int c = 0; c < D / 32; c++) {
+    const int ch = 4 * c + g;
+    f[c] = u32x4{0u, 0u, 0u, 0u};
+    if (tok >= 0 && 8 * ch < dact) f[c] = *reinterpret_cast<const u32x4*>(base + tok * sn + 8 * ch);
+  }
+  if (use_rope && tok >= 0) {
+    const int32_t id = rope.idx[tok];
+#pragma unroll
+    for (int c = 0; c < D / 32; c++) {
+      const int ch = 4 * c + g;
+      const RopeChunk rc = rope_chunk_setup(rope, ch, true);
+      if (rc.mode == 1) {
+        float self[8], partner[8];
+        unpack8<CT>(f[c], self);
+        unpack8<CT>(*reinterpret_cast<const u32x4*>(base + tok * sn + 8 * rc.partner_c), partner);
+        rope_apply8(rope, rc, ch, id, self, partner, [](int) { return 0.f; });
+        f[c] = pack8<CT>(self);
+      }
     }
   }
 }

@@ -68,16 +68,20 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const 
   const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(P.HRP - 1, G.TR - 1 - G.r0 + G.WR);
   const int ch_first = wrow_lo >> 3, ch_last = wrow_hi >> 3;
 
-  StageRegs<swa1_items(D, HCW)> srk, srv;
-  swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, 8 * ch_first, rope_idx, tid);
-  swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, 8 * ch_first, nullptr, tid);
+  constexpr int NI = swa1_items(D, HCW);
+  StagePlan<NI> sp;
+  swa1_plan_init<D, HCW>(sp, G, PITCH, tid);
+  const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
+  const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
+  StageRegs<NI> srk, srv;
+  swa1_regs_zero(srk);
+  swa1_regs_zero(srv);
+  swa1_issue(srk, sp, on_k, kb_, sn2k, G, 8 * ch_first, rope_idx);
+  swa1_issue(srv, sp, on_v, vb_, sn2v, G, 8 * ch_first, nullptr);
 
-  stage_tile<TIO, CT, D>(sK, PITCH, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, 64, own_token, a.p.rope, tid);
-  __syncthreads();
+  // own queries straight into B-operand fragments (rotated on the way when fused)
   u32x4 qf[KC];
-#pragma unroll
-  for (int c = 0; c < KC; c++) qf[c] = lds_read16(sK + (16 * wave + n) * PITCH + (32 * c + 8 * g) * 2);
-  __syncthreads();
+  swa1_load_own<TIO, CT, D>(qf, qb, a.qs[2], a.p.dk, own_token(16 * wave + n), g, a.p.rope, use_rope);
 
   // ---- window of this lane's query in halo coordinates -> additive biases
   const int qr_l = n >> 2, qc_l = n & 3;
@@ -111,15 +115,15 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const 
   const unsigned one2 = pack2<CT>(1.f, 1.f);
   const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
 
-  swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, a.p.rope, use_rope, tid);
-  swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, a.p.rope, false, tid);
+  swa1_commit<CT>(srk, sp, sK, a.rope_pbit, a.p.rope, use_rope && on_k);
+  swa1_commit<CT>(srv, sp, sV, 1, a.p.rope, false);
   __syncthreads();
 
   for (int ch = ch_first; ch <= ch_last; ch++) {
     const int cr0 = 8 * ch;
     if (ch < ch_last) {  // next chunk: HBM -> registers while this one is consumed
-      swa1_issue<TIO, D, HCW>(srk, kb_, (int)a.ks[2], a.p.dk, G, cr0 + 8, rope_idx, tid);
-      swa1_issue<TIO, D, HCW>(srv, vb_, (int)a.vs[2], a.p.dv, G, cr0 + 8, nullptr, tid);
+      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + 8, rope_idx);
+      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + 8, nullptr);
     }
 
     float t[NCGMAX][8];
@@ -193,8 +197,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const 
     }
     __syncthreads();  // every wave is done with this chunk
     if (ch < ch_last) {
-      swa1_commit<CT, D, HCW>(srk, sK, PITCH, a.rope_pbit, a.p.rope, use_rope, tid);
-      swa1_commit<CT, D, HCW>(srv, sV, PITCH, 1, a.p.rope, false, tid);
+      swa1_commit<CT>(srk, sp, sK, a.rope_pbit, a.p.rope, use_rope && on_k);
+      swa1_commit<CT>(srv, sp, sV, 1, a.p.rope, false);
       __syncthreads();
     }
   }

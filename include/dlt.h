@@ -153,6 +153,11 @@ typedef struct {
   int32_t kernel; /* DLT_K_* */
   float ms;
 } dlt_kernel_time_t;
+/* Plain device-to-device copy of `bytes` bytes (16-byte aligned, multiple of 16) by a grid-stride
+ * kernel: a workload of exactly known traffic, used to calibrate what the profiler's
+ * FETCH_SIZE / WRITE_SIZE counters report per byte.  No counterpart in the reference. */
+int dlt_debug_copy(void* dst, const void* src, int64_t bytes, void* stream);
+
 int dlt_timing_enable(int on);
 int dlt_timing_collect(dlt_kernel_time_t* out, int max, int* n);
 
