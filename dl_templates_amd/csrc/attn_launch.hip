@@ -4,6 +4,7 @@
 #include "attn_bwd_kernel.hpp"
 #include "swa1_fwd_kernel.hpp"
 #include "swa1_bwd_kernel.hpp"
+#include "flash_kernel.hpp"
 
 int dlt_launch_fwd_64_64(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_128_128(const FwdArgs&, int, int, hipStream_t);
@@ -13,6 +14,9 @@ int dlt_launch_bwd_64_64(const BwdArgs&, int, const BwdArgs&, int, int, hipStrea
 int dlt_launch_bwd_128_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_64_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 
+int dlt_flash_launch_fwd_64_64(const FlashArgs&, int, int, hipStream_t);
+int dlt_flash_launch_fwd_128_128(const FlashArgs&, int, int, hipStream_t);
+int dlt_flash_launch_fwd_64_128(const FlashArgs&, int, int, hipStream_t);
 int dlt_launch_delta_64_64(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_128_128(const BwdArgs&, hipStream_t);
 int dlt_swa1_launch_bwd_64(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
@@ -113,7 +117,7 @@ void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int
   plan.HRP = roundup(4 + 2 * p.g.WR, 8);
   plan.nblk_r = (p.g.TR + 3) / 4;
   plan.nblk_c = (p.g.TC + 15) / 16;
-  plan.lds_bytes = n_regions * 8 * hcw * (c.D * 2 + 16) + extra_bytes;
+  plan.lds_bytes = n_regions * 8 * hcw * (c.D * 2 + SWA1_PAD) + extra_bytes;
 }
 
 // the token-grid kernels index a [N, D] slab with 32-bit element offsets
@@ -178,6 +182,42 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
                    : dlt_swa1_launch_fwd_128(a, c.wclass, (int)grid, stream);
 }
 
+// ---- dense flash fast path ----------------------------------------------------------------
+// needs 2-byte elements, 16-byte vector access to q, k, v and 32-bit byte offsets inside a slab
+bool flash_eligible(const AttnProblem& p, const AttnTensors& t, bool with_do) {
+  if (p.g.mode != DLT_GEOM_DENSE) return false;
+  if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
+  const int es = 2;
+  if (!vec_ok(t.q, t.qs, 4, p.dk, es) || !vec_ok(t.k, t.ks, 4, p.dk, es) || !vec_ok(t.v, t.vs, 4, p.dv, es)) return false;
+  if (with_do && !vec_ok(t.d_o, t.dos, 4, p.dv, es)) return false;
+  const int64_t lim = ((int64_t)1 << 31) - 1;
+  if ((int64_t)p.g.XLk * t.ks[2] * es > lim || (int64_t)p.g.XLk * t.vs[2] * es > lim) return false;
+  if ((int64_t)p.g.XLq * t.qs[2] * es > lim) return false;
+  if (with_do && (int64_t)p.g.XLq * t.dos[2] * es > lim) return false;
+  return true;
+}
+
+int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc, hipStream_t stream) {
+  FlashArgs a;
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
+  for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.B = p.B; a.H = p.H; a.Lq = p.g.XLq; a.Lk = p.g.XLk; a.dk = p.dk; a.dv = p.dv;
+  const int own = 64 * FLASH_NP;
+  a.nblk = (a.Lq + own - 1) / own;
+  a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, 2);
+  const int chunk = FLASH_CK * (dc.DK * 2 + 16 + dc.DV * 2 + 16), tile = own * (dc.DV * 2 + 16);
+  a.lds_bytes = chunk > tile ? chunk : tile;
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  const int64_t grid = (int64_t)p.B * p.H * a.nblk;
+  if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "flash forward: grid too large");
+  switch (dc.id) {
+    case 0: return dlt_flash_launch_fwd_64_64(a, p.dtype, (int)grid, stream);
+    case 1: return dlt_flash_launch_fwd_128_128(a, p.dtype, (int)grid, stream);
+    default: return dlt_flash_launch_fwd_64_128(a, p.dtype, (int)grid, stream);
+  }
+}
+
 }  // namespace
 
 int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
@@ -193,6 +233,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
       if (rc != -1) return rc;
     }
   }
+  if (flash_eligible(p, t, false)) return flash_forward(p, t, dc, stream);
   const int np = p.g.mode == DLT_GEOM_SWA ? 1 : 2;
   const int own = 64 * np;
   const int PQ = dc.DK * 2 + 16, PK = dc.DK * 2 + 16, PV = dc.DV * 2 + 16, PO = dc.DV * es + 16;

@@ -1,0 +1,26 @@
+// Included by flash_inst_<DK>_<DV>.hip with DLT_DK / DLT_DV defined: dense flash kernels for
+// one pair of padded head dims.
+#include "flash_kernel.hpp"
+
+#define DLT_FCAT3_(a, b, c) a##b##_##c
+#define DLT_FCAT3(a, b, c) DLT_FCAT3_(a, b, c)
+
+namespace {
+template <typename TIO>
+int flash_launch_fwd_t(const FlashArgs& a, int grid, hipStream_t stream) {
+  auto kern = flash_fwd_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK>;
+  if (a.lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, a.lds_bytes);
+    if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", a.lds_bytes, hipGetErrorString(e));
+  }
+  dlt_timing_before(DLT_K_FWD, stream);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), a.lds_bytes, stream, a);
+  dlt_timing_after(stream);
+  DLT_CHECK_LAUNCH("flash forward launch");
+  return DLT_OK;
+}
+}  // namespace
+
+int DLT_FCAT3(dlt_flash_launch_fwd_, DLT_DK, DLT_DV)(const FlashArgs& a, int dtype, int grid, hipStream_t stream) {
+  return dtype == DLT_BF16 ? flash_launch_fwd_t<bf16_t>(a, grid, stream) : flash_launch_fwd_t<f16_t>(a, grid, stream);
+}

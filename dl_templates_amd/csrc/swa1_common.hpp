@@ -11,6 +11,10 @@
 #pragma once
 #include "attn_common.hpp"
 
+#ifndef SWA1_PAD
+#define SWA1_PAD 16  // bytes of padding after each token row of an LDS chunk
+#endif
+
 struct Swa1Plan {
   int32_t HRP;      // halo rows, padded to a multiple of 8 (chunks hold 8 halo rows)
   int32_t ncg;      // 4-column groups per wave window that can hold a visible token

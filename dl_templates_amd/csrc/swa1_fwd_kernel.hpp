@@ -27,7 +27,7 @@ template <typename TIO, int D, int NCGMAX>
 __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const Swa1FwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr int PITCH = D * 2 + 16;
+  constexpr int PITCH = D * 2 + SWA1_PAD;
   constexpr int KC = D / 32, VB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
   constexpr int REGION = 8 * HCW * PITCH;
