@@ -17,8 +17,12 @@ int dlt_launch_bwd_64_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStre
 int dlt_flash_launch_fwd_64_64(const FlashArgs&, int, int, hipStream_t);
 int dlt_flash_launch_fwd_128_128(const FlashArgs&, int, int, hipStream_t);
 int dlt_flash_launch_fwd_64_128(const FlashArgs&, int, int, hipStream_t);
+int dlt_flash_launch_bwd_64_64(const FlashBwdArgs&, int, int, int, hipStream_t);
+int dlt_flash_launch_bwd_128_128(const FlashBwdArgs&, int, int, int, hipStream_t);
+int dlt_flash_launch_bwd_64_128(const FlashBwdArgs&, int, int, int, hipStream_t);
 int dlt_launch_delta_64_64(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_128_128(const BwdArgs&, hipStream_t);
+int dlt_launch_delta_64_128(const BwdArgs&, hipStream_t);
 int dlt_swa1_launch_bwd_64(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
 int dlt_swa1_launch_bwd_128(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
 int dlt_swa1_launch_fwd_64(const Swa1FwdArgs&, int, int, hipStream_t);
@@ -218,6 +222,51 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
   }
 }
 
+int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc, hipStream_t stream) {
+  BwdArgs d;
+  d.p = p;
+  d.o = t.o; d.d_o = t.d_o; d.delta = t.delta;
+  for (int i = 0; i < 4; i++) { d.os[i] = t.os[i]; d.dos[i] = t.dos[i]; }
+  for (int i = 0; i < 3; i++) d.ls[i] = t.ls[i];
+  d.o_vec = vec_ok(t.o, t.os, 4, p.dv, 2);
+  d.do_vec = 1;
+  d.n_tokens_q = p.g.XLq;
+  int rc = dc.id == 0 ? dlt_launch_delta_64_64(d, stream) : dc.id == 1 ? dlt_launch_delta_128_128(d, stream) : dlt_launch_delta_64_128(d, stream);
+  if (rc != DLT_OK) return rc;
+
+  FlashBwdArgs a;
+  a.q = t.q; a.k = t.k; a.v = t.v; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
+  for (int i = 0; i < 4; i++) {
+    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.dos[i] = t.dos[i];
+    a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
+  }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.B = p.B; a.H = p.H; a.Lq = p.g.XLq; a.Lk = p.g.XLk; a.dk_ = p.dk; a.dv_ = p.dv;
+  const int own = 64 * FLASH_NP, own_kv = 64 * flash_np_kv(dc.DK, dc.DV);
+  a.nblk_q = (a.Lq + own - 1) / own;
+  a.nblk_k = (a.Lk + own_kv - 1) / own_kv;
+  a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, 2);
+  a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, 2);
+  a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, 2);
+  const int chunk = FLASH_CK * (dc.DK * 2 + 16 + dc.DV * 2 + 16);
+  const int tile_q = own * (dc.DK * 2 + 16);
+  const int tile_k = own_kv * (dc.DK * 2 + 16), tile_v = own_kv * (dc.DV * 2 + 16);
+  a.lds_q = chunk > tile_q ? chunk : tile_q;
+  a.lds_kv = chunk + 2 * FLASH_CK * 4;
+  if (tile_k > a.lds_kv) a.lds_kv = tile_k;
+  if (tile_v > a.lds_kv) a.lds_kv = tile_v;
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  a.sm_scale = p.sm_scale;
+  const int64_t grid_q = (int64_t)p.B * p.H * a.nblk_q, grid_kv = (int64_t)p.B * p.H * a.nblk_k;
+  if (grid_q > 0x7fffffff || grid_kv > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "flash backward: grid too large");
+  switch (dc.id) {
+    case 0: return dlt_flash_launch_bwd_64_64(a, p.dtype, (int)grid_kv, (int)grid_q, stream);
+    case 1: return dlt_flash_launch_bwd_128_128(a, p.dtype, (int)grid_kv, (int)grid_q, stream);
+    default: return dlt_flash_launch_bwd_64_128(a, p.dtype, (int)grid_kv, (int)grid_q, stream);
+  }
+}
+
 }  // namespace
 
 int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
@@ -271,6 +320,7 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
     Swa1Class c;
     if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(t)) return swa1_backward(p, t, c, stream);
   }
+  if (flash_eligible(p, t, true)) return flash_backward(p, t, dc, stream);
   const int np = 1;
   const int own = 64 * np;
   const int PQ = dc.DK * 2 + 16, PV = dc.DV * 2 + 16;

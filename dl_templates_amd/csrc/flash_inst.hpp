@@ -19,7 +19,43 @@ int flash_launch_fwd_t(const FlashArgs& a, int grid, hipStream_t stream) {
   DLT_CHECK_LAUNCH("flash forward launch");
   return DLT_OK;
 }
+
+template <typename KernT>
+int flash_set_lds(KernT kern, int bytes) {
+  if (bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
+  }
+  return DLT_OK;
+}
+
+template <typename TIO>
+int flash_launch_bwd_t(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
+  {
+    auto kern = flash_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, flash_np_kv(DLT_DK, DLT_DV), FLASH_CK>;
+    int rc = flash_set_lds(kern, a.lds_kv);
+    if (rc != DLT_OK) return rc;
+    dlt_timing_before(DLT_K_BWD_KV, stream);
+    hipLaunchKernelGGL(kern, dim3(grid_kv), dim3(256), a.lds_kv, stream, a);
+    dlt_timing_after(stream);
+    DLT_CHECK_LAUNCH("flash dK/dV launch");
+  }
+  {
+    auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK>;
+    int rc = flash_set_lds(kern, a.lds_q);
+    if (rc != DLT_OK) return rc;
+    dlt_timing_before(DLT_K_BWD_Q, stream);
+    hipLaunchKernelGGL(kern, dim3(grid_q), dim3(256), a.lds_q, stream, a);
+    dlt_timing_after(stream);
+    DLT_CHECK_LAUNCH("flash dQ launch");
+  }
+  return DLT_OK;
+}
 }  // namespace
+
+int DLT_FCAT3(dlt_flash_launch_bwd_, DLT_DK, DLT_DV)(const FlashBwdArgs& a, int dtype, int grid_kv, int grid_q, hipStream_t stream) {
+  return dtype == DLT_BF16 ? flash_launch_bwd_t<bf16_t>(a, grid_kv, grid_q, stream) : flash_launch_bwd_t<f16_t>(a, grid_kv, grid_q, stream);
+}
 
 int DLT_FCAT3(dlt_flash_launch_fwd_, DLT_DK, DLT_DV)(const FlashArgs& a, int dtype, int grid, hipStream_t stream) {
   return dtype == DLT_BF16 ? flash_launch_fwd_t<bf16_t>(a, grid, stream) : flash_launch_fwd_t<f16_t>(a, grid, stream);

@@ -14,6 +14,8 @@
 
 constexpr int FLASH_NP = 2;   // 16-query blocks per wave
 constexpr int FLASH_CK = 64;  // keys per LDS chunk
+// key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
+constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 128 ? 1 : 2; }
 
 struct FlashArgs {
   const void *q, *k, *v;
@@ -205,4 +207,326 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   __syncthreads();
   store_tile<TIO, TL, DV>(smem, PO, ob, a.os[2], a.os[3], a.dv, a.o_vec != 0, OWN,
                           [&](int row) { return x0 + row < a.Lq ? (int64_t)(x0 + row) : (int64_t)-1; }, no_rope, tid);
+}
+
+// =============================================================================================
+// Dense backward: replaces _attn_bwd_dkdv / _attn_bwd_dq / _attn_bwd (src/flash_attn.py:204-449)
+// for the non-causal case, Lq != Lk allowed, with the decoupled structure of the reference
+// (dK/dV pass over key blocks, dQ pass over query blocks) as two kernels; no host-side
+// pre-scaling pass over k (src/flash_attn.py:509-510), no atomics.
+struct FlashBwdArgs {
+  const void *q, *k, *v, *d_o;
+  const float *lse, *delta;
+  void *dq, *dk, *dv;
+  int64_t qs[4], ks[4], vs[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int32_t B, H, Lq, Lk, dk_, dv_;
+  int32_t nblk_q, nblk_k;
+  int32_t dq_vec, dk_vec, dv_vec;
+  int32_t lds_q, lds_kv;
+  float scale_log2, sm_scale;
+};
+
+// Staging of one chunk of CK tokens of two [token][dim] tensors (dims DA and DB) through registers.
+template <int DA, int DB, int CK>
+struct PairStage {
+  static constexpr int ACH = DA / 8, BCH = DB / 8;
+  static constexpr int NAI = CK * ACH / 256, NBI = CK * BCH / 256;
+  static_assert(CK * ACH % 256 == 0 && CK * BCH % 256 == 0, "chunk must split evenly over 256 threads");
+  u32x4 ra[NAI], rb[NBI];
+  int ac, akey0, bc, bkey0;
+  bool on_a, on_b;
+
+  DLT_DEV void init(int tid, int dact_a, int dact_b) {
+    ac = tid % ACH; akey0 = tid / ACH;
+    bc = tid % BCH; bkey0 = tid / BCH;
+    on_a = 8 * ac < dact_a; on_b = 8 * bc < dact_b;
+#pragma unroll
+    for (int it = 0; it < NAI; it++) ra[it] = u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int it = 0; it < NBI; it++) rb[it] = u32x4{0u, 0u, 0u, 0u};
+  }
+  // tokens past `len` are clamped onto the last token (the caller masks them)
+  DLT_DEV void issue(const char* a, int sn2a, const char* b, int sn2b, int t0, int len) {
+#pragma unroll
+    for (int it = 0; it < NAI; it++) {
+      const int tok = dlt_imin(t0 + akey0 + it * (256 / ACH), len - 1);
+      if (on_a) ra[it] = *reinterpret_cast<const u32x4*>(a + (uint32_t)(tok * sn2a + 16 * ac));
+    }
+#pragma unroll
+    for (int it = 0; it < NBI; it++) {
+      const int tok = dlt_imin(t0 + bkey0 + it * (256 / BCH), len - 1);
+      if (on_b) rb[it] = *reinterpret_cast<const u32x4*>(b + (uint32_t)(tok * sn2b + 16 * bc));
+    }
+  }
+  DLT_DEV void commit(char* sa, int pa, char* sb, int pb) const {
+#pragma unroll
+    for (int it = 0; it < NAI; it++) lds_write16(sa + (akey0 + it * (256 / ACH)) * pa + 16 * ac, ra[it]);
+#pragma unroll
+    for (int it = 0; it < NBI; it++) lds_write16(sb + (bkey0 + it * (256 / BCH)) * pb + 16 * bc, rb[it]);
+  }
+};
+
+// accumulators (C layout, [dim][own token]) of NP blocks -> LDS tile -> HBM rows
+template <typename TIO, int D, int NP>
+DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO* base, int64_t sn, int64_t sd, int dact,
+                              bool vec, int x0, int len, int wave, int n, int g, int tid) {
+  typedef typename TileOf<TIO>::type TL;
+  constexpr int PT = D * (int)sizeof(TL) + 16;
+  RopeDev no_rope = RopeDev{};
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    TL* row = reinterpret_cast<TL*>(sT + (wave * 16 * NP + 16 * p + n) * PT);
+#pragma unroll
+    for (int d = 0; d < D / 16; d++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) row[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * mul);
+  }
+  __syncthreads();
+  store_tile<TIO, TL, D>(sT, PT, base, sn, sd, dact, vec, 64 * NP,
+                         [&](int r) { return x0 + r < len ? (int64_t)(x0 + r) : (int64_t)-1; }, no_rope, tid);
+  __syncthreads();
+}
+
+// ---- dQ: own = queries, K and V stream
+template <typename TIO, int DK, int DV, int NP, int CK>
+__global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs a) {
+  typedef typename ComputeOf<TIO>::type CT;
+  extern __shared__ __align__(16) char smem[];
+  constexpr int PK = DK * 2 + 16, PV = DV * 2 + 16;
+  constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, NKB = CK / 32;
+  constexpr int OWN = 64 * NP;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  char* sK = smem;
+  char* sV = smem + CK * PK;
+
+  const int lin = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = lin / a.nblk_q;
+  const int x0 = (lin - bh * a.nblk_q) * OWN;
+  const int b = bh / a.H, h = bh - b * a.H;
+  const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
+  const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
+  const char* kb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1]);
+  const char* vb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1]);
+  const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
+  RopeDev no_rope = RopeDev{};
+
+  PairStage<DK, DV, CK> st;
+  st.init(tid, a.dk_, a.dv_);
+  st.issue(kb_, sn2k, vb_, sn2v, 0, a.Lk);
+
+  u32x4 qf[NP][KC], dof[NP][VC];
+  float nlse[NP], del_n[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int xq = x0 + wave * 16 * NP + 16 * p + n;
+    const int64_t tq = xq < a.Lq ? (int64_t)xq : (int64_t)-1;
+    swa1_load_own<TIO, CT, DK>(qf[p], qb, a.qs[2], a.dk_, tq, g, no_rope, false);
+    swa1_load_own<TIO, CT, DV>(dof[p], dob, a.dos[2], a.dv_, tq, g, no_rope, false);
+    const int64_t off = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
+    nlse[p] = tq >= 0 ? -a.lse[off] : 0.f;
+    del_n[p] = tq >= 0 ? a.delta[off] : 0.f;
+  }
+  f32x4 dq_acc[NP][KB];
+#pragma unroll
+  for (int p = 0; p < NP; p++)
+#pragma unroll
+    for (int d = 0; d < KB; d++) dq_acc[p][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float scale = a.scale_log2;
+
+  st.commit(sK, PK, sV, PV);
+  __syncthreads();
+
+  for (int k0 = 0; k0 < a.Lk; k0 += CK) {
+    const bool has_next = k0 + CK < a.Lk;
+    if (has_next) st.issue(kb_, sn2k, vb_, sn2v, k0 + CK, a.Lk);
+    const bool tail = k0 + CK > a.Lk;
+#pragma unroll
+    for (int kb = 0; kb < NKB; kb++) {
+      u32x4 ka[2][KC], va[2][VC];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+#pragma unroll
+        for (int c = 0; c < KC; c++) ka[mb][c] = lds_read16(sK + (32 * kb + 16 * mb + n) * PK + (32 * c + 8 * g) * 2);
+#pragma unroll
+        for (int c = 0; c < VC; c++) va[mb][c] = lds_read16(sV + (32 * kb + 16 * mb + n) * PV + (32 * c + 8 * g) * 2);
+      }
+      u32x4 dsb[NP];
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        f32x4 s[2], dp[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) {
+          s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+          dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < KC; c++) s[mb] = Mma<CT>::mfma(ka[mb][c], qf[p][c], s[mb]);
+#pragma unroll
+          for (int c = 0; c < VC; c++) dp[mb] = Mma<CT>::mfma(va[mb][c], dof[p][c], dp[mb]);
+        }
+        float ds[8];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            float pv = fast_exp2(fmaf(s[mb][i], scale, nlse[p]));
+            if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) < a.Lk ? pv : 0.f;
+            ds[4 * mb + i] = pv * (dp[mb][i] - del_n[p]);
+          }
+        dsb[p] = pack8<CT>(ds);
+      }
+#pragma unroll
+      for (int d = 0; d < KB; d++) {
+        const u32x4 kt = lds_read_tokens_as_k(sK, PK, 32 * kb, 16 * d, n, g);
+#pragma unroll
+        for (int p = 0; p < NP; p++) dq_acc[p][d] = Mma<CT>::mfma(kt, dsb[p], dq_acc[p][d]);
+      }
+    }
+    __syncthreads();
+    if (has_next) {
+      st.commit(sK, PK, sV, PV);
+      __syncthreads();
+    }
+  }
+  TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
+  flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, a.dqs[2], a.dqs[3], a.dk_, a.dq_vec != 0, x0, a.Lq, wave, n, g, tid);
+}
+
+// ---- dK / dV: own = keys, Q, dO, lse2 and delta stream
+template <typename TIO, int DK, int DV, int NP, int CK>
+__global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
+  typedef typename ComputeOf<TIO>::type CT;
+  extern __shared__ __align__(16) char smem[];
+  constexpr int PQ = DK * 2 + 16, PD = DV * 2 + 16;
+  constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16, NQB = CK / 32;
+  constexpr int OWN = 64 * NP;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  char* sQ = smem;
+  char* sDO = smem + CK * PQ;
+  float* sLse = reinterpret_cast<float*>(smem + CK * (PQ + PD));
+  float* sDel = sLse + CK;
+
+  const int lin = xcd_remap(blockIdx.x, gridDim.x);
+  const int bh = lin / a.nblk_k;
+  const int x0 = (lin - bh * a.nblk_k) * OWN;
+  const int b = bh / a.H, h = bh - b * a.H;
+  const TIO* kb_ = reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1];
+  const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
+  const char* qb = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1]);
+  const char* dob = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1]);
+  const float* lseb = a.lse + b * a.ls[0] + h * a.ls[1];
+  const float* delb = a.delta + b * a.ls[0] + h * a.ls[1];
+  const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
+  RopeDev no_rope = RopeDev{};
+
+  PairStage<DK, DV, CK> st;
+  st.init(tid, a.dk_, a.dv_);
+  st.issue(qb, sn2q, dob, sn2d, 0, a.Lq);
+  float r_lse = 0.f, r_del = 0.f;
+  auto issue_scalars = [&](int q0) {
+    if (tid < CK) {
+      const int64_t tok = dlt_imin(q0 + tid, a.Lq - 1);
+      r_lse = lseb[tok * a.ls[2]];
+      r_del = delb[tok * a.ls[2]];
+    }
+  };
+  issue_scalars(0);
+
+  u32x4 kf[NP][KC], vf[NP][VC];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int xk = x0 + wave * 16 * NP + 16 * p + n;
+    const int64_t tk = xk < a.Lk ? (int64_t)xk : (int64_t)-1;
+    swa1_load_own<TIO, CT, DK>(kf[p], kb_, a.ks[2], a.dk_, tk, g, no_rope, false);
+    swa1_load_own<TIO, CT, DV>(vf[p], vb_, a.vs[2], a.dv_, tk, g, no_rope, false);
+  }
+  f32x4 dk_acc[NP][KB], dv_acc[NP][VB];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+#pragma unroll
+    for (int d = 0; d < KB; d++) dk_acc[p][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int d = 0; d < VB; d++) dv_acc[p][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float scale = a.scale_log2;
+
+  st.commit(sQ, PQ, sDO, PD);
+  if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
+  __syncthreads();
+
+  for (int q0 = 0; q0 < a.Lq; q0 += CK) {
+    const bool has_next = q0 + CK < a.Lq;
+    if (has_next) {
+      st.issue(qb, sn2q, dob, sn2d, q0 + CK, a.Lq);
+      issue_scalars(q0 + CK);
+    }
+    const bool tail = q0 + CK > a.Lq;
+#pragma unroll
+    for (int qb_ = 0; qb_ < NQB; qb_++) {
+      u32x4 qa[2][KC], da[2][VC];
+      f32x4 lq[2], dl[2];
+#pragma unroll
+      for (int mb = 0; mb < 2; mb++) {
+#pragma unroll
+        for (int c = 0; c < KC; c++) qa[mb][c] = lds_read16(sQ + (32 * qb_ + 16 * mb + n) * PQ + (32 * c + 8 * g) * 2);
+#pragma unroll
+        for (int c = 0; c < VC; c++) da[mb][c] = lds_read16(sDO + (32 * qb_ + 16 * mb + n) * PD + (32 * c + 8 * g) * 2);
+        lq[mb] = *reinterpret_cast<const f32x4*>(sLse + 32 * qb_ + 16 * mb + 4 * g);
+        dl[mb] = *reinterpret_cast<const f32x4*>(sDel + 32 * qb_ + 16 * mb + 4 * g);
+      }
+      u32x4 pb[NP], dsb[NP];
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        f32x4 s[2], dp[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) {
+          s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+          dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int c = 0; c < KC; c++) s[mb] = Mma<CT>::mfma(qa[mb][c], kf[p][c], s[mb]);
+#pragma unroll
+          for (int c = 0; c < VC; c++) dp[mb] = Mma<CT>::mfma(da[mb][c], vf[p][c], dp[mb]);
+        }
+        float pr[8], ds[8];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            float pv = fast_exp2(fmaf(s[mb][i], scale, -lq[mb][i]));
+            if (tail) pv = (q0 + 32 * qb_ + 16 * mb + 4 * g + i) < a.Lq ? pv : 0.f;
+            pr[4 * mb + i] = pv;
+            ds[4 * mb + i] = pv * (dp[mb][i] - dl[mb][i]);
+          }
+        pb[p] = pack8<CT>(pr);
+        dsb[p] = pack8<CT>(ds);
+      }
+#pragma unroll
+      for (int d = 0; d < VB; d++) {
+        const u32x4 dt = lds_read_tokens_as_k(sDO, PD, 32 * qb_, 16 * d, n, g);
+#pragma unroll
+        for (int p = 0; p < NP; p++) dv_acc[p][d] = Mma<CT>::mfma(dt, pb[p], dv_acc[p][d]);
+      }
+#pragma unroll
+      for (int d = 0; d < KB; d++) {
+        const u32x4 qt = lds_read_tokens_as_k(sQ, PQ, 32 * qb_, 16 * d, n, g);
+#pragma unroll
+        for (int p = 0; p < NP; p++) dk_acc[p][d] = Mma<CT>::mfma(qt, dsb[p], dk_acc[p][d]);
+      }
+    }
+    __syncthreads();
+    if (has_next) {
+      st.commit(sQ, PQ, sDO, PD);
+      if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
+      __syncthreads();
+    }
+  }
+  TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
+  TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
+  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, a.dks[2], a.dks[3], a.dk_, a.dk_vec != 0, x0, a.Lk, wave, n, g, tid);
+  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.dv_, a.dv_vec != 0, x0, a.Lk, wave, n, g, tid);
 }
