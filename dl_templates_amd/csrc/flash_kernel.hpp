@@ -12,8 +12,14 @@
 #pragma once
 #include "swa1_common.hpp"
 
-constexpr int FLASH_NP = 2;   // 16-query blocks per wave
-constexpr int FLASH_CK = 64;  // keys per LDS chunk
+#ifndef FLASH_NP_DEF
+#define FLASH_NP_DEF 2
+#endif
+#ifndef FLASH_CK_DEF
+#define FLASH_CK_DEF 64
+#endif
+constexpr int FLASH_NP = FLASH_NP_DEF;  // 16-query blocks per wave (forward and dQ)
+constexpr int FLASH_CK = FLASH_CK_DEF;  // streamed tokens per LDS chunk
 // key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
 constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 128 ? 1 : 2; }
 
