@@ -115,13 +115,15 @@ bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streame
 }
 
 // n_regions: [8 rows x HCW tokens] LDS regions the kernel keeps resident
-void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int extra_bytes, Swa1Plan& plan) {
+void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int extra_bytes, Swa1Plan& plan, int cr = 8) {
   plan.ncg = (4 + 2 * p.g.WC + 3) / 4;
   const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
-  plan.HRP = roundup(4 + 2 * p.g.WR, 8);
+  plan.HRP = roundup(4 + 2 * p.g.WR, cr);
   plan.nblk_r = (p.g.TR + 3) / 4;
   plan.nblk_c = (p.g.TC + 15) / 16;
-  plan.lds_bytes = n_regions * 8 * hcw * (c.D * 2 + SWA1_PAD) + extra_bytes;
+  plan.lds_bytes = n_regions * cr * hcw * (c.D * 2 + SWA1_PAD) + extra_bytes;
+  const int own_tile = 64 * (c.D * 2 + 16);  // output tile of the epilogue
+  if (plan.lds_bytes < own_tile) plan.lds_bytes = own_tile;
 }
 
 // the token-grid kernels index a [N, D] slab with 32-bit element offsets
@@ -146,9 +148,13 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
 
   Swa1BwdArgs a;
   a.p = p;
+  // the dQ kernel streams 4-row chunks, the dK/dV kernel 8-row chunks; HRP (a multiple of 8 here)
+  // serves both
+  Swa1Plan plan_q;
+  swa1_make_plan(p, c, 2, 0, plan_q, SWA1_FWD_CR);
   swa1_make_plan(p, c, 2, 0, a.plan);
   const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
-  const int lds_q = a.plan.lds_bytes, lds_kv = a.plan.lds_bytes + 2 * 8 * hcw * 4;
+  const int lds_q = plan_q.lds_bytes, lds_kv = a.plan.lds_bytes + 2 * 8 * hcw * 4;
   a.q = t.q; a.k = t.k; a.v = t.v; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
   a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
   for (int i = 0; i < 4; i++) {
@@ -172,7 +178,7 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
   const int es = dlt_elem_size(p.dtype);
   Swa1FwdArgs a;
   a.p = p;
-  swa1_make_plan(p, c, 2, 0, a.plan);
+  swa1_make_plan(p, c, 2, 0, a.plan, SWA1_FWD_CR);
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
   for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];

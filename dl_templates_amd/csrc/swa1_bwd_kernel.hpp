@@ -65,7 +65,7 @@ struct Swa1Lane {
   bool wave_ok;
   int ch_first, ch_last;
 
-  DLT_DEV void init(const AttnProblem& p, const Swa1Plan& P, int wave, int n) {
+  DLT_DEV void init(const AttnProblem& p, const Swa1Plan& P, int wave, int n, int cr = 8) {
     const int lin = xcd_remap(blockIdx.x, gridDim.x);
     const int per_bh = P.nblk_r * P.nblk_c;
     const int bh = lin / per_bh;
@@ -91,9 +91,9 @@ struct Swa1Lane {
     wcol_lo = dlt_imax(0, G.WC - cw);
     wcol_hi = G.TC - 1 - cw + G.WC;
     wave_ok = cw < G.TC;
-    const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(P.HRP - 1, G.TR - 1 - G.r0 + G.WR);
-    ch_first = wrow_lo >> 3;
-    ch_last = wrow_hi >> 3;
+    const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(3 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
+    ch_first = wrow_lo / cr;
+    ch_last = wrow_hi / cr;
   }
   DLT_DEV int64_t own_token(int row) const {
     const int r = G.r0 + ((row & 15) >> 2), c = G.c0 + 4 * (row >> 4) + (row & 3);
@@ -237,8 +237,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
       const int kt0 = 4 * wave + 4 * cg;
 #pragma unroll
       for (int d = 0; d < DB; d++) {
-        dv_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sDO, PITCH, HCW, kt0, 16 * d, n, g), pb, dv_acc[d]);
-        dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PITCH, HCW, kt0, 16 * d, n, g), dsb, dk_acc[d]);
+        dv_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sDO, PITCH, HCW, kt0, 16 * d, n, g, 4 * HCW), pb, dv_acc[d]);
+        dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PITCH, HCW, kt0, 16 * d, n, g, 4 * HCW), dsb, dk_acc[d]);
       }
     }
     __syncthreads();
@@ -258,14 +258,16 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
 }
 
 // =============================================================================================
-template <typename TIO, int D, int NCGMAX>
-__global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
+template <typename TIO, int D, int NCGMAX, int CR>
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr int PITCH = D * 2 + SWA1_PAD;
   constexpr int KC = D / 32, DB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
-  constexpr int REGION = 8 * HCW * PITCH;
+  constexpr int REGION = CR * HCW * PITCH;
+  constexpr int NKB = CR == 8 ? NCGMAX : NCGMAX / 2;
+  constexpr int MB_STEP = CR == 8 ? 4 * HCW : 4;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -275,7 +277,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(cons
   char* sV = smem + REGION;
 
   Swa1Lane<NCGMAX> L;
-  L.init(a.p, P, wave, n);
+  L.init(a.p, P, wave, n, CR);
   const Swa1Geom& G = L.G;
   const int b = L.b, h = L.h;
 
@@ -290,16 +292,16 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(cons
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  constexpr int NI = swa1_items(D, HCW);
+  constexpr int NI = swa1_items(D, HCW, CR);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW>(sp, G, PITCH, tid);
+  swa1_plan_init<D, HCW, CR>(sp, G, PITCH, tid);
   const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   swa1_regs_zero(srv);
-  swa1_issue(srk, sp, on_k, kb_, sn2k, G, 8 * L.ch_first, rope_idx);
-  swa1_issue(srv, sp, on_v, vb_, sn2v, G, 8 * L.ch_first, nullptr);
+  swa1_issue(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx);
+  swa1_issue(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr);
 
   // own queries / output gradients straight into B-operand fragments
   u32x4 qf[KC], dof[KC];
@@ -320,21 +322,22 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(cons
   __syncthreads();
 
   for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
-    const int cr0 = 8 * ch;
+    const int cr0 = CR * ch;
     if (ch < L.ch_last) {
-      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + 8, rope_idx);
-      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + 8, nullptr);
+      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
+      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
     }
     float rbias[2];
 #pragma unroll
     for (int mb = 0; mb < 2; mb++) {
-      const int hrow = cr0 + 4 * mb + g;
+      const int hrow = cr0 + (CR == 8 ? 4 * mb : 0) + g;
       rbias[mb] = ((hrow >= L.rlo && hrow <= L.rhi) ? 0.f : -INFINITY) - lse_n;
     }
 #pragma unroll
-    for (int cg = 0; cg < NCGMAX; cg++) {
-      if (!L.block_on(P, cg)) continue;
-      const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg + (n & 3);
+    for (int kb = 0; kb < NKB; kb++) {
+      const int cg0 = CR == 8 ? kb : 2 * kb, cg1 = CR == 8 ? kb : 2 * kb + 1;
+      if (!(L.wave_ok && cg0 < P.ncg && 4 * cg0 <= L.wcol_hi && 4 * cg1 + 3 >= L.wcol_lo)) continue;
+      const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg0 + (n & 3);
       f32x4 s[2], dp[2];
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
@@ -342,8 +345,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(cons
         dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KC; c++) {
-          s[mb] = Mma<CT>::mfma(lds_read16(sK + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), qf[c], s[mb]);
-          dp[mb] = Mma<CT>::mfma(lds_read16(sV + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), dof[c], dp[mb]);
+          s[mb] = Mma<CT>::mfma(lds_read16(sK + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), qf[c], s[mb]);
+          dp[mb] = Mma<CT>::mfma(lds_read16(sV + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), dof[c], dp[mb]);
         }
       }
       float ds[8];
@@ -351,14 +354,14 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_q_kernel(cons
       for (int mb = 0; mb < 2; mb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const float pv = fast_exp2(fmaf(s[mb][i], scale, L.cbias[cg][i] + rbias[mb]));
+          const float pv = fast_exp2(fmaf(s[mb][i], scale, L.cbias[mb == 0 ? cg0 : cg1][i] + rbias[mb]));
           ds[4 * mb + i] = pv * (dp[mb][i] - del_n);
         }
       const u32x4 dsb = pack8<CT>(ds);
-      const int kt0 = 4 * wave + 4 * cg;
+      const int kt0 = 4 * wave + 4 * cg0;
 #pragma unroll
       for (int d = 0; d < DB; d++)
-        dq_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sK, PITCH, HCW, kt0, 16 * d, n, g), dsb, dq_acc[d]);
+        dq_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sK, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dq_acc[d]);
     }
     __syncthreads();
     if (ch < L.ch_last) {

@@ -27,7 +27,7 @@ struct Swa1Plan {
 constexpr int swa1_hcw(int ncgmax) { return 12 + 4 * ncgmax; }
 
 // 64-byte items (4 chunks of 8 dims of one token) a thread stages per 8-row chunk of one tensor
-constexpr int swa1_items(int d, int hcw) { return (8 * hcw * (d / 32) + 255) / 256; }
+constexpr int swa1_items(int d, int hcw, int cr = 8) { return (cr * hcw * (d / 32) + 255) / 256; }
 
 struct Swa1Geom {
   int r0, c0;      // first grid row / column of the workgroup's band
@@ -47,14 +47,14 @@ struct StagePlan {
   int qoff;      // byte offset of the thread's 64-byte piece inside a token row
 };
 
-template <int D, int HCW>
-DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW)>& sp, const Swa1Geom& G, int pitch, int tid) {
+template <int D, int HCW, int CR = 8>
+DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW, CR)>& sp, const Swa1Geom& G, int pitch, int tid) {
   constexpr int QUADS = D / 32;
   const int qd = tid % QUADS, key0 = tid / QUADS;
 #pragma unroll
-  for (int it = 0; it < swa1_items(D, HCW); it++) {
+  for (int it = 0; it < swa1_items(D, HCW, CR); it++) {
     const int key = key0 + it * (256 / QUADS);
-    const bool live = key < 8 * HCW;
+    const bool live = key < CR * HCW;
     const int k = live ? key : 0;
     const int hr = k / HCW, hc = k - hr * HCW;
     sp.hr[it] = hr;
@@ -182,10 +182,12 @@ DLT_DEV void swa1_load_own(u32x4 (&f)[D / 32], const TIO* base, int64_t sn, int 
 // A operand for a product that contracts over the 32 tokens of an 8x4 block: dims
 // dim0..dim0+15 of the [token][dim] chunk become the operand rows.  `key0` is the LDS token
 // index of the block's first row at the wave's column group.
-DLT_DEV u32x4 swa1_read_tokens_as_k(const char* tile, int pitch, int hcw, int key0, int dim0, int n, int g) {
+// `mb_step`: token distance between the two 4x4 halves of the block (4 * hcw: the half below,
+// 4: the half to the right).
+DLT_DEV u32x4 swa1_read_tokens_as_k(const char* tile, int pitch, int hcw, int key0, int dim0, int n, int g, int mb_step) {
   const char* p = tile + (key0 + g * hcw + (n >> 2)) * pitch + (dim0 + 4 * (n & 3)) * 2;
   const u32x2 lo = lds_read_tr16(p);
-  const u32x2 hi = lds_read_tr16(p + 4 * hcw * pitch);
+  const u32x2 hi = lds_read_tr16(p + mb_step * pitch);
   u32x4 r;
   r.x = lo.x; r.y = lo.y; r.z = hi.x; r.w = hi.y;
   return r;

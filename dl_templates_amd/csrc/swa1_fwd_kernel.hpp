@@ -11,6 +11,10 @@
 #pragma once
 #include "swa1_common.hpp"
 
+#ifndef SWA1_FWD_CR
+#define SWA1_FWD_CR 4  // halo rows per chunk in the forward kernel
+#endif
+
 struct Swa1FwdArgs {
   AttnProblem p;
   Swa1Plan plan;
@@ -23,14 +27,19 @@ struct Swa1FwdArgs {
   float scale_log2;
 };
 
-template <typename TIO, int D, int NCGMAX>
-__global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const Swa1FwdArgs a) {
+// CR: halo rows per chunk.  8: a 32-token block is 8 rows x 4 columns; 4: 4 rows x 8 columns
+// (half the LDS and staging registers per workgroup, hence more resident workgroups per CU).
+template <typename TIO, int D, int NCGMAX, int CR>
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 2) : (CR == 4 ? 2 : 1))) void swa1_fwd_kernel(const Swa1FwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr int PITCH = D * 2 + SWA1_PAD;
   constexpr int KC = D / 32, VB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
-  constexpr int REGION = 8 * HCW * PITCH;
+  constexpr int REGION = CR * HCW * PITCH;
+  constexpr int NKB = CR == 8 ? NCGMAX : NCGMAX / 2;      // 32-token blocks per wave and chunk
+  constexpr int MB_STEP = CR == 8 ? 4 * HCW : 4;          // token distance between the halves of a block
+  static_assert(CR == 8 || NCGMAX % 2 == 0, "4-row chunks pair column groups");
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -65,19 +74,19 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const 
   };
 
   // halo rows that hold at least one grid row; chunks outside are skipped by the whole workgroup
-  const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(P.HRP - 1, G.TR - 1 - G.r0 + G.WR);
-  const int ch_first = wrow_lo >> 3, ch_last = wrow_hi >> 3;
+  const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(3 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
+  const int ch_first = wrow_lo / CR, ch_last = wrow_hi / CR;
 
-  constexpr int NI = swa1_items(D, HCW);
+  constexpr int NI = swa1_items(D, HCW, CR);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW>(sp, G, PITCH, tid);
+  swa1_plan_init<D, HCW, CR>(sp, G, PITCH, tid);
   const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   swa1_regs_zero(srv);
-  swa1_issue(srk, sp, on_k, kb_, sn2k, G, 8 * ch_first, rope_idx);
-  swa1_issue(srv, sp, on_v, vb_, sn2v, G, 8 * ch_first, nullptr);
+  swa1_issue(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx);
+  swa1_issue(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr);
 
   // own queries straight into B-operand fragments (rotated on the way when fused)
   u32x4 qf[KC];
@@ -120,49 +129,52 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const 
   __syncthreads();
 
   for (int ch = ch_first; ch <= ch_last; ch++) {
-    const int cr0 = 8 * ch;
+    const int cr0 = CR * ch;
     if (ch < ch_last) {  // next chunk: HBM -> registers while this one is consumed
-      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + 8, rope_idx);
-      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + 8, nullptr);
+      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
+      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
     }
 
-    float t[NCGMAX][8];
+    // block kb, half mb -> (row offset inside the chunk, column group)
+    float t[NKB][8];
     float mloc = -INFINITY;
     float rbias[2];
 #pragma unroll
     for (int mb = 0; mb < 2; mb++) {
-      const int hrow = cr0 + 4 * mb + g;
+      const int hrow = cr0 + (CR == 8 ? 4 * mb : 0) + g;
       rbias[mb] = (hrow >= rlo && hrow <= rhi) ? 0.f : -INFINITY;
     }
     const bool row_edge = __builtin_amdgcn_ballot_w64(rbias[0] != 0.f || rbias[1] != 0.f) != 0;
+    bool on[NKB];
 #pragma unroll
-    for (int cg = 0; cg < NCGMAX; cg++) {
-      const bool on = wave_ok && cg < P.ncg && 4 * cg <= wcol_hi && 4 * cg + 3 >= wcol_lo;
-      if (on) {
-        const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg + (n & 3);
+    for (int kb = 0; kb < NKB; kb++) {
+      const int cg0 = CR == 8 ? kb : 2 * kb, cg1 = CR == 8 ? kb : 2 * kb + 1;
+      on[kb] = wave_ok && cg0 < P.ncg && 4 * cg0 <= wcol_hi && 4 * cg1 + 3 >= wcol_lo;
+      if (on[kb]) {
+        const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg0 + (n & 3);
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KC; c++) {
           const u32x4 k0 = lds_read16(sK + key0 * PITCH + (32 * c + 8 * g) * 2);
-          const u32x4 k1 = lds_read16(sK + (key0 + 4 * HCW) * PITCH + (32 * c + 8 * g) * 2);
+          const u32x4 k1 = lds_read16(sK + (key0 + MB_STEP) * PITCH + (32 * c + 8 * g) * 2);
           s0 = Mma<CT>::mfma(k0, qf[c], s0);
           s1 = Mma<CT>::mfma(k1, qf[c], s1);
         }
 #pragma unroll
-        for (int i = 0; i < 4; i++) { t[cg][i] = s0[i]; t[cg][4 + i] = s1[i]; }
-        if (cg_edge[cg]) {
+        for (int i = 0; i < 4; i++) { t[kb][i] = s0[i]; t[kb][4 + i] = s1[i]; }
+        if (cg_edge[cg0] || cg_edge[cg1]) {
 #pragma unroll
-          for (int i = 0; i < 4; i++) { t[cg][i] += cbias[cg][i]; t[cg][4 + i] += cbias[cg][i]; }
+          for (int i = 0; i < 4; i++) { t[kb][i] += cbias[cg0][i]; t[kb][4 + i] += cbias[cg1][i]; }
         }
         if (row_edge) {
 #pragma unroll
-          for (int i = 0; i < 4; i++) { t[cg][i] += rbias[0]; t[cg][4 + i] += rbias[1]; }
+          for (int i = 0; i < 4; i++) { t[kb][i] += rbias[0]; t[kb][4 + i] += rbias[1]; }
         }
-        mloc = fmaxf(mloc, fmaxf(fmaxf(fmaxf(t[cg][0], t[cg][1]), fmaxf(t[cg][2], t[cg][3])),
-                                 fmaxf(fmaxf(t[cg][4], t[cg][5]), fmaxf(t[cg][6], t[cg][7]))));
+        mloc = fmaxf(mloc, fmaxf(fmaxf(fmaxf(t[kb][0], t[kb][1]), fmaxf(t[kb][2], t[kb][3])),
+                                 fmaxf(fmaxf(t[kb][4], t[kb][5]), fmaxf(t[kb][6], t[kb][7]))));
       } else {
 #pragma unroll
-        for (int i = 0; i < 8; i++) t[cg][i] = -INFINITY;
+        for (int i = 0; i < 8; i++) t[kb][i] = -INFINITY;
       }
     }
     // one online-softmax update per chunk: p = exp2(s * scale - m * scale)
@@ -172,12 +184,12 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const 
     const float alpha = fast_exp2((m_run - m_use) * scale);
     const float neg_m2 = -m_use * scale;
     m_run = m_new;
-    u32x4 pb[NCGMAX];
+    u32x4 pb[NKB];
 #pragma unroll
-    for (int cg = 0; cg < NCGMAX; cg++) {
+    for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
-      for (int i = 0; i < 8; i++) t[cg][i] = fast_exp2(fmaf(t[cg][i], scale, neg_m2));
-      pb[cg] = pack8<CT>(t[cg]);
+      for (int i = 0; i < 8; i++) t[kb][i] = fast_exp2(fmaf(t[kb][i], scale, neg_m2));
+      pb[kb] = pack8<CT>(t[kb]);
     }
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
@@ -185,14 +197,13 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_fwd_kernel(const 
       acc_l *= alpha;
     }
 #pragma unroll
-    for (int cg = 0; cg < NCGMAX; cg++) {
-      const bool on = wave_ok && cg < P.ncg && 4 * cg <= wcol_hi && 4 * cg + 3 >= wcol_lo;
-      if (on) {
-        const int key0 = 4 * wave + 4 * cg;
+    for (int kb = 0; kb < NKB; kb++) {
+      if (on[kb]) {
+        const int key0 = 4 * wave + 4 * (CR == 8 ? kb : 2 * kb);
 #pragma unroll
         for (int d = 0; d < VB; d++)
-          acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PITCH, HCW, key0, 16 * d, n, g), pb[cg], acc[d]);
-        acc_l = Mma<CT>::mfma(ones, pb[cg], acc_l);
+          acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PITCH, HCW, key0, 16 * d, n, g, MB_STEP), pb[kb], acc[d]);
+        acc_l = Mma<CT>::mfma(ones, pb[kb], acc_l);
       }
     }
     __syncthreads();  // every wave is done with this chunk

@@ -17,7 +17,7 @@ int swa1_set_lds(KernT kern, int bytes) {
 
 template <typename TIO, int NCGMAX>
 int swa1_launch_fwd_t(const Swa1FwdArgs& a, int grid, hipStream_t stream) {
-  auto kern = swa1_fwd_kernel<TIO, DLT_D, NCGMAX>;
+  auto kern = swa1_fwd_kernel<TIO, DLT_D, NCGMAX, SWA1_FWD_CR>;
   int rc = swa1_set_lds(kern, a.plan.lds_bytes);
   if (rc != DLT_OK) return rc;
   dlt_timing_before(DLT_K_FWD, stream);
@@ -39,7 +39,7 @@ int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hip
     DLT_CHECK_LAUNCH("token-grid attention dK/dV launch");
   }
   {
-    auto kern = swa1_bwd_q_kernel<TIO, DLT_D, NCGMAX>;
+    auto kern = swa1_bwd_q_kernel<TIO, DLT_D, NCGMAX, SWA1_FWD_CR>;
     int rc = swa1_set_lds(kern, lds_q);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_Q, stream);
