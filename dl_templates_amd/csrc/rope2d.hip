@@ -10,7 +10,6 @@
 // keeps its 8 (cos, sin) pairs in registers while it walks over the batch rows, so the
 // table is read once per thread and the x traffic is 16-byte vector loads/stores.
 #include "dlt_internal.hpp"
-#include <stdlib.h>
 
 namespace {
 
@@ -202,7 +201,6 @@ int rope_impl(void* const x[2], const int64_t* const st[2], const int64_t nb[2],
   int bb = (int)maxb;
   while (bb > UNR && bx * ((maxb + bb - 1) / bb) * ntens < 2048) bb = (bb + 1) / 2;
   a.bb = bb < 1 ? 1 : bb;
-  if (const char* e = getenv("DLT_ROPE_BB")) { const int v = atoi(e); if (v > 0) a.bb = v; }
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case DLT_BF16: return launch_rope<bf16_t>(a, vec, s, ntens);

@@ -259,7 +259,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
 
 // =============================================================================================
 template <typename TIO, int D, int NCGMAX, int CR>
-__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr int PITCH = D * 2 + SWA1_PAD;

@@ -30,7 +30,7 @@ struct Swa1FwdArgs {
 // CR: halo rows per chunk.  8: a 32-token block is 8 rows x 4 columns; 4: 4 rows x 8 columns
 // (half the LDS and staging registers per workgroup, hence more resident workgroups per CU).
 template <typename TIO, int D, int NCGMAX, int CR>
-__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 2) : (CR == 4 ? 2 : 1))) void swa1_fwd_kernel(const Swa1FwdArgs a) {
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_fwd_kernel(const Swa1FwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr int PITCH = D * 2 + SWA1_PAD;
@@ -40,6 +40,9 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   constexpr int NKB = CR == 8 ? NCGMAX : NCGMAX / 2;      // 32-token blocks per wave and chunk
   constexpr int MB_STEP = CR == 8 ? 4 * HCW : 4;          // token distance between the halves of a block
   static_assert(CR == 8 || NCGMAX % 2 == 0, "4-row chunks pair column groups");
+  // Row sums: one extra MFMA against a row of ones per block (ONES); the VALU alternative is kept
+  // for experiments.
+  constexpr bool ONES = true;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -98,26 +101,23 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const bool q_ok = (G.r0 + qr_l < G.TR) && (cw + qc_l < G.TC);
   const int rlo = dlt_imax(qr_l, G.WR - G.r0), rhi = dlt_imin(qr_l + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
   const int clo = dlt_imax(qc_l, G.WC - cw), chi = dlt_imin(qc_l + 2 * G.WC, G.TC - 1 - cw + G.WC);
-  float cbias[NCGMAX][4];
-#pragma unroll
-  for (int cg = 0; cg < NCGMAX; cg++)
-#pragma unroll
-    for (int i = 0; i < 4; i++) cbias[cg][i] = (q_ok && 4 * cg + i >= clo && 4 * cg + i <= chi) ? 0.f : -INFINITY;
   // window columns of this wave that hold at least one grid column
   const int wcol_lo = dlt_imax(0, G.WC - cw), wcol_hi = G.TC - 1 - cw + G.WC;
   const bool wave_ok = cw < G.TC;
-
-  // which column groups need the per-element bias at all (wave-uniform)
+  // per-lane column window [clo, clo + cspan] in window coordinates (empty for a query outside the
+  // grid); column groups whose 4 columns are inside every lane's window need no test (wave-uniform)
+  const int cspan = q_ok ? chi - clo : -1;
   bool cg_edge[NCGMAX];
 #pragma unroll
   for (int cg = 0; cg < NCGMAX; cg++)
-    cg_edge[cg] = __builtin_amdgcn_ballot_w64(cbias[cg][0] != 0.f || cbias[cg][1] != 0.f || cbias[cg][2] != 0.f ||
-                                              cbias[cg][3] != 0.f) != 0;
+    cg_edge[cg] = __builtin_amdgcn_ballot_w64(!((unsigned)(4 * cg - clo) <= (unsigned)cspan &&
+                                                (unsigned)(4 * cg + 3 - clo) <= (unsigned)cspan)) != 0;
 
   // running max of the RAW scores (sm_scale > 0 keeps the order), sum in acc_l through an
   // extra MFMA whose A operand is a row of ones: row 0 of the result is sum_k P[k][query]
   float m_run = -INFINITY;
   f32x4 acc[VB], acc_l = {0.f, 0.f, 0.f, 0.f};
+  float l_run = 0.f;  // per-lane partial row sum (only without the ones trick)
 #pragma unroll
   for (int d = 0; d < VB; d++) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float scale = a.scale_log2;
@@ -164,7 +164,10 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
         for (int i = 0; i < 4; i++) { t[kb][i] = s0[i]; t[kb][4 + i] = s1[i]; }
         if (cg_edge[cg0] || cg_edge[cg1]) {
 #pragma unroll
-          for (int i = 0; i < 4; i++) { t[kb][i] += cbias[cg0][i]; t[kb][4 + i] += cbias[cg1][i]; }
+          for (int i = 0; i < 4; i++) {
+            t[kb][i] = (unsigned)(4 * cg0 + i - clo) <= (unsigned)cspan ? t[kb][i] : -INFINITY;
+            t[kb][4 + i] = (unsigned)(4 * cg1 + i - clo) <= (unsigned)cspan ? t[kb][4 + i] : -INFINITY;
+          }
         }
         if (row_edge) {
 #pragma unroll
@@ -185,16 +188,21 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
     const float neg_m2 = -m_use * scale;
     m_run = m_new;
     u32x4 pb[NKB];
+    float psum = 0.f;
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
-      for (int i = 0; i < 8; i++) t[kb][i] = fast_exp2(fmaf(t[kb][i], scale, neg_m2));
+      for (int i = 0; i < 8; i++) {
+        t[kb][i] = fast_exp2(fmaf(t[kb][i], scale, neg_m2));
+        if (!ONES) psum += t[kb][i];
+      }
       pb[kb] = pack8<CT>(t[kb]);
     }
+    if (!ONES) l_run = l_run * alpha + psum;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
 #pragma unroll
       for (int d = 0; d < VB; d++) acc[d] *= alpha;
-      acc_l *= alpha;
+      if (ONES) acc_l *= alpha;
     }
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++) {
@@ -203,7 +211,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
 #pragma unroll
         for (int d = 0; d < VB; d++)
           acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PITCH, HCW, key0, 16 * d, n, g, MB_STEP), pb[kb], acc[d]);
-        acc_l = Mma<CT>::mfma(ones, pb[kb], acc_l);
+        if (ONES) acc_l = Mma<CT>::mfma(ones, pb[kb], acc_l);
       }
     }
     __syncthreads();  // every wave is done with this chunk
@@ -217,7 +225,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   // ---- epilogue
   typedef typename TileOf<TIO>::type TL;
   constexpr int PO = D * (int)sizeof(TL) + 16;
-  const float lt = __shfl(acc_l[0], n);  // row 0 of the ones product lives in lane group 0
+  // row 0 of the ones product lives in lane group 0; per-lane partial sums are added over the 4 groups
+  const float lt = ONES ? __shfl(acc_l[0], n) : wave_sum4(l_run);
   const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
   TL* orow = reinterpret_cast<TL*>(smem + (16 * wave + n) * PO);
 #pragma unroll
