@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
 
 One "step" is one forward + backward pass of the fused RoPE-2D + tiled 2D sliding-window
-attention over one synthetic batch of BASELINE config 3 (bf16, B=2, H=8, 64x64 token grid,
+attention over one synthetic batch of benchmark config 3 (bf16, B=2, H=8, 64x64 token grid,
 d=64, 13x13 window), inputs resident in HBM.  `value` is the effective TFLOP/s of that
 step (in-window FLOPs only: fwd 2*pairs*(dk+dv), bwd 2*pairs*(3dk+2dv)).  The JSON line also
 carries the roofline of the dominant kernel (per-kernel HIP-event durations taken inside the
@@ -117,13 +117,13 @@ def try_graph(wl, steps, warmup):
 
 # ------------------------------------------------------------------------------------------ SWA
 class SwaWorkload:
-    def __init__(self, name, B, H, th, tw, W, d, fused_rope, nsets, seed=0, dtype=torch.bfloat16):
+    def __init__(self, name, B, H, th, tw, W, d, fused_rope, nsets, seed=0, dtype=torch.bfloat16, b_size=1, scale=None):
         from dl_templates_amd import _lib, tiled_swa
         from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
         from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as Rope
         self.name, self.B, self.H, self.th, self.tw, self.W, self.d = name, B, H, th, tw, W, d
         dev = torch.device("cuda:0")
-        N = th * tw
+        N = th * tw * b_size
         self.sets = []
         for i in range(nsets):
             q, k, v, do = make_inputs(seed + i, B, H, N, N, d, d, dtype, dev)
@@ -132,7 +132,8 @@ class SwaWorkload:
             delta = torch.empty_like(lse)
             dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
             self.sets.append((q, k, v, do, o, lse, delta, dq, dk, dv))
-        self.shape = _lib.SwaShape(B, H, 1, th, tw, W, W, d, d, 1.0 / math.sqrt(d), _lib.dtype_code(self.sets[0][0]))
+        self.shape = _lib.SwaShape(B, H, b_size, th, tw, W, W, d, d, scale if scale is not None else 1.0 / math.sqrt(d),
+                                   _lib.dtype_code(self.sets[0][0]))
         self.rope = None
         if fused_rope:
             g = torch.Generator().manual_seed(seed + 1000)
@@ -147,7 +148,7 @@ class SwaWorkload:
         self.stream = _lib.stream_of(self.sets[0][0])
         self.calls = [self._build_calls(s) for s in self.sets]
         self.i = 0
-        self.pairs = swa_pairs(B, H, 1, th, tw, W, W)
+        self.pairs = swa_pairs(B, H, b_size, th, tw, W, W)
         self.flops_fwd = 2 * self.pairs * (d + d)
         self.flops_bwd = 2 * self.pairs * (3 * d + 2 * d)
 
@@ -294,6 +295,23 @@ def calibration_copy():
     torch.cuda.synchronize()
 
 
+def copy_bandwidth():
+    """What the memory system sustains for a plain copy (read + write bytes per second): 64 MiB
+    (resident in the 256 MB infinity cache after the first pass) and 1 GiB (HBM)."""
+    from dl_templates_amd import _lib
+    lib = _lib.load()
+    out = {}
+    for name, nbytes, reps in (("64MiB_cache_resident", 64 << 20, 20), ("1GiB_hbm", 1 << 30, 5)):
+        a = torch.empty(nbytes, dtype=torch.uint8, device="cuda:0")
+        b = torch.empty_like(a)
+        st = _lib.stream_of(a)
+        fn = lambda: _lib.check(lib.dlt_debug_copy(_lib.ptr(b), _lib.ptr(a), nbytes, st))
+        ms, _ = Timer.run(fn, reps, 2)
+        out[name] = {"ms": ms, "gbps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9}
+        del a, b
+    return out
+
+
 def recorded_traffic(kernel):
     """HBM bytes per launch of `kernel` on the C3 workload as recorded under profiles/ (two
     rocprofv3 --pmc runs of this script, scaled by the calibration copy); None if absent."""
@@ -352,6 +370,7 @@ def main():
 
     rope = bench_rope(K, W)
     extra["rope2d_c2"] = rope
+    extra["copy_bandwidth"] = copy_bandwidth()
 
     if not args.quick:
         for name, (B, H, th, tw, Wn, d) in {"C4_128x128": (1, 16, 128, 128, 10, 128), "C4_96x160": (1, 16, 96, 160, 10, 128)}.items():
@@ -363,6 +382,13 @@ def main():
                            "frac_mfma_peak": f4 / (ms4 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
                            "kernels_ms": {k_: v_["avg_ms"] for k_, v_ in kb4.items()}}
             del w4
+        # the reference's own demo shape (src/tiled_swa.py:736-750): 16-token tiles, generic kernels
+        wd = SwaWorkload("ref_demo", 4, 8, 16, 16, 1, 32, fused_rope=False, nsets=1, dtype=torch.float16, b_size=16, scale=0.25)
+        msd, _ = Timer.run(wd.step, max(K // 5, 3), 2)
+        fd = wd.flops_fwd + wd.flops_bwd
+        extra["ref_demo_b16"] = {"ms_per_step": msd, "eff_tflops": fd / (msd * 1e-3) / 1e12,
+                                 "workload": "B=4 H=8 16x16 tiles of 16 tokens, d=32, 3x3 window, fp16, fwd+bwd"}
+        del wd
         w5 = FlashWorkload(2, 16, 4096, 8192, 64, 128)
         ms5, _ = Timer.run(w5.step, max(K // 5, 3), 2)
         kb5 = kernel_breakdown(w5.step, 3)

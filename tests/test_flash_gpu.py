@@ -3,7 +3,7 @@
 Follows the reference's own check (src/flash_attn.py:616-659: q, k L2-normalised, loss =
 o.sum(), allclose(1e-2, 1e-2) on o, dq, dk, dv, Z=4, H in {4,8}, N in {512,2048},
 dv in {16,32}, dk in {16,64}) with seeded inputs, plus Lq != Lk, odd lengths, bf16 and the
-BASELINE tolerances (forward max-abs <= 2e-2, gradients relative <= 5e-2).
+stated tolerances (forward max-abs <= 2e-2, gradients relative <= 5e-2).
 """
 import itertools
 import math
@@ -68,7 +68,7 @@ def test_cross_attention_distinct_dims_and_lengths(Lq, Lk, dk, dv, dtype):
 
 
 def test_c5_shape_reduced_batch():
-    # BASELINE config 5 shape with B=1, H=2 (CPU oracle time): Lq=4096, Lk=8192, 64/128
+    # benchmark config 5 shape with B=1, H=2 (CPU oracle time): Lq=4096, Lk=8192, 64/128
     q, k, v, do = orc.make_qkv(55, 1, 2, 4096, 8192, 64, 128, torch.bfloat16)
     o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), False, 0.125)
     qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))

@@ -1,4 +1,4 @@
-"""Parity at BASELINE's full sizes, where the CPU oracle would take minutes: size-independent
+"""Parity at the benchmark's full sizes, where the CPU oracle would take minutes: size-independent
 properties and a cross-check between two independent GPU implementations.
 
 * config 4 (B=1, H=16, 128x128 and 96x160 grids, d=128, 21x21 window): the token-grid kernels

@@ -98,7 +98,7 @@ def test_swa_tile_tokens_share_neighbour_set():
 
 
 def test_c1_golden_fixture():
-    # BASELINE config 1: B=1, H=2, 16x16, d=32, 7x7 window, fp32, scale 1/sqrt(32)
+    # benchmark config 1: B=1, H=2, 16x16, d=32, 7x7 window, fp32, scale 1/sqrt(32)
     f = np.load(os.path.join(GOLDEN, "c1_swa_fwd.npz"))
     q, k, v, _ = orc.make_qkv(int(f["seed"]), 1, 2, 256, 256, 32, 32)
     assert np.array_equal(q.numpy(), f["q"]) and np.array_equal(v.numpy(), f["v"])

@@ -75,7 +75,7 @@ def test_pe_mask_bit_exact():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_c2_shape(dtype):
-    # BASELINE config 2: B=4, H=8, 64x64 grid, d=64, first 32 dims rotated, 5% no-PE
+    # benchmark config 2: B=4, H=8, 64x64 grid, d=64, first 32 dims rotated, 5% no-PE
     torch.manual_seed(0)
     x = torch.randn(32, 4096, 64).to(dtype)
     idx = orc.make_rope_idx(11, 64, 64, 0.05)

@@ -67,7 +67,7 @@ def test_head_dims(dk, dv):
 
 
 def test_c3_shape_unfused_one_batch():
-    # BASELINE config 3 shape with B=1 (CPU oracle time), 64x64, d=64, 13x13
+    # benchmark config 3 shape with B=1 (CPU oracle time), 64x64, d=64, 13x13
     errs = _run(6, 1, 8, 1, 64, 64, 6, 6, 64, 64, torch.bfloat16)
     print("c3 rel errs", errs)
 

@@ -39,7 +39,7 @@ def _run(seed, B, H, b_size, th, tw, wr, wc, dk, dv, dtype, scale=None, check_ls
 
 
 def test_c1_tiny_fp32_and_golden():
-    # BASELINE config 1 + the committed fixture
+    # benchmark config 1 + the committed fixture
     import os
     f = np.load(os.path.join(os.path.dirname(__file__), "golden", "c1_swa_fwd.npz"))
     q, k, v, _ = orc.make_qkv(int(f["seed"]), 1, 2, 256, 256, 32, 32)
@@ -68,7 +68,7 @@ def test_head_dims(dk, dv):
 
 
 def test_c3_shape_fwd():
-    # BASELINE config 3 shape (unfused): B=2, H=8, 64x64, d=64, 13x13
+    # benchmark config 3 shape (unfused): B=2, H=8, 64x64, d=64, 13x13
     err = _run(5, 2, 8, 1, 64, 64, 6, 6, 64, 64, torch.bfloat16)
     print("c3 fwd max abs err", err)
 
