@@ -148,13 +148,13 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
 
   Swa1BwdArgs a;
   a.p = p;
-  // the dQ kernel streams 4-row chunks, the dK/dV kernel 8-row chunks; HRP (a multiple of 8 here)
-  // serves both
+  // chunk heights of the two kernels may differ; the plan fields the kernels read (ncg, block
+  // counts) do not depend on it
   Swa1Plan plan_q;
   swa1_make_plan(p, c, 2, 0, plan_q, SWA1_FWD_CR);
-  swa1_make_plan(p, c, 2, 0, a.plan);
   const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
-  const int lds_q = plan_q.lds_bytes, lds_kv = a.plan.lds_bytes + 2 * 8 * hcw * 4;
+  swa1_make_plan(p, c, 2, 2 * SWA1_KV_CR * hcw * 4, a.plan, SWA1_KV_CR);
+  const int lds_q = plan_q.lds_bytes, lds_kv = a.plan.lds_bytes;
   a.q = t.q; a.k = t.k; a.v = t.v; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
   a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
   for (int i = 0; i < 4; i++) {

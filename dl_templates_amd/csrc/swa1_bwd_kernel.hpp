@@ -4,7 +4,7 @@
 // fewer than 16 tokens (src/tiled_swa.py:660-661).
 //
 //   dK/dV: a wave owns a 4x4 patch of keys; the queries that can see them (their halo, by the
-//          symmetry of the window) stream through LDS in chunks of 8 rows: Q (rotated when
+//          symmetry of the window) stream through LDS in chunks of CR rows: Q (rotated when
 //          the rotary encoding is fused), dO, lse2 and delta.
 //   dQ   : a wave owns a 4x4 patch of queries; K (rotated) and V stream through LDS.
 // Both recompute P = exp2(s * scale - lse2) per block; tokens of the streamed side are the MFMA
@@ -24,17 +24,17 @@ struct Swa1BwdArgs {
   float scale_log2;
 };
 
-// per-token fp32 values (lse2 / delta) of halo rows [cr0, cr0 + 8): 8 * HCW values over 256 threads
-template <int HCW>
-struct ScalarRegs { float v[(8 * HCW + 255) / 256]; };
+// per-token fp32 values (lse2 / delta) of halo rows [cr0, cr0 + CR): CR * HCW values over 256 threads
+template <int HCW, int CR>
+struct ScalarRegs { float v[(CR * HCW + 255) / 256]; };
 
-template <int HCW>
-DLT_DEV void swa1_issue_scalar(ScalarRegs<HCW>& sr, const float* base, int64_t stride, const Swa1Geom& G, int cr0, int tid) {
+template <int HCW, int CR>
+DLT_DEV void swa1_issue_scalar(ScalarRegs<HCW, CR>& sr, const float* base, int64_t stride, const Swa1Geom& G, int cr0, int tid) {
 #pragma unroll
-  for (int it = 0; it < (8 * HCW + 255) / 256; it++) {
+  for (int it = 0; it < (CR * HCW + 255) / 256; it++) {
     const int idx = tid + 256 * it;
     sr.v[it] = 0.f;
-    if (idx < 8 * HCW) {
+    if (idx < CR * HCW) {
       // clamped like the tile staging: out-of-grid halo positions are masked by the window bias
       const int hr = idx / HCW, hc = idx - hr * HCW;
       const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + cr0 + hr, G.TR - 1));
@@ -44,12 +44,12 @@ DLT_DEV void swa1_issue_scalar(ScalarRegs<HCW>& sr, const float* base, int64_t s
   }
 }
 
-template <int HCW>
-DLT_DEV void swa1_commit_scalar(const ScalarRegs<HCW>& sr, float* s, int tid) {
+template <int HCW, int CR>
+DLT_DEV void swa1_commit_scalar(const ScalarRegs<HCW, CR>& sr, float* s, int tid) {
 #pragma unroll
-  for (int it = 0; it < (8 * HCW + 255) / 256; it++) {
+  for (int it = 0; it < (CR * HCW + 255) / 256; it++) {
     const int idx = tid + 256 * it;
-    if (idx < 8 * HCW) s[idx] = sr.v[it];
+    if (idx < CR * HCW) s[idx] = sr.v[it];
   }
 }
 
@@ -59,7 +59,7 @@ struct Swa1Lane {
   Swa1Geom G;
   int b, h;
   int rlo, rhi;
-  float cbias[NCGMAX][4];
+  int clo, cspan;  // column window [clo, clo + cspan] of this lane's own token (cspan < 0: none)
   bool cg_edge[NCGMAX];
   int wcol_lo, wcol_hi;
   bool wave_ok;
@@ -80,14 +80,14 @@ struct Swa1Lane {
     const bool q_ok = (G.r0 + qr_l < G.TR) && (cw + qc_l < G.TC);
     rlo = dlt_imax(qr_l, G.WR - G.r0);
     rhi = dlt_imin(qr_l + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
-    const int clo = dlt_imax(qc_l, G.WC - cw), chi = dlt_imin(qc_l + 2 * G.WC, G.TC - 1 - cw + G.WC);
+    clo = dlt_imax(qc_l, G.WC - cw);
+    const int chi = dlt_imin(qc_l + 2 * G.WC, G.TC - 1 - cw + G.WC);
+    cspan = q_ok ? chi - clo : -1;
+    // column groups whose 4 columns lie inside every lane's window need no test (wave-uniform flag)
 #pragma unroll
-    for (int cg = 0; cg < NCGMAX; cg++) {
-#pragma unroll
-      for (int i = 0; i < 4; i++) cbias[cg][i] = (q_ok && 4 * cg + i >= clo && 4 * cg + i <= chi) ? 0.f : -INFINITY;
-      cg_edge[cg] = __builtin_amdgcn_ballot_w64(cbias[cg][0] != 0.f || cbias[cg][1] != 0.f || cbias[cg][2] != 0.f ||
-                                                cbias[cg][3] != 0.f) != 0;
-    }
+    for (int cg = 0; cg < NCGMAX; cg++)
+      cg_edge[cg] = __builtin_amdgcn_ballot_w64(!((unsigned)(4 * cg - clo) <= (unsigned)cspan &&
+                                                  (unsigned)(4 * cg + 3 - clo) <= (unsigned)cspan)) != 0;
     wcol_lo = dlt_imax(0, G.WC - cw);
     wcol_hi = G.TC - 1 - cw + G.WC;
     wave_ok = cw < G.TC;
@@ -99,6 +99,8 @@ struct Swa1Lane {
     const int r = G.r0 + ((row & 15) >> 2), c = G.c0 + 4 * (row >> 4) + (row & 3);
     return (r < G.TR && c < G.TC) ? (int64_t)r * G.TC + c : (int64_t)-1;
   }
+  // window column 4 * cg + i visible from this lane's own token
+  DLT_DEV bool col_ok(int cg, int i) const { return (unsigned)(4 * cg + i - clo) <= (unsigned)cspan; }
   DLT_DEV bool block_on(const Swa1Plan& P, int cg) const {
     return wave_ok && cg < P.ncg && 4 * cg <= wcol_hi && 4 * cg + 3 >= wcol_lo;
   }
@@ -121,14 +123,16 @@ DLT_DEV void swa1_write_grad(char* sT, f32x4 (&acc)[D / 16], float mul, TIO* bas
 }
 
 // =============================================================================================
-template <typename TIO, int D, int NCGMAX>
-__global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
+template <typename TIO, int D, int NCGMAX, int CR>
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr int PITCH = D * 2 + SWA1_PAD;
   constexpr int KC = D / 32, DB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
-  constexpr int REGION = 8 * HCW * PITCH;
+  constexpr int REGION = CR * HCW * PITCH;
+  constexpr int NKB = CR == 8 ? NCGMAX : NCGMAX / 2;
+  constexpr int MB_STEP = CR == 8 ? 4 * HCW : 4;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -137,10 +141,10 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
   char* sQ = smem;
   char* sDO = smem + REGION;
   float* sLse = reinterpret_cast<float*>(smem + 2 * REGION);
-  float* sDel = sLse + 8 * HCW;
+  float* sDel = sLse + CR * HCW;
 
   Swa1Lane<NCGMAX> L;
-  L.init(a.p, P, wave, n);
+  L.init(a.p, P, wave, n, CR);
   const Swa1Geom& G = L.G;
   const int b = L.b, h = L.h;
 
@@ -157,19 +161,19 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  constexpr int NI = swa1_items(D, HCW);
+  constexpr int NI = swa1_items(D, HCW, CR);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW>(sp, G, PITCH, tid);
+  swa1_plan_init<D, HCW, CR>(sp, G, PITCH, tid);
   const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
   const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
   StageRegs<NI> srq, srd;
   swa1_regs_zero(srq);
   swa1_regs_zero(srd);
-  swa1_issue(srq, sp, on_k, qb, sn2q, G, 8 * L.ch_first, rope_idx);
-  swa1_issue(srd, sp, on_v, dob, sn2d, G, 8 * L.ch_first, nullptr);
-  ScalarRegs<HCW> r_lse, r_del;
-  swa1_issue_scalar<HCW>(r_lse, lseb, a.ls[2], G, 8 * L.ch_first, tid);
-  swa1_issue_scalar<HCW>(r_del, delb, a.ls[2], G, 8 * L.ch_first, tid);
+  swa1_issue(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx);
+  swa1_issue(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr);
+  ScalarRegs<HCW, CR> r_lse, r_del;
+  swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, CR * L.ch_first, tid);
+  swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, CR * L.ch_first, tid);
 
   // own keys / values straight into B-operand fragments
   u32x4 kf[KC], vf[KC];
@@ -186,29 +190,30 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
 
   swa1_commit<CT>(srq, sp, sQ, a.rope_pbit, fwd_rope, use_rope && on_k);
   swa1_commit<CT>(srd, sp, sDO, 1, no_rope, false);
-  swa1_commit_scalar<HCW>(r_lse, sLse, tid);
-  swa1_commit_scalar<HCW>(r_del, sDel, tid);
+  swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
+  swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
   __syncthreads();
 
   for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
-    const int cr0 = 8 * ch;
+    const int cr0 = CR * ch;
     if (ch < L.ch_last) {
-      swa1_issue(srq, sp, on_k, qb, sn2q, G, cr0 + 8, rope_idx);
-      swa1_issue(srd, sp, on_v, dob, sn2d, G, cr0 + 8, nullptr);
-      swa1_issue_scalar<HCW>(r_lse, lseb, a.ls[2], G, cr0 + 8, tid);
-      swa1_issue_scalar<HCW>(r_del, delb, a.ls[2], G, cr0 + 8, tid);
+      swa1_issue(srq, sp, on_k, qb, sn2q, G, cr0 + CR, rope_idx);
+      swa1_issue(srd, sp, on_v, dob, sn2d, G, cr0 + CR, nullptr);
+      swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, cr0 + CR, tid);
+      swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, cr0 + CR, tid);
     }
     float rbias[2];
 #pragma unroll
     for (int mb = 0; mb < 2; mb++) {
-      const int hrow = cr0 + 4 * mb + g;
+      const int hrow = cr0 + (CR == 8 ? 4 * mb : 0) + g;
       rbias[mb] = (hrow >= L.rlo && hrow <= L.rhi) ? 0.f : -INFINITY;
     }
 #pragma unroll
-    for (int cg = 0; cg < NCGMAX; cg++) {
-      if (!L.block_on(P, cg)) continue;
-      const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg + (n & 3);   // A-operand row of this lane
-      const int tok0 = g * HCW + 4 * wave + 4 * cg;                     // first of the 4 result columns
+    for (int kb = 0; kb < NKB; kb++) {
+      const int cg0 = CR == 8 ? kb : 2 * kb, cg1 = CR == 8 ? kb : 2 * kb + 1;
+      if (!(L.wave_ok && cg0 < P.ncg && 4 * cg0 <= L.wcol_hi && 4 * cg1 + 3 >= L.wcol_lo)) continue;
+      const int key0 = (n >> 2) * HCW + 4 * wave + 4 * cg0 + (n & 3);  // A-operand row of this lane
+      const int tok0 = g * HCW + 4 * wave + 4 * cg0;                    // first of the 4 result columns
       f32x4 s[2], dp[2];
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
@@ -216,37 +221,39 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
         dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KC; c++) {
-          s[mb] = Mma<CT>::mfma(lds_read16(sQ + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), kf[c], s[mb]);
-          dp[mb] = Mma<CT>::mfma(lds_read16(sDO + (key0 + 4 * mb * HCW) * PITCH + (32 * c + 8 * g) * 2), vf[c], dp[mb]);
+          s[mb] = Mma<CT>::mfma(lds_read16(sQ + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), kf[c], s[mb]);
+          dp[mb] = Mma<CT>::mfma(lds_read16(sDO + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), vf[c], dp[mb]);
         }
       }
       float pr[8], ds[8];
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
-        const f32x4 lq = *reinterpret_cast<const f32x4*>(sLse + tok0 + 4 * mb * HCW);
-        const f32x4 dq_ = *reinterpret_cast<const f32x4*>(sDel + tok0 + 4 * mb * HCW);
+        const f32x4 lq = *reinterpret_cast<const f32x4*>(sLse + tok0 + mb * MB_STEP);
+        const f32x4 dq_ = *reinterpret_cast<const f32x4*>(sDel + tok0 + mb * MB_STEP);
+        const int cg = mb == 0 ? cg0 : cg1;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const float nl = (L.cbias[cg][i] + rbias[mb]) - lq[i];
+          float nl = rbias[mb] - lq[i];
+          if (L.cg_edge[cg]) nl = L.col_ok(cg, i) ? nl : -INFINITY;
           const float pv = fast_exp2(fmaf(s[mb][i], scale, nl));
           pr[4 * mb + i] = pv;
           ds[4 * mb + i] = pv * (dp[mb][i] - dq_[i]);
         }
       }
       const u32x4 pb = pack8<CT>(pr), dsb = pack8<CT>(ds);
-      const int kt0 = 4 * wave + 4 * cg;
+      const int kt0 = 4 * wave + 4 * cg0;
 #pragma unroll
       for (int d = 0; d < DB; d++) {
-        dv_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sDO, PITCH, HCW, kt0, 16 * d, n, g, 4 * HCW), pb, dv_acc[d]);
-        dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PITCH, HCW, kt0, 16 * d, n, g, 4 * HCW), dsb, dk_acc[d]);
+        dv_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sDO, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), pb, dv_acc[d]);
+        dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dk_acc[d]);
       }
     }
     __syncthreads();
     if (ch < L.ch_last) {
       swa1_commit<CT>(srq, sp, sQ, a.rope_pbit, fwd_rope, use_rope && on_k);
       swa1_commit<CT>(srd, sp, sDO, 1, no_rope, false);
-      swa1_commit_scalar<HCW>(r_lse, sLse, tid);
-  swa1_commit_scalar<HCW>(r_del, sDel, tid);
+      swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
+      swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
       __syncthreads();
     }
   }
@@ -259,7 +266,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? 2 : 1)) void swa1_bwd_kv_kernel(con
 
 // =============================================================================================
 template <typename TIO, int D, int NCGMAX, int CR>
-__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr int PITCH = D * 2 + SWA1_PAD;
@@ -354,7 +361,10 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
       for (int mb = 0; mb < 2; mb++)
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const float pv = fast_exp2(fmaf(s[mb][i], scale, L.cbias[mb == 0 ? cg0 : cg1][i] + rbias[mb]));
+          const int cg = mb == 0 ? cg0 : cg1;
+          float nl = rbias[mb];
+          if (L.cg_edge[cg]) nl = L.col_ok(cg, i) ? nl : -INFINITY;
+          const float pv = fast_exp2(fmaf(s[mb][i], scale, nl));
           ds[4 * mb + i] = pv * (dp[mb][i] - del_n);
         }
       const u32x4 dsb = pack8<CT>(ds);

@@ -12,7 +12,10 @@
 #include "swa1_common.hpp"
 
 #ifndef SWA1_FWD_CR
-#define SWA1_FWD_CR 4  // halo rows per chunk in the forward kernel
+#define SWA1_FWD_CR 4  // halo rows per chunk in the forward and dQ kernels
+#endif
+#ifndef SWA1_KV_CR
+#define SWA1_KV_CR 4   // halo rows per chunk in the dK/dV kernel
 #endif
 
 struct Swa1FwdArgs {
@@ -30,7 +33,7 @@ struct Swa1FwdArgs {
 // CR: halo rows per chunk.  8: a 32-token block is 8 rows x 4 columns; 4: 4 rows x 8 columns
 // (half the LDS and staging registers per workgroup, hence more resident workgroups per CU).
 template <typename TIO, int D, int NCGMAX, int CR>
-__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_fwd_kernel(const Swa1FwdArgs a) {
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 2) : (CR == 4 ? 2 : 1))) void swa1_fwd_kernel(const Swa1FwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr int PITCH = D * 2 + SWA1_PAD;

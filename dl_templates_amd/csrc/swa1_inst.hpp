@@ -30,7 +30,7 @@ int swa1_launch_fwd_t(const Swa1FwdArgs& a, int grid, hipStream_t stream) {
 template <typename TIO, int NCGMAX>
 int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hipStream_t stream) {
   {
-    auto kern = swa1_bwd_kv_kernel<TIO, DLT_D, NCGMAX>;
+    auto kern = swa1_bwd_kv_kernel<TIO, DLT_D, NCGMAX, SWA1_KV_CR>;
     int rc = swa1_set_lds(kern, lds_kv);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_KV, stream);

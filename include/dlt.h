@@ -5,8 +5,10 @@
  *   - returns DLT_OK (0) or a DLT_ERR_* code; dlt_last_error() gives the message of the
  *     last failing call made by the calling thread (thread-local, never NULL);
  *   - every data pointer is a DEVICE pointer owned by the caller; the library allocates
- *     no device memory, never synchronises and keeps no state between calls, so calls
- *     are re-entrant (forward on the caller thread, backward on the autograd thread);
+ *     no device memory, never synchronises and keeps no state between calls (the optional
+ *     timing facility below is the one exception: a thread-local list of host-side event
+ *     handles), so calls are re-entrant (forward on the caller thread, backward on the
+ *     autograd thread);
  *   - strides are in ELEMENTS (int64), tensors are [B, H, N, D] unless said otherwise;
  *   - `stream` is a hipStream_t (NULL = the default stream); work is only enqueued;
  *   - arguments are validated on the host before anything is launched: a call that
