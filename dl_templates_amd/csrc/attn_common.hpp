@@ -41,9 +41,13 @@ template <> struct Mma<f16_t> {
   }
 };
 
+// two floats -> one dword of two 16-bit values (round to nearest even), converted as a vector so
+// that the compiler emits a single packed conversion
 template <typename CT> DLT_DEV unsigned int pack2(float lo, float hi) {
-  CT a = (CT)lo, b = (CT)hi;
-  return (unsigned int)__builtin_bit_cast(unsigned short, a) | ((unsigned int)__builtin_bit_cast(unsigned short, b) << 16);
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef CT ctx2 __attribute__((ext_vector_type(2)));
+  const f32x2 v = {lo, hi};
+  return __builtin_bit_cast(unsigned int, __builtin_convertvector(v, ctx2));
 }
 template <typename CT> DLT_DEV float unpack_lo(unsigned int w) {
   return (float)__builtin_bit_cast(CT, (unsigned short)(w & 0xffffu));

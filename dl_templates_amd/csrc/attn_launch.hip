@@ -134,7 +134,9 @@ bool swa1_strides_fit(const AttnTensors& t) {
 
 int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c, hipStream_t stream) {
   const int es = dlt_elem_size(p.dtype);
-  // delta pre-pass (shared with the generic path)
+  // delta = rowsum(o * dO): folded into the dQ kernel when o can be read in 16-byte pieces like the
+  // other operands, else the pre-pass kernel shared with the generic path
+  const bool fuse_delta = vec_ok(t.o, t.os, 4, p.dv, es) && t.os[2] < ((int64_t)1 << 20);
   BwdArgs d;
   d.p = p;
   d.o = t.o; d.d_o = t.d_o; d.delta = t.delta;
@@ -143,8 +145,10 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
   d.o_vec = vec_ok(t.o, t.os, 4, p.dv, es);
   d.do_vec = vec_ok(t.d_o, t.dos, 4, p.dv, es);
   d.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
-  int rc = c.D == 64 ? dlt_launch_delta_64_64(d, stream) : dlt_launch_delta_128_128(d, stream);
-  if (rc != DLT_OK) return rc;
+  if (!fuse_delta) {
+    int rc = c.D == 64 ? dlt_launch_delta_64_64(d, stream) : dlt_launch_delta_128_128(d, stream);
+    if (rc != DLT_OK) return rc;
+  }
 
   Swa1BwdArgs a;
   a.p = p;
@@ -155,10 +159,12 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
   const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
   swa1_make_plan(p, c, 2, 2 * SWA1_KV_CR * hcw * 4, a.plan, SWA1_KV_CR);
   const int lds_q = plan_q.lds_bytes, lds_kv = a.plan.lds_bytes;
-  a.q = t.q; a.k = t.k; a.v = t.v; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.o; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.delta_out = t.delta;
+  a.fuse_delta = fuse_delta ? 1 : 0;
   a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
   for (int i = 0; i < 4; i++) {
-    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.dos[i] = t.dos[i];
+    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; a.dos[i] = t.dos[i];
     a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
   }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];

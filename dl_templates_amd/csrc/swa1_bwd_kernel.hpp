@@ -6,7 +6,10 @@
 //   dK/dV: a wave owns a 4x4 patch of keys; the queries that can see them (their halo, by the
 //          symmetry of the window) stream through LDS in chunks of CR rows: Q (rotated when
 //          the rotary encoding is fused), dO, lse2 and delta.
-//   dQ   : a wave owns a 4x4 patch of queries; K (rotated) and V stream through LDS.
+//   dQ   : a wave owns a 4x4 patch of queries; K (rotated) and V stream through LDS.  It runs
+//          first and can compute delta = rowsum(o * dO) of its own queries on the way (the
+//          reference's separate pre-pass, src/tiled_swa.py:253-282), which the dK/dV kernel
+//          launched after it reads back.
 // Both recompute P = exp2(s * scale - lse2) per block; tokens of the streamed side are the MFMA
 // rows, so P / dS leave the first products in the layout the second products take as B operand.
 #pragma once
@@ -15,10 +18,12 @@
 struct Swa1BwdArgs {
   AttnProblem p;
   Swa1Plan plan;
-  const void *q, *k, *v, *d_o;
+  const void *q, *k, *v, *o, *d_o;
   const float *lse, *delta;
+  float* delta_out;   // fuse_delta: the dQ kernel computes delta = rowsum(o * dO) of its own tokens and stores it here
   void *dq, *dk, *dv;
-  int64_t qs[4], ks[4], vs[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int32_t fuse_delta;
   int32_t q_vec, k_vec, v_vec, do_vec, dq_vec, dk_vec, dv_vec;
   int32_t rope_pbit;
   float scale_log2;
@@ -260,6 +265,12 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
 
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
+  if (a.dk_vec != 0 && a.dv_vec != 0) {  // the loop ended with a workgroup barrier: the chunk buffers are free
+    char* sW = smem + wave * 16 * (D * 2 + 16);
+    swa1_store_own<TIO, CT, D>(sW, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.p.dk, G, wave, lane, inv_rope, use_rope);
+    swa1_store_own<TIO, CT, D>(sW, dv_acc, 1.0f, dvb, a.dvs[2], a.p.dv, G, wave, lane, no_rope, false);
+    return;
+  }
   swa1_write_grad<TIO, D>(smem, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.dks[3], a.p.dk, a.dk_vec != 0, L, inv_rope, wave, n, g, tid);
   swa1_write_grad<TIO, D>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.p.dv, a.dv_vec != 0, L, no_rope, wave, n, g, tid);
 }
@@ -317,7 +328,26 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   swa1_load_own<TIO, CT, D>(dof, dob, a.dos[2], a.p.dv, tq, g, no_rope, false);
   const int64_t loff = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
   const float lse_n = tq >= 0 ? a.lse[loff] : 0.f;
-  const float del_n = tq >= 0 ? a.delta[loff] : 0.f;
+  float del_n;
+  if (a.fuse_delta != 0) {
+    // delta of the own tokens, computed here and published for the dK/dV kernel that runs next
+    const TIO* ob = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1];
+    u32x4 of[KC];
+    swa1_load_own<TIO, CT, D>(of, ob, a.os[2], a.p.dv, tq, g, no_rope, false);
+    float part = 0.f;
+#pragma unroll
+    for (int c = 0; c < KC; c++) {
+      float fo[8], fd[8];
+      unpack8<CT>(of[c], fo);
+      unpack8<CT>(dof[c], fd);
+#pragma unroll
+      for (int j = 0; j < 8; j++) part += fo[j] * fd[j];
+    }
+    del_n = wave_sum4(part);
+    if (g == 0 && tq >= 0) a.delta_out[loff] = del_n;
+  } else {
+    del_n = tq >= 0 ? a.delta[loff] : 0.f;
+  }
 
   f32x4 dq_acc[DB];
 #pragma unroll
@@ -382,5 +412,10 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   }
 
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
+  if (a.dq_vec != 0) {
+    swa1_store_own<TIO, CT, D>(smem + wave * 16 * (D * 2 + 16), dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.p.dk, G, wave, lane,
+                               inv_rope, use_rope);
+    return;
+  }
   swa1_write_grad<TIO, D>(smem, dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.dqs[3], a.p.dk, a.dq_vec != 0, L, inv_rope, wave, n, g, tid);
 }

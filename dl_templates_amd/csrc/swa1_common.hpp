@@ -192,3 +192,50 @@ DLT_DEV u32x4 swa1_read_tokens_as_k(const char* tile, int pitch, int hcw, int ke
   r.x = lo.x; r.y = lo.y; r.z = hi.x; r.w = hi.y;
   return r;
 }
+
+// Epilogue: accumulators in C layout (lane (n, g) holds dims 16 d + 4 g .. +3 of own token n,
+// scaled by `mul`) -> wave-private LDS tile [16 tokens][D] of output elements -> 16-byte pieces
+// -> HBM rows (element stride 1, 16-byte aligned rows).  A wave reads back only what it wrote
+// itself, so no workgroup barrier is involved; LDS operations of one wave execute in order.
+// With `use_rope` the rotation selected by rope.inverse is applied to the rounded values, exactly
+// as the standalone operator would see them.
+template <typename TIO, typename CT, int D>
+DLT_DEV void swa1_store_own(char* sW, const f32x4 (&acc)[D / 16], float mul, TIO* base, int64_t sn, int dact,
+                            const Swa1Geom& G, int wave, int lane, const RopeDev& rope, bool use_rope) {
+  constexpr int PT = D * 2 + 16, CH = D / 8;
+  const int n = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int d = 0; d < D / 16; d++) {
+    u32x2 w;
+    w.x = pack2<CT>(acc[d][0] * mul, acc[d][1] * mul);
+    w.y = pack2<CT>(acc[d][2] * mul, acc[d][3] * mul);
+    *reinterpret_cast<u32x2*>(sW + n * PT + (16 * d + 4 * g) * 2) = w;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+  for (int it = 0; it < 16 * CH / 64; it++) {
+    const int p = lane + 64 * it;
+    const int row = p / CH, c = p % CH;
+    const int r = G.r0 + (row >> 2), col = G.c0 + 4 * wave + (row & 3);
+    if (r < G.TR && col < G.TC && 8 * c < dact) {
+      const int tok = r * G.TC + col;
+      const char* lrow = sW + row * PT;
+      u32x4 v = lds_read16(lrow + 16 * c);
+      if (use_rope) {
+        const RopeChunk rc = rope_chunk_setup(rope, c, true);
+        if (rc.mode == 1) {
+          float self[8], partner[8];
+          unpack8<CT>(v, self);
+          unpack8<CT>(lds_read16(lrow + 16 * rc.partner_c), partner);
+          rope_apply8(rope, rc, c, rope.idx[tok], self, partner, [](int) { return 0.f; });
+          v = pack8<CT>(self);
+        }
+      }
+      *reinterpret_cast<u32x4*>(base + (int64_t)tok * sn + 8 * c) = v;
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+}

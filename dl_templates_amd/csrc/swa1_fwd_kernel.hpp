@@ -231,13 +231,17 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   // row 0 of the ones product lives in lane group 0; per-lane partial sums are added over the 4 groups
   const float lt = ONES ? __shfl(acc_l[0], n) : wave_sum4(l_run);
   const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
+  const int64_t tq = own_token(16 * wave + n);
+  if (g == 0 && tq >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq * a.ls[2]] = m_run * scale + fast_log2(lt);
+  if (a.o_vec != 0) {  // the loop ended with a workgroup barrier: the chunk buffers are free
+    swa1_store_own<TIO, CT, D>(smem + wave * 16 * PO, acc, inv, ob, a.os[2], a.p.dv, G, wave, lane, no_rope, false);
+    return;
+  }
   TL* orow = reinterpret_cast<TL*>(smem + (16 * wave + n) * PO);
 #pragma unroll
   for (int d = 0; d < VB; d++)
 #pragma unroll
     for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[d][i] * inv);
-  const int64_t tq = own_token(16 * wave + n);
-  if (g == 0 && tq >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq * a.ls[2]] = m_run * scale + fast_log2(lt);
   __syncthreads();
   store_tile<TIO, TL, D>(smem, PO, ob, a.os[2], a.os[3], a.p.dv, a.o_vec != 0, 64, own_token, no_rope, tid);
 }

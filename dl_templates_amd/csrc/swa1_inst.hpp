@@ -29,15 +29,7 @@ int swa1_launch_fwd_t(const Swa1FwdArgs& a, int grid, hipStream_t stream) {
 
 template <typename TIO, int NCGMAX>
 int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hipStream_t stream) {
-  {
-    auto kern = swa1_bwd_kv_kernel<TIO, DLT_D, NCGMAX, SWA1_KV_CR>;
-    int rc = swa1_set_lds(kern, lds_kv);
-    if (rc != DLT_OK) return rc;
-    dlt_timing_before(DLT_K_BWD_KV, stream);
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_kv, stream, a);
-    dlt_timing_after(stream);
-    DLT_CHECK_LAUNCH("token-grid attention dK/dV launch");
-  }
+  // dQ first: with fuse_delta it produces the delta vector the dK/dV kernel consumes
   {
     auto kern = swa1_bwd_q_kernel<TIO, DLT_D, NCGMAX, SWA1_FWD_CR>;
     int rc = swa1_set_lds(kern, lds_q);
@@ -46,6 +38,15 @@ int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hip
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_q, stream, a);
     dlt_timing_after(stream);
     DLT_CHECK_LAUNCH("token-grid attention dQ launch");
+  }
+  {
+    auto kern = swa1_bwd_kv_kernel<TIO, DLT_D, NCGMAX, SWA1_KV_CR>;
+    int rc = swa1_set_lds(kern, lds_kv);
+    if (rc != DLT_OK) return rc;
+    dlt_timing_before(DLT_K_BWD_KV, stream);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds_kv, stream, a);
+    dlt_timing_after(stream);
+    DLT_CHECK_LAUNCH("token-grid attention dK/dV launch");
   }
   return DLT_OK;
 }
