@@ -86,7 +86,7 @@ int make_plan(const AttnProblem& p, int own, int own_bytes, int per_tok, int XL_
 }
 
 // ---- token-grid (b_size == 1) fast path ----------------------------------------------------
-struct Swa1Class { int D, wclass, pbit; };
+struct Swa1Class { int D, wclass, pbit, rope_mode; };
 
 // Can the token-grid kernels take this problem?  They need 16-byte vector access to the
 // streamed tensors, both head dims in one padded class, a window of at most 21 columns and,
@@ -105,11 +105,15 @@ bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streame
   if (ncg > 6) return false;
   c.wclass = ncg <= 4 ? 0 : 1;
   c.pbit = 1;
+  c.rope_mode = 0;
   if (p.rope.enabled && p.rope.R > 0) {
     const int r8 = p.rope.R / 8;
     if (p.rope.R % 8 != 0 || (r8 & (r8 - 1)) != 0 || 4 * p.rope.R > c.D) return false;
     if ((uintptr_t)p.rope.row_cs % 4 != 0) return false;
     c.pbit = r8;
+    // balanced staging map: the rotation covers exactly half of a fully used head dim, so there
+    // are as many rotary chunk pairs per token as staging threads
+    c.rope_mode = (2 * r8 == c.D / 32 && p.dk == c.D && p.dv == c.D) ? 2 : 1;
   }
   return true;
 }
@@ -173,6 +177,7 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
   a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, es);
   a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, es);
   a.rope_pbit = c.pbit;
+  a.rope_mode = c.rope_mode;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
   if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward: grid too large");
@@ -191,6 +196,7 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
   a.q_vec = vec_ok(t.q, t.qs, 4, p.dk, es);
   a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, es);
   a.rope_pbit = c.pbit;
+  a.rope_mode = c.rope_mode;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
   if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: grid too large");

@@ -24,6 +24,7 @@ struct Swa1BwdArgs {
   void *dq, *dk, *dv;
   int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
   int32_t fuse_delta;
+  int32_t rope_mode;  // 0 none, 1 rotation with the plain staging map, 2 balanced staging map
   int32_t q_vec, k_vec, v_vec, do_vec, dq_vec, dk_vec, dv_vec;
   int32_t rope_pbit;
   float scale_log2;
@@ -128,7 +129,7 @@ DLT_DEV void swa1_write_grad(char* sT, f32x4 (&acc)[D / 16], float mul, TIO* bas
 }
 
 // =============================================================================================
-template <typename TIO, int D, int NCGMAX, int CR>
+template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
@@ -162,20 +163,21 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
-  const bool use_rope = a.p.rope.enabled != 0;
+  constexpr bool use_rope = ROPE != 0;
+  constexpr bool BAL = ROPE == 2;
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
   constexpr int NI = swa1_items(D, HCW, CR);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR>(sp, G, PITCH, tid);
-  const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
+  swa1_plan_init<D, HCW, CR, BAL>(sp, G, PITCH, tid, a.rope_pbit);
+  const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
   StageRegs<NI> srq, srd;
   swa1_regs_zero(srq);
   swa1_regs_zero(srd);
-  swa1_issue(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx);
-  swa1_issue(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr);
+  swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx);
+  swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr);
   ScalarRegs<HCW, CR> r_lse, r_del;
   swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, CR * L.ch_first, tid);
   swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, CR * L.ch_first, tid);
@@ -193,8 +195,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   for (int d = 0; d < DB; d++) { dk_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; dv_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
   const float scale = a.scale_log2;
 
-  swa1_commit<CT>(srq, sp, sQ, a.rope_pbit, fwd_rope, use_rope && on_k);
-  swa1_commit<CT>(srd, sp, sDO, 1, no_rope, false);
+  swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k);
+  swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
   swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
   __syncthreads();
@@ -202,8 +204,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
     const int cr0 = CR * ch;
     if (ch < L.ch_last) {
-      swa1_issue(srq, sp, on_k, qb, sn2q, G, cr0 + CR, rope_idx);
-      swa1_issue(srd, sp, on_v, dob, sn2d, G, cr0 + CR, nullptr);
+      swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, cr0 + CR, rope_idx);
+      swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, cr0 + CR, nullptr);
       swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, cr0 + CR, tid);
       swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, cr0 + CR, tid);
     }
@@ -255,8 +257,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
     }
     __syncthreads();
     if (ch < L.ch_last) {
-      swa1_commit<CT>(srq, sp, sQ, a.rope_pbit, fwd_rope, use_rope && on_k);
-      swa1_commit<CT>(srd, sp, sDO, 1, no_rope, false);
+      swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k);
+      swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
       swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
       swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
       __syncthreads();
@@ -271,12 +273,12 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
     swa1_store_own<TIO, CT, D>(sW, dv_acc, 1.0f, dvb, a.dvs[2], a.p.dv, G, wave, lane, no_rope, false);
     return;
   }
-  swa1_write_grad<TIO, D>(smem, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.dks[3], a.p.dk, a.dk_vec != 0, L, inv_rope, wave, n, g, tid);
+  swa1_write_grad<TIO, D>(smem, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.dks[3], a.p.dk, a.dk_vec != 0, L, use_rope ? inv_rope : no_rope, wave, n, g, tid);
   swa1_write_grad<TIO, D>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.p.dv, a.dv_vec != 0, L, no_rope, wave, n, g, tid);
 }
 
 // =============================================================================================
-template <typename TIO, int D, int NCGMAX, int CR>
+template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
@@ -306,20 +308,21 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
-  const bool use_rope = a.p.rope.enabled != 0;
+  constexpr bool use_rope = ROPE != 0;
+  constexpr bool BAL = ROPE == 2;
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
   constexpr int NI = swa1_items(D, HCW, CR);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR>(sp, G, PITCH, tid);
-  const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
+  swa1_plan_init<D, HCW, CR, BAL>(sp, G, PITCH, tid, a.rope_pbit);
+  const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   swa1_regs_zero(srv);
-  swa1_issue(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx);
-  swa1_issue(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr);
+  swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx);
+  swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr);
 
   // own queries / output gradients straight into B-operand fragments
   u32x4 qf[KC], dof[KC];
@@ -354,15 +357,15 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   for (int d = 0; d < DB; d++) dq_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float scale = a.scale_log2;
 
-  swa1_commit<CT>(srk, sp, sK, a.rope_pbit, fwd_rope, use_rope && on_k);
-  swa1_commit<CT>(srv, sp, sV, 1, no_rope, false);
+  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k);
+  swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
   __syncthreads();
 
   for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
     const int cr0 = CR * ch;
     if (ch < L.ch_last) {
-      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
-      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
+      swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
+      swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
     }
     float rbias[2];
 #pragma unroll
@@ -405,8 +408,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
     }
     __syncthreads();
     if (ch < L.ch_last) {
-      swa1_commit<CT>(srk, sp, sK, a.rope_pbit, fwd_rope, use_rope && on_k);
-      swa1_commit<CT>(srv, sp, sV, 1, no_rope, false);
+      swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k);
+      swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
       __syncthreads();
     }
   }
@@ -417,5 +420,5 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
                                inv_rope, use_rope);
     return;
   }
-  swa1_write_grad<TIO, D>(smem, dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.dqs[3], a.p.dk, a.dq_vec != 0, L, inv_rope, wave, n, g, tid);
+  swa1_write_grad<TIO, D>(smem, dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.dqs[3], a.p.dk, a.dq_vec != 0, L, use_rope ? inv_rope : no_rope, wave, n, g, tid);
 }

@@ -39,18 +39,44 @@ struct Swa1Geom {
 // the nearest grid token instead of being zero-filled: such positions are always masked by the
 // -inf window bias, so their (finite) values never reach a result, and the loads need neither
 // a branch nor a zero fill.
+//
+// A token row of D dims is staged by D / 32 neighbouring threads, four 16-byte chunks each.
+// Plain mapping: thread qd takes chunks 4 qd .. 4 qd + 3.  Balanced mapping (`bal_r8` > 0, used
+// when the rotary encoding covers exactly half of the head dim, R = D / 8 = 8 bal_r8): there are
+// as many rotary pairs of chunks as threads, so thread qd takes pair qd (chunks x0, x0 + bal_r8)
+// plus two of the unrotated chunks, and every lane rotates one pair instead of half of the
+// lanes rotating two.
 template <int NI>
 struct StagePlan {
   int hr[NI];    // halo row inside the chunk (0..7)
   int cc[NI];    // grid column, clamped
-  int loff[NI];  // byte offset inside the LDS chunk, -1: no such item
-  int qoff;      // byte offset of the thread's 64-byte piece inside a token row
+  int loff[NI];  // byte offset of the token row inside the LDS chunk, -1: no such item
+  int coff[4];   // byte offsets of the thread's four 16-byte chunks inside a token row
+  int bal;       // balanced mapping: chunks 0 and 1 are a rotary pair
+  int axis;      // balanced: 0 row angle, 1 column angle
+  int tab_off;   // balanced: float offset of the pair's (cos, sin) values inside a table row
 };
 
-template <int D, int HCW, int CR = 8>
-DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW, CR)>& sp, const Swa1Geom& G, int pitch, int tid) {
+template <int D, int HCW, int CR, bool BAL>
+DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW, CR)>& sp, const Swa1Geom& G, int pitch, int tid, int bal_r8) {
   constexpr int QUADS = D / 32;
   const int qd = tid % QUADS, key0 = tid / QUADS;
+  sp.bal = BAL;
+  if (BAL) {
+    const int region2 = qd / bal_r8, ci = qd - region2 * bal_r8;
+    const int x0 = 2 * region2 * bal_r8 + ci;
+    sp.coff[0] = 16 * x0;
+    sp.coff[1] = 16 * (x0 + bal_r8);
+    sp.coff[2] = 16 * (4 * bal_r8 + 2 * qd);
+    sp.coff[3] = sp.coff[2] + 16;
+    sp.axis = region2;
+    sp.tab_off = 16 * ci;
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; j++) sp.coff[j] = 64 * qd + 16 * j;
+    sp.axis = 0;
+    sp.tab_off = 0;
+  }
 #pragma unroll
   for (int it = 0; it < swa1_items(D, HCW, CR); it++) {
     const int key = key0 + it * (256 / QUADS);
@@ -59,9 +85,8 @@ DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW, CR)>& sp, const Swa1Geo
     const int hr = k / HCW, hc = k - hr * HCW;
     sp.hr[it] = hr;
     sp.cc[it] = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));
-    sp.loff[it] = live ? k * pitch + 64 * qd : -1;
+    sp.loff[it] = live ? k * pitch : -1;
   }
-  sp.qoff = 64 * qd;
 }
 
 // One thread's share of a halo chunk in flight between HBM and LDS (rotary partners, 8 or 16
@@ -85,7 +110,7 @@ DLT_DEV void swa1_regs_zero(StageRegs<NI>& sr) {
 // Issue the global loads of halo rows [cr0, cr0 + 8) into registers.  `sn2` is the token stride
 // in BYTES; offsets are 32-bit (the host checks that a [N, D] slab stays below 2 GiB).  `on`:
 // the thread's 64-byte piece lies below the actual head dim (pieces above it stay zero).
-template <int NI>
+template <int NI, bool BAL>
 DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, const void* base, int sn2, const Swa1Geom& G,
                         int cr0, const int32_t* rope_idx) {
   const int rbase = G.r0 - G.WR + cr0;
@@ -94,24 +119,43 @@ DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, con
     const int r = dlt_imax(0, dlt_imin(rbase + sp.hr[it], G.TR - 1));
     const int tok = r * G.TC + sp.cc[it];
     if (on) {
-      const char* p = reinterpret_cast<const char*>(base) + (uint32_t)(tok * sn2 + sp.qoff);
+      const char* p = reinterpret_cast<const char*>(base) + (uint32_t)(tok * sn2);
 #pragma unroll
-      for (int j = 0; j < 4; j++) sr.v[it][j] = *reinterpret_cast<const u32x4*>(p + 16 * j);
+      for (int j = 0; j < 4; j++) sr.v[it][j] = *reinterpret_cast<const u32x4*>(p + (BAL ? sp.coff[j] : sp.coff[0] + 16 * j));
     }
     if (rope_idx != nullptr) sr.id[it] = rope_idx[tok];
   }
 }
 
 // Rotate (K / Q side only) and write the staged registers into an LDS chunk.
-// pbit: chunk distance between rotary partners (1 or 2).
-template <typename CT, int NI>
+// ROT: 0 no rotation, 1 rotation with the plain chunk mapping, 2 rotation of the balanced
+// mapping's pair (chunks 0 and 1).  pbit: chunk distance between rotary partners (1 or 2).
+template <typename CT, int NI, bool BAL, int ROT>
 DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, int pbit, const RopeDev& rope, bool use_rope) {
+  static_assert(ROT != 2 || BAL, "pair rotation needs the balanced mapping");
 #pragma unroll
   for (int it = 0; it < NI; it++) {
     if (sp.loff[it] < 0) continue;
-    if (use_rope && sp.qoff < 8 * rope.R) {
+    if (ROT == 2 && use_rope) {
+      bool rotated;
+      const float* tab = rope_table_row(rope, sp.axis, sr.id[it], rotated) + sp.tab_off;
+      if (rotated) {
+        float x0[8], x1[8];
+        unpack8<CT>(sr.v[it][0], x0);
+        unpack8<CT>(sr.v[it][1], x1);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const float cs = tab[2 * j], sn = tab[2 * j + 1];
+          const float y0 = rope_mix(x0[j], x1[j], cs, sn, true);
+          const float y1 = rope_mix(x1[j], x0[j], cs, sn, false);
+          x0[j] = y0; x1[j] = y1;
+        }
+        sr.v[it][0] = pack8<CT>(x0);
+        sr.v[it][1] = pack8<CT>(x1);
+      }
+    } else if (ROT == 1 && use_rope && sp.coff[0] < 8 * rope.R) {
       const int r8 = rope.R >> 3;
-      const int qd4 = sp.qoff >> 4;  // first chunk of this piece
+      const int qd4 = sp.coff[0] >> 4;  // first chunk of this piece
 #pragma unroll
       for (int pr = 0; pr < 2; pr++) {
         // pbit 1: pairs (0,1), (2,3); pbit 2: pairs (0,2), (1,3)
@@ -147,7 +191,7 @@ DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, in
     }
     char* row = s + sp.loff[it];
 #pragma unroll
-    for (int j = 0; j < 4; j++) lds_write16(row + 16 * j, sr.v[it][j]);
+    for (int j = 0; j < 4; j++) lds_write16(row + (BAL ? sp.coff[j] : sp.coff[0] + 16 * j), sr.v[it][j]);
   }
 }
 

@@ -27,12 +27,13 @@ struct Swa1FwdArgs {
   int64_t qs[4], ks[4], vs[4], os[4], ls[3];
   int32_t q_vec, o_vec;
   int32_t rope_pbit;  // chunk distance between rotary partners (R / 8), 1 without rotation
+  int32_t rope_mode;  // 0 none, 1 rotation with the plain staging map, 2 balanced staging map
   float scale_log2;
 };
 
 // CR: halo rows per chunk.  8: a 32-token block is 8 rows x 4 columns; 4: 4 rows x 8 columns
 // (half the LDS and staging registers per workgroup, hence more resident workgroups per CU).
-template <typename TIO, int D, int NCGMAX, int CR>
+template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 2) : (CR == 4 ? 2 : 1))) void swa1_fwd_kernel(const Swa1FwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
@@ -70,7 +71,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   TIO* ob = reinterpret_cast<TIO*>(a.o) + b * a.os[0] + h * a.os[1];
   RopeDev no_rope = a.p.rope;
   no_rope.enabled = 0;
-  const bool use_rope = a.p.rope.enabled != 0;
+  constexpr bool use_rope = ROPE != 0;
+  constexpr bool BAL = ROPE == 2;
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
 
   // own queries: LDS row 16 w + n <-> grid (r0 + (n >> 2), c0 + 4 w + (n & 3))
@@ -85,14 +87,14 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
 
   constexpr int NI = swa1_items(D, HCW, CR);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR>(sp, G, PITCH, tid);
-  const bool on_k = (sp.qoff >> 1) < a.p.dk, on_v = (sp.qoff >> 1) < a.p.dv;
+  swa1_plan_init<D, HCW, CR, BAL>(sp, G, PITCH, tid, a.rope_pbit);
+  const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   swa1_regs_zero(srv);
-  swa1_issue(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx);
-  swa1_issue(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr);
+  swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx);
+  swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr);
 
   // own queries straight into B-operand fragments (rotated on the way when fused)
   u32x4 qf[KC];
@@ -127,15 +129,15 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const unsigned one2 = pack2<CT>(1.f, 1.f);
   const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
 
-  swa1_commit<CT>(srk, sp, sK, a.rope_pbit, a.p.rope, use_rope && on_k);
-  swa1_commit<CT>(srv, sp, sV, 1, a.p.rope, false);
+  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k);
+  swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
   __syncthreads();
 
   for (int ch = ch_first; ch <= ch_last; ch++) {
     const int cr0 = CR * ch;
     if (ch < ch_last) {  // next chunk: HBM -> registers while this one is consumed
-      swa1_issue(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
-      swa1_issue(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
+      swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
+      swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
     }
 
     // block kb, half mb -> (row offset inside the chunk, column group)
@@ -219,8 +221,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
     }
     __syncthreads();  // every wave is done with this chunk
     if (ch < ch_last) {
-      swa1_commit<CT>(srk, sp, sK, a.rope_pbit, a.p.rope, use_rope && on_k);
-      swa1_commit<CT>(srv, sp, sV, 1, a.p.rope, false);
+      swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k);
+      swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
       __syncthreads();
     }
   }

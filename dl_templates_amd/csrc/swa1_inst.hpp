@@ -15,9 +15,9 @@ int swa1_set_lds(KernT kern, int bytes) {
   return DLT_OK;
 }
 
-template <typename TIO, int NCGMAX>
-int swa1_launch_fwd_t(const Swa1FwdArgs& a, int grid, hipStream_t stream) {
-  auto kern = swa1_fwd_kernel<TIO, DLT_D, NCGMAX, SWA1_FWD_CR>;
+template <typename TIO, int NCGMAX, int ROPE>
+int swa1_launch_fwd_r(const Swa1FwdArgs& a, int grid, hipStream_t stream) {
+  auto kern = swa1_fwd_kernel<TIO, DLT_D, NCGMAX, SWA1_FWD_CR, ROPE>;
   int rc = swa1_set_lds(kern, a.plan.lds_bytes);
   if (rc != DLT_OK) return rc;
   dlt_timing_before(DLT_K_FWD, stream);
@@ -27,11 +27,21 @@ int swa1_launch_fwd_t(const Swa1FwdArgs& a, int grid, hipStream_t stream) {
   return DLT_OK;
 }
 
+// rotation mode -> kernel variant (the rotation code is compiled out of the plain kernels)
 template <typename TIO, int NCGMAX>
-int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hipStream_t stream) {
+int swa1_launch_fwd_t(const Swa1FwdArgs& a, int grid, hipStream_t stream) {
+  switch (a.rope_mode) {
+    case 0: return swa1_launch_fwd_r<TIO, NCGMAX, 0>(a, grid, stream);
+    case 1: return swa1_launch_fwd_r<TIO, NCGMAX, 1>(a, grid, stream);
+    default: return swa1_launch_fwd_r<TIO, NCGMAX, 2>(a, grid, stream);
+  }
+}
+
+template <typename TIO, int NCGMAX, int ROPE>
+int swa1_launch_bwd_r(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hipStream_t stream) {
   // dQ first: with fuse_delta it produces the delta vector the dK/dV kernel consumes
   {
-    auto kern = swa1_bwd_q_kernel<TIO, DLT_D, NCGMAX, SWA1_FWD_CR>;
+    auto kern = swa1_bwd_q_kernel<TIO, DLT_D, NCGMAX, SWA1_FWD_CR, ROPE>;
     int rc = swa1_set_lds(kern, lds_q);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_Q, stream);
@@ -40,7 +50,7 @@ int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hip
     DLT_CHECK_LAUNCH("token-grid attention dQ launch");
   }
   {
-    auto kern = swa1_bwd_kv_kernel<TIO, DLT_D, NCGMAX, SWA1_KV_CR>;
+    auto kern = swa1_bwd_kv_kernel<TIO, DLT_D, NCGMAX, SWA1_KV_CR, ROPE>;
     int rc = swa1_set_lds(kern, lds_kv);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_KV, stream);
@@ -49,6 +59,15 @@ int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hip
     DLT_CHECK_LAUNCH("token-grid attention dK/dV launch");
   }
   return DLT_OK;
+}
+
+template <typename TIO, int NCGMAX>
+int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hipStream_t stream) {
+  switch (a.rope_mode) {
+    case 0: return swa1_launch_bwd_r<TIO, NCGMAX, 0>(a, grid, lds_kv, lds_q, stream);
+    case 1: return swa1_launch_bwd_r<TIO, NCGMAX, 1>(a, grid, lds_kv, lds_q, stream);
+    default: return swa1_launch_bwd_r<TIO, NCGMAX, 2>(a, grid, lds_kv, lds_q, stream);
+  }
 }
 }  // namespace
 
