@@ -183,7 +183,7 @@ class SwaWorkload:
 
 
 class FlashWorkload:
-    def __init__(self, B, H, Lq, Lk, dk, dv, seed=0, dtype=torch.bfloat16):
+    def __init__(self, B, H, Lq, Lk, dk, dv, seed=0, dtype=torch.bfloat16, causal=False, scale=None):
         from dl_templates_amd import _lib
         dev = torch.device("cuda:0")
         q, k, v, do = make_inputs(seed, B, H, Lq, Lk, dk, dv, dtype, dev)
@@ -193,7 +193,7 @@ class FlashWorkload:
         dq, dkk, dvv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         self.keep = (q, k, v, do, o, lse, delta, dq, dkk, dvv)
         L = _lib
-        shape = L.FlashShape(B, H, Lq, Lk, dk, dv, 1.0 / math.sqrt(dk), 0, L.dtype_code(q))
+        shape = L.FlashShape(B, H, Lq, Lk, dk, dv, scale if scale is not None else 1.0 / math.sqrt(dk), int(causal), L.dtype_code(q))
         st = L.stream_of(q)
         self.fwd = (L.ptr(q), L.strides(q), L.ptr(k), L.strides(k), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
                     L.ptr(lse), L.strides(lse), shape, st)
@@ -201,12 +201,17 @@ class FlashWorkload:
                     L.ptr(do), L.strides(do), L.ptr(lse), L.ptr(delta), L.strides(lse), L.ptr(dq), L.strides(dq),
                     L.ptr(dkk), L.strides(dkk), L.ptr(dvv), L.strides(dvv), shape, st)
         self.lib, self._lib = L.load(), L
-        pairs = B * H * Lq * Lk
+        pairs = B * H * Lq * Lk * (0.5 if causal else 1.0)  # the reference's convention for causal (src/flash_attn.py:608-614)
         self.flops_fwd = 2 * pairs * (dk + dv)
         self.flops_bwd = 2 * pairs * (3 * dk + 2 * dv)
 
     def step(self):
         rc = self.lib.dlt_flash_fwd(*self.fwd) or self.lib.dlt_flash_bwd(*self.bwd)
+        if rc:
+            self._lib.check(rc)
+
+    def fwd_only(self):
+        rc = self.lib.dlt_flash_fwd(*self.fwd)
         if rc:
             self._lib.check(rc)
 
@@ -389,6 +394,19 @@ def main():
         extra["ref_demo_b16"] = {"ms_per_step": msd, "eff_tflops": fd / (msd * 1e-3) / 1e12,
                                  "workload": "B=4 H=8 16x16 tiles of 16 tokens, d=32, 3x3 window, fp16, fwd+bwd"}
         del wd
+        # the shape the reference publishes flash numbers for (B=4, H=32, d=64, fp16, sm_scale 1.3,
+        # src/flash_attn.py:548,580-586; its CSVs name no hardware), at N_CTX = 4096
+        ref = {}
+        for causal in (False, True):
+            wr = FlashWorkload(4, 32, 4096, 4096, 64, 64, dtype=torch.float16, causal=causal, scale=1.3)
+            ms_f, _ = Timer.run(wr.fwd_only, max(K // 5, 3), 2)
+            ms_s, _ = Timer.run(wr.step, max(K // 5, 3), 2)
+            ref["causal" if causal else "non_causal"] = {
+                "fwd_ms": ms_f, "fwd_tflops": wr.flops_fwd / (ms_f * 1e-3) / 1e12,
+                "bwd_ms": ms_s - ms_f, "bwd_tflops": wr.flops_bwd / ((ms_s - ms_f) * 1e-3) / 1e12}
+            del wr
+        ref["published_triton_fp16_unstated_hw_tflops"] = {"fwd_non_causal": 73.56, "fwd_causal": 71.11, "bwd_causal": 38.22}
+        extra["flash_ref_b4_h32_d64_n4096_fp16"] = ref
         w5 = FlashWorkload(2, 16, 4096, 8192, 64, 128)
         ms5, _ = Timer.run(w5.step, max(K // 5, 3), 2)
         kb5 = kernel_breakdown(w5.step, 3)

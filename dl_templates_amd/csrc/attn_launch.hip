@@ -207,7 +207,7 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
 // ---- dense flash fast path ----------------------------------------------------------------
 // needs 2-byte elements, 16-byte vector access to q, k, v and 32-bit byte offsets inside a slab
 bool flash_eligible(const AttnProblem& p, const AttnTensors& t, bool with_do) {
-  if (p.g.mode != DLT_GEOM_DENSE) return false;
+  if (p.g.mode != DLT_GEOM_DENSE && p.g.mode != DLT_GEOM_CAUSAL) return false;
   if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
   const int es = 2;
   if (!vec_ok(t.q, t.qs, 4, p.dk, es) || !vec_ok(t.k, t.ks, 4, p.dk, es) || !vec_ok(t.v, t.vs, 4, p.dv, es)) return false;
@@ -227,6 +227,7 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
   a.B = p.B; a.H = p.H; a.Lq = p.g.XLq; a.Lk = p.g.XLk; a.dk = p.dk; a.dv = p.dv;
   const int own = 64 * FLASH_NP;
   a.nblk = (a.Lq + own - 1) / own;
+  a.causal = p.g.mode == DLT_GEOM_CAUSAL;
   a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, 2);
   const int chunk = FLASH_CK * (dc.DK * 2 + 16 + dc.DV * 2 + 16), tile = own * (dc.DV * 2 + 16);
   a.lds_bytes = chunk > tile ? chunk : tile;
@@ -264,6 +265,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   const int own = 64 * FLASH_NP, own_kv = 64 * flash_np_kv(dc.DK, dc.DV);
   a.nblk_q = (a.Lq + own - 1) / own;
   a.nblk_k = (a.Lk + own_kv - 1) / own_kv;
+  a.causal = p.g.mode == DLT_GEOM_CAUSAL;
   a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, 2);
   a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, 2);
   a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, 2);

@@ -1,7 +1,9 @@
-// Dense (non-causal) flash attention forward for gfx950 with separate qk / vo head dims.
+// Dense and causal flash attention forward for gfx950 with separate qk / vo head dims.
 //
-// Replaces _attn_fwd_inner / _attn_fwd (src/flash_attn.py:9-172) for the non-causal case and
-// extends it to Lq != Lk.  A workgroup of 4 waves owns 64*NP consecutive queries of one
+// Replaces _attn_fwd_inner / _attn_fwd (src/flash_attn.py:9-172) and extends the non-causal case
+// to Lq != Lk.  CAUSAL (Lq == Lk, query i sees keys j <= i; the STAGE logic of
+// src/flash_attn.py:17-24,152-166): a workgroup stops at its last query, a wave skips chunks
+// that lie entirely above its queries, and only chunks that cross the diagonal pay for a mask.  A workgroup of 4 waves owns 64*NP consecutive queries of one
 // (batch, head); a wave owns NP blocks of 16 queries whose fragments come straight from HBM.
 // K and V stream through LDS in chunks of CK keys; the next chunk travels HBM -> registers
 // while the current one is consumed.  Per chunk and query block: S^T = K Q^T for all 32-key
@@ -30,12 +32,13 @@ struct FlashArgs {
   int64_t qs[4], ks[4], vs[4], os[4], ls[3];
   int32_t B, H, Lq, Lk, dk, dv;
   int32_t nblk;       // workgroups per (batch, head)
+  int32_t causal;
   int32_t o_vec;
   int32_t lds_bytes;
   float scale_log2;
 };
 
-template <typename TIO, int DK, int DV, int NP, int CK>
+template <typename TIO, int DK, int DV, int NP, int CK, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef typename TileOf<TIO>::type TL;
@@ -55,7 +58,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = lin / a.nblk;
-  const int x0 = (lin - bh * a.nblk) * OWN;
+  // causal: the blocks with the most keys to visit are launched first
+  const int xb = CAUSAL ? a.nblk - 1 - (lin - bh * a.nblk) : lin - bh * a.nblk;
+  const int x0 = xb * OWN;
+  const int wq0 = x0 + wave * 16 * NP;                            // first query of this wave
+  const int k_end = CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk;     // keys [0, k_end) are visited
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
   const char* kb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1]);
@@ -96,10 +103,12 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   // ---- own queries -> B-operand fragments
   u32x4 qf[NP][KC];
   int64_t tq[NP];
+  int klim[NP];  // last key this lane's query may see
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int xq = x0 + wave * 16 * NP + 16 * p + n;
     tq[p] = xq < a.Lq ? (int64_t)xq : (int64_t)-1;
+    klim[p] = CAUSAL ? dlt_imin(xq, a.Lk - 1) : a.Lk - 1;
     swa1_load_own<TIO, CT, DK>(qf[p], qb, a.qs[2], a.dk, tq[p], g, no_rope, false);
   }
 
@@ -119,13 +128,16 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   commit();
   __syncthreads();
 
-  for (int k0 = 0; k0 < a.Lk; k0 += CK) {
-    const bool has_next = k0 + CK < a.Lk;
+  for (int k0 = 0; k0 < k_end; k0 += CK) {
+    const bool has_next = k0 + CK < k_end;
     if (has_next) issue(k0 + CK);
-    const bool tail = k0 + CK > a.Lk;  // some keys of this chunk lie past Lk
+    // some keys of this chunk lie past Lk or (causal) above the wave's first query
+    const bool tail = k0 + CK > a.Lk || (CAUSAL && k0 + CK - 1 > wq0);
+    // causal: every key of the chunk lies above every query of this wave (wave-uniform)
+    const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
 
     u32x4 pb[NP][NKB];
-    {
+    if (live) {
       float t[NP][NKB][8];
 #pragma unroll
       for (int kb = 0; kb < NKB; kb++) {
@@ -151,7 +163,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
 #pragma unroll
             for (int i = 0; i < 8; i++) {
               const int key = k0 + 32 * kb + 16 * (i >> 2) + 4 * g + (i & 3);
-              t[p][kb][i] = key < a.Lk ? t[p][kb][i] : -INFINITY;
+              t[p][kb][i] = key <= klim[p] ? t[p][kb][i] : -INFINITY;
             }
         }
       }
@@ -180,16 +192,18 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
         }
       }
     }
+    if (live) {
 #pragma unroll
-    for (int kb = 0; kb < NKB; kb++) {
+      for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
-      for (int d = 0; d < VB; d++) {
-        const u32x4 vt = lds_read_tokens_as_k(sV, PV, 32 * kb, 16 * d, n, g);
+        for (int d = 0; d < VB; d++) {
+          const u32x4 vt = lds_read_tokens_as_k(sV, PV, 32 * kb, 16 * d, n, g);
 #pragma unroll
-        for (int p = 0; p < NP; p++) acc[p][d] = Mma<CT>::mfma(vt, pb[p][kb], acc[p][d]);
+          for (int p = 0; p < NP; p++) acc[p][d] = Mma<CT>::mfma(vt, pb[p][kb], acc[p][d]);
+        }
+#pragma unroll
+        for (int p = 0; p < NP; p++) acc_l[p] = Mma<CT>::mfma(ones, pb[p][kb], acc_l[p]);
       }
-#pragma unroll
-      for (int p = 0; p < NP; p++) acc_l[p] = Mma<CT>::mfma(ones, pb[p][kb], acc_l[p]);
     }
     __syncthreads();
     if (has_next) {
@@ -216,8 +230,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
 }
 
 // =============================================================================================
-// Dense backward: replaces _attn_bwd_dkdv / _attn_bwd_dq / _attn_bwd (src/flash_attn.py:204-449)
-// for the non-causal case, Lq != Lk allowed, with the decoupled structure of the reference
+// Dense and causal backward: replaces _attn_bwd_dkdv / _attn_bwd_dq / _attn_bwd
+// (src/flash_attn.py:204-449; causal masking :361-379, :416-434), Lq != Lk allowed when not
+// causal, with the decoupled structure of the reference
 // (dK/dV pass over key blocks, dQ pass over query blocks) as two kernels; no host-side
 // pre-scaling pass over k (src/flash_attn.py:509-510), no atomics.
 struct FlashBwdArgs {
@@ -227,6 +242,7 @@ struct FlashBwdArgs {
   int64_t qs[4], ks[4], vs[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
   int32_t B, H, Lq, Lk, dk_, dv_;
   int32_t nblk_q, nblk_k;
+  int32_t causal;
   int32_t dq_vec, dk_vec, dv_vec;
   int32_t lds_q, lds_kv;
   float scale_log2, sm_scale;
@@ -294,7 +310,7 @@ DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO
 }
 
 // ---- dQ: own = queries, K and V stream
-template <typename TIO, int DK, int DV, int NP, int CK>
+template <typename TIO, int DK, int DV, int NP, int CK, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
@@ -310,7 +326,10 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
   const int bh = lin / a.nblk_q;
-  const int x0 = (lin - bh * a.nblk_q) * OWN;
+  const int xb = CAUSAL ? a.nblk_q - 1 - (lin - bh * a.nblk_q) : lin - bh * a.nblk_q;
+  const int x0 = xb * OWN;
+  const int wq0 = x0 + wave * 16 * NP;
+  const int k_end = CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk;
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
   const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
@@ -325,10 +344,12 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
 
   u32x4 qf[NP][KC], dof[NP][VC];
   float nlse[NP], del_n[NP];
+  int klim[NP];
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int xq = x0 + wave * 16 * NP + 16 * p + n;
     const int64_t tq = xq < a.Lq ? (int64_t)xq : (int64_t)-1;
+    klim[p] = CAUSAL ? dlt_imin(xq, a.Lk - 1) : a.Lk - 1;
     swa1_load_own<TIO, CT, DK>(qf[p], qb, a.qs[2], a.dk_, tq, g, no_rope, false);
     swa1_load_own<TIO, CT, DV>(dof[p], dob, a.dos[2], a.dv_, tq, g, no_rope, false);
     const int64_t off = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
@@ -345,12 +366,14 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
   st.commit(sK, PK, sV, PV);
   __syncthreads();
 
-  for (int k0 = 0; k0 < a.Lk; k0 += CK) {
-    const bool has_next = k0 + CK < a.Lk;
+  for (int k0 = 0; k0 < k_end; k0 += CK) {
+    const bool has_next = k0 + CK < k_end;
     if (has_next) st.issue(kb_, sn2k, vb_, sn2v, k0 + CK, a.Lk);
-    const bool tail = k0 + CK > a.Lk;
+    const bool tail = k0 + CK > a.Lk || (CAUSAL && k0 + CK - 1 > wq0);
+    const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++) {
+      if (!live) continue;
       u32x4 ka[2][KC], va[2][VC];
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
@@ -378,7 +401,7 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             float pv = fast_exp2(fmaf(s[mb][i], scale, nlse[p]));
-            if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) < a.Lk ? pv : 0.f;
+            if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? pv : 0.f;
             ds[4 * mb + i] = pv * (dp[mb][i] - del_n[p]);
           }
         dsb[p] = pack8<CT>(ds);
@@ -401,7 +424,7 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
 }
 
 // ---- dK / dV: own = keys, Q, dO, lse2 and delta stream
-template <typename TIO, int DK, int DV, int NP, int CK>
+template <typename TIO, int DK, int DV, int NP, int CK, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
@@ -432,7 +455,10 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
 
   PairStage<DK, DV, CK> st;
   st.init(tid, a.dk_, a.dv_);
-  st.issue(qb, sn2q, dob, sn2d, 0, a.Lq);
+  // causal: queries below the first own key see none of the own keys
+  const int q_start = CAUSAL ? (x0 / CK) * CK : 0;
+  const int wk0 = x0 + wave * 16 * NP;  // first own key of this wave
+  st.issue(qb, sn2q, dob, sn2d, q_start, a.Lq);
   float r_lse = 0.f, r_del = 0.f;
   auto issue_scalars = [&](int q0) {
     if (tid < CK) {
@@ -441,13 +467,15 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
       r_del = delb[tok * a.ls[2]];
     }
   };
-  issue_scalars(0);
+  issue_scalars(q_start);
 
   u32x4 kf[NP][KC], vf[NP][VC];
+  int qmin[NP];  // first query that sees this lane's key
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int xk = x0 + wave * 16 * NP + 16 * p + n;
     const int64_t tk = xk < a.Lk ? (int64_t)xk : (int64_t)-1;
+    qmin[p] = CAUSAL ? xk : 0;
     swa1_load_own<TIO, CT, DK>(kf[p], kb_, a.ks[2], a.dk_, tk, g, no_rope, false);
     swa1_load_own<TIO, CT, DV>(vf[p], vb_, a.vs[2], a.dv_, tk, g, no_rope, false);
   }
@@ -465,15 +493,19 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
   if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
   __syncthreads();
 
-  for (int q0 = 0; q0 < a.Lq; q0 += CK) {
+  for (int q0 = q_start; q0 < a.Lq; q0 += CK) {
     const bool has_next = q0 + CK < a.Lq;
     if (has_next) {
       st.issue(qb, sn2q, dob, sn2d, q0 + CK, a.Lq);
       issue_scalars(q0 + CK);
     }
-    const bool tail = q0 + CK > a.Lq;
+    // some queries of the chunk lie past Lq or (causal) below the wave's last own key
+    const bool tail = q0 + CK > a.Lq || (CAUSAL && q0 < wk0 + 16 * NP - 1);
+    // causal: every query of the chunk lies below every own key of this wave
+    const bool live = !CAUSAL || q0 + CK - 1 >= wk0;
 #pragma unroll
     for (int qb_ = 0; qb_ < NQB; qb_++) {
+      if (!live) continue;
       u32x4 qa[2][KC], da[2][VC];
       f32x4 lq[2], dl[2];
 #pragma unroll
@@ -504,7 +536,10 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             float pv = fast_exp2(fmaf(s[mb][i], scale, -lq[mb][i]));
-            if (tail) pv = (q0 + 32 * qb_ + 16 * mb + 4 * g + i) < a.Lq ? pv : 0.f;
+            if (tail) {
+              const int qi = q0 + 32 * qb_ + 16 * mb + 4 * g + i;
+              pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
+            }
             pr[4 * mb + i] = pv;
             ds[4 * mb + i] = pv * (dp[mb][i] - dl[mb][i]);
           }

@@ -90,6 +90,23 @@ def test_causal_matches_sdpa_bf16():
     assert max(_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w)) <= 5e-2
 
 
+@pytest.mark.parametrize("N,dk,dv,dtype", [
+    (1, 64, 64, torch.bfloat16), (63, 64, 128, torch.bfloat16), (64, 128, 128, torch.bfloat16),
+    (65, 64, 64, torch.float16), (129, 64, 128, torch.bfloat16), (1000, 128, 128, torch.bfloat16),
+    (384, 32, 32, torch.float16)])
+def test_causal_lengths_and_dims(N, dk, dv, dtype):
+    """Causal fast path: lengths around the 64-key chunk and the 128-query block, all head-dim classes."""
+    q, k, v, do = orc.make_qkv(N + dk, 2, 2, N, N, dk, dv, dtype)
+    scale = 1 / math.sqrt(dk)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), True, scale)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(qg, kg, vg, True, scale)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert max(errs) <= 5e-2, errs
+
+
 def test_bad_arguments_raise():
     from dl_templates_amd._lib import DltError
     q = torch.randn(1, 1, 64, 64, dtype=torch.bfloat16).cuda()
