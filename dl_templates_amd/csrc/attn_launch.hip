@@ -6,20 +6,25 @@
 #include "swa1_bwd_kernel.hpp"
 #include "flash_kernel.hpp"
 
+int dlt_launch_fwd_32_32(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_64_64(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_128_128(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_64_128(const FwdArgs&, int, int, hipStream_t);
 
+int dlt_launch_bwd_32_32(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_64_64(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_128_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_64_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 
+int dlt_flash_launch_fwd_32_32(const FlashArgs&, int, int, hipStream_t);
 int dlt_flash_launch_fwd_64_64(const FlashArgs&, int, int, hipStream_t);
 int dlt_flash_launch_fwd_128_128(const FlashArgs&, int, int, hipStream_t);
 int dlt_flash_launch_fwd_64_128(const FlashArgs&, int, int, hipStream_t);
+int dlt_flash_launch_bwd_32_32(const FlashBwdArgs&, int, int, int, hipStream_t);
 int dlt_flash_launch_bwd_64_64(const FlashBwdArgs&, int, int, int, hipStream_t);
 int dlt_flash_launch_bwd_128_128(const FlashBwdArgs&, int, int, int, hipStream_t);
 int dlt_flash_launch_bwd_64_128(const FlashBwdArgs&, int, int, int, hipStream_t);
+int dlt_launch_delta_32_32(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_64_64(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_128_128(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_64_128(const BwdArgs&, hipStream_t);
@@ -35,7 +40,8 @@ constexpr int LDS_TOTAL = 160 * 1024;
 struct DimClass { int DK, DV, id; };
 
 int pick_dims(const AttnProblem& p, DimClass& dc) {
-  if (p.dk <= 64 && p.dv <= 64) dc = {64, 64, 0};
+  if (p.dk <= 32 && p.dv <= 32) dc = {32, 32, 3};  // the reference's demo and test head dims (src/tiled_swa.py:741, src/flash_attn.py:653)
+  else if (p.dk <= 64 && p.dv <= 64) dc = {64, 64, 0};
   else if (p.dk <= 64 && p.dv <= 128) dc = {64, 128, 2};
   else if (p.dk <= 128 && p.dv <= 128) dc = {128, 128, 1};
   else return dlt_set_error(DLT_ERR_UNSUPPORTED, "head dims dk=%d dv=%d: at most 128 is supported", p.dk, p.dv);
@@ -237,6 +243,7 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
   switch (dc.id) {
     case 0: return dlt_flash_launch_fwd_64_64(a, p.dtype, (int)grid, stream);
     case 1: return dlt_flash_launch_fwd_128_128(a, p.dtype, (int)grid, stream);
+    case 3: return dlt_flash_launch_fwd_32_32(a, p.dtype, (int)grid, stream);
     default: return dlt_flash_launch_fwd_64_128(a, p.dtype, (int)grid, stream);
   }
 }
@@ -250,7 +257,8 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   d.o_vec = vec_ok(t.o, t.os, 4, p.dv, 2);
   d.do_vec = 1;
   d.n_tokens_q = p.g.XLq;
-  int rc = dc.id == 0 ? dlt_launch_delta_64_64(d, stream) : dc.id == 1 ? dlt_launch_delta_128_128(d, stream) : dlt_launch_delta_64_128(d, stream);
+  int rc = dc.id == 0 ? dlt_launch_delta_64_64(d, stream) : dc.id == 1 ? dlt_launch_delta_128_128(d, stream)
+         : dc.id == 3 ? dlt_launch_delta_32_32(d, stream) : dlt_launch_delta_64_128(d, stream);
   if (rc != DLT_OK) return rc;
 
   FlashBwdArgs a;
@@ -283,6 +291,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   switch (dc.id) {
     case 0: return dlt_flash_launch_bwd_64_64(a, p.dtype, (int)grid_kv, (int)grid_q, stream);
     case 1: return dlt_flash_launch_bwd_128_128(a, p.dtype, (int)grid_kv, (int)grid_q, stream);
+    case 3: return dlt_flash_launch_bwd_32_32(a, p.dtype, (int)grid_kv, (int)grid_q, stream);
     default: return dlt_flash_launch_bwd_64_128(a, p.dtype, (int)grid_kv, (int)grid_q, stream);
   }
 }
@@ -325,6 +334,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
   switch (dc.id) {
     case 0: return dlt_launch_fwd_64_64(a, np, (int)grid, stream);
     case 1: return dlt_launch_fwd_128_128(a, np, (int)grid, stream);
+    case 3: return dlt_launch_fwd_32_32(a, np, (int)grid, stream);
     default: return dlt_launch_fwd_64_128(a, np, (int)grid, stream);
   }
 }
@@ -392,6 +402,7 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
   switch (dc.id) {
     case 0: return dlt_launch_bwd_64_64(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
     case 1: return dlt_launch_bwd_128_128(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
+    case 3: return dlt_launch_bwd_32_32(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
     default: return dlt_launch_bwd_64_128(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
   }
 }

@@ -162,6 +162,23 @@ def test_pair_launch_matches_two_single_launches():
     assert torch.equal(gq.cpu(), wq) and torch.equal(gk.cpu(), wk)
 
 
+def test_pair_launch_on_packed_qk_projection():
+    """q and k as the two interleaved halves of one fused projection output (the stride-2 views of
+    src/fused_rope2d.py:255-259), rotated in ONE launch; the packed tensor is written nowhere else."""
+    fr = _mods()
+    torch.manual_seed(8)
+    B, N, D = 4, 80, 64
+    qk = torch.randn(B, N, D, 2).to(torch.bfloat16)
+    idx = torch.cat([orc.encode_idx(8, 8), torch.full((16,), -1, dtype=torch.int32)])
+    row_cs, col_cs = _tables(8, 8, 8)
+    wq = orc.rope2d_ref(qk[..., 0], idx, row_cs, col_cs)
+    wk = orc.rope2d_ref(qk[..., 1], idx, row_cs, col_cs)
+    g = qk.cuda()
+    gq, gk = fr.rope2d_qk_(g[..., 0], g[..., 1], idx.cuda(), row_cs.cuda(), col_cs.cuda())
+    assert gq.data_ptr() == g.data_ptr() and gk.data_ptr() == g.data_ptr() + 2
+    assert torch.equal(g[..., 0].cpu(), wq) and torch.equal(g[..., 1].cpu(), wk)
+
+
 def test_module_forward_4d():
     fr = _mods()
     torch.manual_seed(7)
