@@ -210,18 +210,23 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
                    : dlt_swa1_launch_fwd_128(a, c.wclass, (int)grid, stream);
 }
 
-// ---- dense flash fast path ----------------------------------------------------------------
-// needs 2-byte elements, 16-byte vector access to q, k, v and 32-bit byte offsets inside a slab
+// ---- flash fast path: dense, causal, and sliding windows over tiles of 16 k tokens -----------
+// needs 2-byte elements, 16-byte vector access to q, k, v and 32-bit byte offsets inside a slab;
+// tile mode takes no fused rotation (those calls use the generic kernels)
 bool flash_eligible(const AttnProblem& p, const AttnTensors& t, bool with_do) {
-  if (p.g.mode != DLT_GEOM_DENSE && p.g.mode != DLT_GEOM_CAUSAL) return false;
+  if (p.g.mode == DLT_GEOM_SWA) {
+    if (p.g.S < 16 || p.g.S % 16 != 0) return false;
+    if (p.rope.enabled && p.rope.R > 0) return false;
+  }
   if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
   const int es = 2;
   if (!vec_ok(t.q, t.qs, 4, p.dk, es) || !vec_ok(t.k, t.ks, 4, p.dk, es) || !vec_ok(t.v, t.vs, 4, p.dv, es)) return false;
   if (with_do && !vec_ok(t.d_o, t.dos, 4, p.dv, es)) return false;
   const int64_t lim = ((int64_t)1 << 31) - 1;
-  if ((int64_t)p.g.XLk * t.ks[2] * es > lim || (int64_t)p.g.XLk * t.vs[2] * es > lim) return false;
-  if ((int64_t)p.g.XLq * t.qs[2] * es > lim) return false;
-  if (with_do && (int64_t)p.g.XLq * t.dos[2] * es > lim) return false;
+  const int64_t nq = (int64_t)p.g.TR * p.g.XLq, nk = (int64_t)p.g.TR * p.g.XLk;  // tokens of one (batch, head)
+  if (nk * t.ks[2] * es > lim || nk * t.vs[2] * es > lim) return false;
+  if (nq * t.qs[2] * es > lim) return false;
+  if (with_do && nq * t.dos[2] * es > lim) return false;
   return true;
 }
 
@@ -234,11 +239,13 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
   const int own = 64 * FLASH_NP;
   a.nblk = (a.Lq + own - 1) / own;
   a.causal = p.g.mode == DLT_GEOM_CAUSAL;
+  a.tile = p.g.mode == DLT_GEOM_SWA;
+  a.g = p.g;
   a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, 2);
   const int chunk = FLASH_CK * (dc.DK * 2 + 16 + dc.DV * 2 + 16), tile = own * (dc.DV * 2 + 16);
   a.lds_bytes = chunk > tile ? chunk : tile;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
-  const int64_t grid = (int64_t)p.B * p.H * a.nblk;
+  const int64_t grid = (int64_t)p.B * p.H * p.g.TR * a.nblk;
   if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "flash forward: grid too large");
   switch (dc.id) {
     case 0: return dlt_flash_launch_fwd_64_64(a, p.dtype, (int)grid, stream);
@@ -256,7 +263,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   for (int i = 0; i < 3; i++) d.ls[i] = t.ls[i];
   d.o_vec = vec_ok(t.o, t.os, 4, p.dv, 2);
   d.do_vec = 1;
-  d.n_tokens_q = p.g.XLq;
+  d.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
   int rc = dc.id == 0 ? dlt_launch_delta_64_64(d, stream) : dc.id == 1 ? dlt_launch_delta_128_128(d, stream)
          : dc.id == 3 ? dlt_launch_delta_32_32(d, stream) : dlt_launch_delta_64_128(d, stream);
   if (rc != DLT_OK) return rc;
@@ -274,6 +281,8 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   a.nblk_q = (a.Lq + own - 1) / own;
   a.nblk_k = (a.Lk + own_kv - 1) / own_kv;
   a.causal = p.g.mode == DLT_GEOM_CAUSAL;
+  a.tile = p.g.mode == DLT_GEOM_SWA;
+  a.g = p.g;
   a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, 2);
   a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, 2);
   a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, 2);
@@ -286,7 +295,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   if (tile_v > a.lds_kv) a.lds_kv = tile_v;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   a.sm_scale = p.sm_scale;
-  const int64_t grid_q = (int64_t)p.B * p.H * a.nblk_q, grid_kv = (int64_t)p.B * p.H * a.nblk_k;
+  const int64_t grid_q = (int64_t)p.B * p.H * p.g.TR * a.nblk_q, grid_kv = (int64_t)p.B * p.H * p.g.TR * a.nblk_k;
   if (grid_q > 0x7fffffff || grid_kv > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "flash backward: grid too large");
   switch (dc.id) {
     case 0: return dlt_flash_launch_bwd_64_64(a, p.dtype, (int)grid_kv, (int)grid_q, stream);

@@ -6,9 +6,9 @@
 #define DLT_FCAT3(a, b, c) DLT_FCAT3_(a, b, c)
 
 namespace {
-template <typename TIO, bool CAUSAL>
+template <typename TIO, int MODE>
 int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
-  auto kern = flash_fwd_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK, CAUSAL>;
+  auto kern = flash_fwd_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK, MODE>;
   if (a.lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, a.lds_bytes);
     if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", a.lds_bytes, hipGetErrorString(e));
@@ -22,7 +22,8 @@ int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
 
 template <typename TIO>
 int flash_launch_fwd_t(const FlashArgs& a, int grid, hipStream_t stream) {
-  return a.causal ? flash_launch_fwd_c<TIO, true>(a, grid, stream) : flash_launch_fwd_c<TIO, false>(a, grid, stream);
+  if (a.tile) return flash_launch_fwd_c<TIO, 2>(a, grid, stream);
+  return a.causal ? flash_launch_fwd_c<TIO, 1>(a, grid, stream) : flash_launch_fwd_c<TIO, 0>(a, grid, stream);
 }
 
 template <typename KernT>
@@ -34,10 +35,10 @@ int flash_set_lds(KernT kern, int bytes) {
   return DLT_OK;
 }
 
-template <typename TIO, bool CAUSAL>
+template <typename TIO, int MODE>
 int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
   {
-    auto kern = flash_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, flash_np_kv(DLT_DK, DLT_DV), FLASH_CK, CAUSAL>;
+    auto kern = flash_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, flash_np_kv(DLT_DK, DLT_DV), FLASH_CK, MODE>;
     int rc = flash_set_lds(kern, a.lds_kv);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_KV, stream);
@@ -46,7 +47,7 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
     DLT_CHECK_LAUNCH("flash dK/dV launch");
   }
   {
-    auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK, CAUSAL>;
+    auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK, MODE>;
     int rc = flash_set_lds(kern, a.lds_q);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_Q, stream);
@@ -59,7 +60,8 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
 
 template <typename TIO>
 int flash_launch_bwd_t(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
-  return a.causal ? flash_launch_bwd_c<TIO, true>(a, grid_kv, grid_q, stream) : flash_launch_bwd_c<TIO, false>(a, grid_kv, grid_q, stream);
+  if (a.tile) return flash_launch_bwd_c<TIO, 2>(a, grid_kv, grid_q, stream);
+  return a.causal ? flash_launch_bwd_c<TIO, 1>(a, grid_kv, grid_q, stream) : flash_launch_bwd_c<TIO, 0>(a, grid_kv, grid_q, stream);
 }
 }  // namespace
 

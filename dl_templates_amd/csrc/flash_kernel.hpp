@@ -1,4 +1,9 @@
-// Dense and causal flash attention forward for gfx950 with separate qk / vo head dims.
+// Dense, causal and tile-window flash attention forward for gfx950 with separate qk / vo head dims.
+//
+// MODE 0 dense, 1 causal, 2 tiled 2D sliding window with b_size a multiple of 16 (the regime
+// tiled_swa_fwd_large_kernel was written for, src/tiled_swa.py:142-244): a block of 16 own tokens
+// lies inside one tile and every 16-token half of a streamed block lies inside one tile, so the
+// window test is wave-uniform per half: no per-element mask exists, invisible blocks are skipped.
 //
 // Replaces _attn_fwd_inner / _attn_fwd (src/flash_attn.py:9-172) and extends the non-causal case
 // to Lq != Lk.  CAUSAL (Lq == Lk, query i sees keys j <= i; the STAGE logic of
@@ -25,24 +30,82 @@ constexpr int FLASH_CK = FLASH_CK_DEF;  // streamed tokens per LDS chunk
 // key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
 constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 128 ? 1 : 2; }
 
+// One chunk of streamed tokens: first token (index inside the [N, D] slab), its x inside the grid
+// row (tile mode) or the sequence, and how many of the CK staged tokens exist.
+struct FlashChunk { int tok0, x, nvalid; };
+
+// Streamed tokens a workgroup visits.  Dense / causal: [first, len) of the sequence.  Tile mode:
+// for every grid row in [rlo, rhi] the x range [X0, X1) that some own token can see, CK at a time.
+template <int MODE, int CK>
+struct FlashWalk {
+  int first, nchunks;
+  int len;                    // dense / causal
+  int nxc, X0, X1, rlo, XL;   // tile mode
+  DLT_DEV void init_seq(int first_, int len_) {
+    first = first_; len = len_;
+    nchunks = len_ > first_ ? (len_ - first_ + CK - 1) / CK : 0;
+    nxc = 1; X0 = X1 = rlo = XL = 0;
+  }
+  // own tokens: grid row r, x in [x0, x0 + own); `transpose`: the own side are keys
+  DLT_DEV void init_tile(const DltGeom& g, int r, int x0, int own, bool transpose) {
+    const int XLo = transpose ? g.XLk : g.XLq;
+    int rl, rh, xl0, xh0, xl1, xh1;
+    const int xa = dlt_imin(x0, XLo - 1), xb = dlt_imin(x0 + own - 1, XLo - 1);
+    if (transpose) { dlt_query_range(g, r, xa, rl, rh, xl0, xh0); dlt_query_range(g, r, xb, rl, rh, xl1, xh1); }
+    else { dlt_key_range(g, r, xa, rl, rh, xl0, xh0); dlt_key_range(g, r, xb, rl, rh, xl1, xh1); }
+    X0 = xl0; X1 = xh1; rlo = rl;
+    XL = transpose ? g.XLq : g.XLk;
+    nxc = (X1 - X0 + CK - 1) / CK;
+    nchunks = (rh - rl + 1) * nxc;
+    first = 0; len = 0;
+  }
+  DLT_DEV FlashChunk at(int i) const {
+    FlashChunk c;
+    if (MODE == 2) {
+      const int ri = i / nxc;
+      c.x = X0 + (i - ri * nxc) * CK;
+      c.tok0 = (rlo + ri) * XL + c.x;
+      c.nvalid = dlt_imin(CK, X1 - c.x);
+    } else {
+      c.x = first + i * CK;
+      c.tok0 = c.x;
+      c.nvalid = dlt_imin(CK, len - c.x);
+    }
+    return c;
+  }
+};
+
+// workgroup -> (batch * head, grid row, first own x).  `rev`: heavy blocks first (causal).
+DLT_DEV void flash_block(int lin, int nblk, int TR, int own, bool rev, int& bh, int& r, int& x0) {
+  const int per = nblk * TR;
+  bh = lin / per;
+  const int rem = lin - bh * per;
+  r = rem / nblk;
+  const int xb = rem - r * nblk;
+  x0 = (rev ? nblk - 1 - xb : xb) * own;
+}
+
 struct FlashArgs {
   const void *q, *k, *v;
   void* o;
   float* lse;
   int64_t qs[4], ks[4], vs[4], os[4], ls[3];
   int32_t B, H, Lq, Lk, dk, dv;
-  int32_t nblk;       // workgroups per (batch, head)
+  int32_t nblk;       // workgroups per (batch, head) and grid row
   int32_t causal;
+  int32_t tile;       // MODE 2: Lq = Lk = tokens per grid row, geometry in g
+  DltGeom g;
   int32_t o_vec;
   int32_t lds_bytes;
   float scale_log2;
 };
 
-template <typename TIO, int DK, int DV, int NP, int CK, bool CAUSAL>
+template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
 __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef typename TileOf<TIO>::type TL;
   extern __shared__ __align__(16) char smem[];
+  constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
   constexpr int PK = DK * 2 + 16, PV = DV * 2 + 16, PO = DV * (int)sizeof(TL) + 16;
   constexpr int KC = DK / 32, VB = DV / 16, NKB = CK / 32;
   constexpr int OWN = 64 * NP;
@@ -57,12 +120,10 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   char* sV = smem + CK * PK;
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = lin / a.nblk;
+  int bh, r_own, x0;
   // causal: the blocks with the most keys to visit are launched first
-  const int xb = CAUSAL ? a.nblk - 1 - (lin - bh * a.nblk) : lin - bh * a.nblk;
-  const int x0 = xb * OWN;
+  flash_block(lin, a.nblk, TILE ? a.g.TR : 1, OWN, CAUSAL, bh, r_own, x0);
   const int wq0 = x0 + wave * 16 * NP;                            // first query of this wave
-  const int k_end = CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk;     // keys [0, k_end) are visited
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
   const char* kb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1]);
@@ -70,6 +131,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   TIO* ob = reinterpret_cast<TIO*>(a.o) + b * a.os[0] + h * a.os[1];
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   RopeDev no_rope = RopeDev{};
+  const int own_base = TILE ? r_own * a.Lq : 0;                   // token index of own x = 0
+
+  FlashWalk<MODE, CK> W;
+  if (TILE) W.init_tile(a.g, r_own, x0, OWN, false);
+  else W.init_seq(0, CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk);   // causal: keys up to the last own query
 
   // ---- staging plan (chunk invariant): vector `it` of this thread = chunk ck*/vc* of key kkey/vkey + it * step
   const int kc_ = tid % KCH, kkey0 = tid / KCH;
@@ -80,15 +146,16 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   for (int it = 0; it < NKI; it++) rk[it] = u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
   for (int it = 0; it < NVI; it++) rv[it] = u32x4{0u, 0u, 0u, 0u};
-  auto issue = [&](int k0) {
+  // tokens past the end of a chunk are clamped onto its last token (they are masked or skipped)
+  auto issue = [&](const FlashChunk& c) {
 #pragma unroll
     for (int it = 0; it < NKI; it++) {
-      const int key = dlt_imin(k0 + kkey0 + it * (256 / KCH), a.Lk - 1);
+      const int key = c.tok0 + dlt_imin(kkey0 + it * (256 / KCH), c.nvalid - 1);
       if (on_k) rk[it] = *reinterpret_cast<const u32x4*>(kb_ + (uint32_t)(key * sn2k + 16 * kc_));
     }
 #pragma unroll
     for (int it = 0; it < NVI; it++) {
-      const int key = dlt_imin(k0 + vkey0 + it * (256 / VCH), a.Lk - 1);
+      const int key = c.tok0 + dlt_imin(vkey0 + it * (256 / VCH), c.nvalid - 1);
       if (on_v) rv[it] = *reinterpret_cast<const u32x4*>(vb_ + (uint32_t)(key * sn2v + 16 * vc_));
     }
   };
@@ -98,17 +165,23 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
 #pragma unroll
     for (int it = 0; it < NVI; it++) lds_write16(sV + (vkey0 + it * (256 / VCH)) * PV + 16 * vc_, rv[it]);
   };
-  issue(0);
+  if (W.nchunks > 0) issue(W.at(0));
 
   // ---- own queries -> B-operand fragments
   u32x4 qf[NP][KC];
   int64_t tq[NP];
-  int klim[NP];  // last key this lane's query may see
+  int klim[NP];           // dense / causal: last key this lane's query may see
+  int vlo[NP], vhi[NP];   // tile mode: x interval this query block sees in every visited row (wave-uniform)
 #pragma unroll
   for (int p = 0; p < NP; p++) {
-    const int xq = x0 + wave * 16 * NP + 16 * p + n;
-    tq[p] = xq < a.Lq ? (int64_t)xq : (int64_t)-1;
+    const int xq = wq0 + 16 * p + n;
+    tq[p] = xq < a.Lq ? (int64_t)(own_base + xq) : (int64_t)-1;
     klim[p] = CAUSAL ? dlt_imin(xq, a.Lk - 1) : a.Lk - 1;
+    vlo[p] = vhi[p] = 0;
+    if (TILE && wq0 + 16 * p < a.Lq) {
+      int rl, rh;
+      dlt_key_range(a.g, r_own, wq0 + 16 * p, rl, rh, vlo[p], vhi[p]);
+    }
     swa1_load_own<TIO, CT, DK>(qf[p], qb, a.qs[2], a.dk, tq[p], g, no_rope, false);
   }
 
@@ -125,16 +198,34 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   const unsigned one2 = pack2<CT>(1.f, 1.f);
   const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
 
-  commit();
+  if (W.nchunks > 0) commit();
   __syncthreads();
 
-  for (int k0 = 0; k0 < k_end; k0 += CK) {
-    const bool has_next = k0 + CK < k_end;
-    if (has_next) issue(k0 + CK);
-    // some keys of this chunk lie past Lk or (causal) above the wave's first query
-    const bool tail = k0 + CK > a.Lk || (CAUSAL && k0 + CK - 1 > wq0);
+  for (int ci = 0; ci < W.nchunks; ci++) {
+    const FlashChunk c = W.at(ci);
+    const int k0 = c.x;
+    const bool has_next = ci + 1 < W.nchunks;
+    if (has_next) issue(W.at(ci + 1));
+    // dense / causal: some keys of this chunk lie past the end or (causal) above the wave's first query
+    const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && k0 + CK - 1 > wq0));
     // causal: every key of the chunk lies above every query of this wave (wave-uniform)
-    const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
+    bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
+    // tile mode: which 32-key blocks hold a 16-key half that query block p sees (wave-uniform)
+    bool bv[NP][NKB], any[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      any[p] = !TILE;
+#pragma unroll
+      for (int kb = 0; kb < NKB; kb++) {
+        bv[p][kb] = !TILE || (k0 + 32 * kb + 32 > vlo[p] && k0 + 32 * kb < vhi[p]);
+        any[p] = any[p] || bv[p][kb];
+      }
+    }
+    if (TILE) {
+      live = false;
+#pragma unroll
+      for (int p = 0; p < NP; p++) live = live || any[p];
+    }
 
     u32x4 pb[NP][NKB];
     if (live) {
@@ -145,17 +236,25 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
 #pragma unroll
         for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-          for (int c = 0; c < KC; c++) ka[mb][c] = lds_read16(sK + (32 * kb + 16 * mb + n) * PK + (32 * c + 8 * g) * 2);
+          for (int c_ = 0; c_ < KC; c_++) ka[mb][c_] = lds_read16(sK + (32 * kb + 16 * mb + n) * PK + (32 * c_ + 8 * g) * 2);
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-          f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+          if (bv[p][kb]) {
+            f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int c = 0; c < KC; c++) {
-            s0 = Mma<CT>::mfma(ka[0][c], qf[p][c], s0);
-            s1 = Mma<CT>::mfma(ka[1][c], qf[p][c], s1);
+            for (int c_ = 0; c_ < KC; c_++) {
+              s0 = Mma<CT>::mfma(ka[0][c_], qf[p][c_], s0);
+              s1 = Mma<CT>::mfma(ka[1][c_], qf[p][c_], s1);
+            }
+            // tile mode: a 16-key half outside the window of the block is dropped as a whole
+            const bool h0 = !TILE || (k0 + 32 * kb >= vlo[p] && k0 + 32 * kb < vhi[p]);
+            const bool h1 = !TILE || (k0 + 32 * kb + 16 >= vlo[p] && k0 + 32 * kb + 16 < vhi[p]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) { t[p][kb][i] = h0 ? s0[i] : -INFINITY; t[p][kb][4 + i] = h1 ? s1[i] : -INFINITY; }
+          } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) t[p][kb][i] = -INFINITY;
           }
-#pragma unroll
-          for (int i = 0; i < 4; i++) { t[p][kb][i] = s0[i]; t[p][kb][4 + i] = s1[i]; }
         }
         if (tail) {
 #pragma unroll
@@ -169,6 +268,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
       }
 #pragma unroll
       for (int p = 0; p < NP; p++) {
+        if (!any[p]) continue;
         float mloc = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++)
@@ -176,8 +276,9 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
                                    fmaxf(fmaxf(t[p][kb][4], t[p][kb][5]), fmaxf(t[p][kb][6], t[p][kb][7]))));
         mloc = wave_max4(mloc);
         const float m_new = fmaxf(m_run[p], mloc);
-        const float alpha = fast_exp2((m_run[p] - m_new) * scale);
-        const float neg_m2 = -m_new * scale;
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a block that has seen no key yet
+        const float alpha = fast_exp2((m_run[p] - m_use) * scale);
+        const float neg_m2 = -m_use * scale;
         m_run[p] = m_new;
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
@@ -195,14 +296,20 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
     if (live) {
 #pragma unroll
       for (int kb = 0; kb < NKB; kb++) {
+        bool need = false;
+#pragma unroll
+        for (int p = 0; p < NP; p++) need = need || bv[p][kb];
+        if (!need) continue;
 #pragma unroll
         for (int d = 0; d < VB; d++) {
           const u32x4 vt = lds_read_tokens_as_k(sV, PV, 32 * kb, 16 * d, n, g);
 #pragma unroll
-          for (int p = 0; p < NP; p++) acc[p][d] = Mma<CT>::mfma(vt, pb[p][kb], acc[p][d]);
+          for (int p = 0; p < NP; p++)
+            if (bv[p][kb]) acc[p][d] = Mma<CT>::mfma(vt, pb[p][kb], acc[p][d]);
         }
 #pragma unroll
-        for (int p = 0; p < NP; p++) acc_l[p] = Mma<CT>::mfma(ones, pb[p][kb], acc_l[p]);
+        for (int p = 0; p < NP; p++)
+          if (bv[p][kb]) acc_l[p] = Mma<CT>::mfma(ones, pb[p][kb], acc_l[p]);
       }
     }
     __syncthreads();
@@ -226,7 +333,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   }
   __syncthreads();
   store_tile<TIO, TL, DV>(smem, PO, ob, a.os[2], a.os[3], a.dv, a.o_vec != 0, OWN,
-                          [&](int row) { return x0 + row < a.Lq ? (int64_t)(x0 + row) : (int64_t)-1; }, no_rope, tid);
+                          [&](int row) { return x0 + row < a.Lq ? (int64_t)(own_base + x0 + row) : (int64_t)-1; }, no_rope, tid);
 }
 
 // =============================================================================================
@@ -243,6 +350,8 @@ struct FlashBwdArgs {
   int32_t B, H, Lq, Lk, dk_, dv_;
   int32_t nblk_q, nblk_k;
   int32_t causal;
+  int32_t tile;
+  DltGeom g;
   int32_t dq_vec, dk_vec, dv_vec;
   int32_t lds_q, lds_kv;
   float scale_log2, sm_scale;
@@ -267,16 +376,16 @@ struct PairStage {
 #pragma unroll
     for (int it = 0; it < NBI; it++) rb[it] = u32x4{0u, 0u, 0u, 0u};
   }
-  // tokens past `len` are clamped onto the last token (the caller masks them)
-  DLT_DEV void issue(const char* a, int sn2a, const char* b, int sn2b, int t0, int len) {
+  // tokens past the end of the chunk are clamped onto its last token (the caller masks them)
+  DLT_DEV void issue(const char* a, int sn2a, const char* b, int sn2b, const FlashChunk& c) {
 #pragma unroll
     for (int it = 0; it < NAI; it++) {
-      const int tok = dlt_imin(t0 + akey0 + it * (256 / ACH), len - 1);
+      const int tok = c.tok0 + dlt_imin(akey0 + it * (256 / ACH), c.nvalid - 1);
       if (on_a) ra[it] = *reinterpret_cast<const u32x4*>(a + (uint32_t)(tok * sn2a + 16 * ac));
     }
 #pragma unroll
     for (int it = 0; it < NBI; it++) {
-      const int tok = dlt_imin(t0 + bkey0 + it * (256 / BCH), len - 1);
+      const int tok = c.tok0 + dlt_imin(bkey0 + it * (256 / BCH), c.nvalid - 1);
       if (on_b) rb[it] = *reinterpret_cast<const u32x4*>(b + (uint32_t)(tok * sn2b + 16 * bc));
     }
   }
@@ -291,7 +400,7 @@ struct PairStage {
 // accumulators (C layout, [dim][own token]) of NP blocks -> LDS tile -> HBM rows
 template <typename TIO, int D, int NP>
 DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO* base, int64_t sn, int64_t sd, int dact,
-                              bool vec, int x0, int len, int wave, int n, int g, int tid) {
+                              bool vec, int own_base, int x0, int len, int wave, int n, int g, int tid) {
   typedef typename TileOf<TIO>::type TL;
   constexpr int PT = D * (int)sizeof(TL) + 16;
   RopeDev no_rope = RopeDev{};
@@ -305,15 +414,16 @@ DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO
   }
   __syncthreads();
   store_tile<TIO, TL, D>(sT, PT, base, sn, sd, dact, vec, 64 * NP,
-                         [&](int r) { return x0 + r < len ? (int64_t)(x0 + r) : (int64_t)-1; }, no_rope, tid);
+                         [&](int r) { return x0 + r < len ? (int64_t)(own_base + x0 + r) : (int64_t)-1; }, no_rope, tid);
   __syncthreads();
 }
 
 // ---- dQ: own = queries, K and V stream
-template <typename TIO, int DK, int DV, int NP, int CK, bool CAUSAL>
+template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
 __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
+  constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
   constexpr int PK = DK * 2 + 16, PV = DV * 2 + 16;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, NKB = CK / 32;
   constexpr int OWN = 64 * NP;
@@ -325,11 +435,9 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
   char* sV = smem + CK * PK;
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = lin / a.nblk_q;
-  const int xb = CAUSAL ? a.nblk_q - 1 - (lin - bh * a.nblk_q) : lin - bh * a.nblk_q;
-  const int x0 = xb * OWN;
+  int bh, r_own, x0;
+  flash_block(lin, a.nblk_q, TILE ? a.g.TR : 1, OWN, CAUSAL, bh, r_own, x0);
   const int wq0 = x0 + wave * 16 * NP;
-  const int k_end = CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk;
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
   const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
@@ -337,19 +445,29 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
   const char* vb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1]);
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   RopeDev no_rope = RopeDev{};
+  const int own_base = TILE ? r_own * a.Lq : 0;
+
+  FlashWalk<MODE, CK> W;
+  if (TILE) W.init_tile(a.g, r_own, x0, OWN, false);
+  else W.init_seq(0, CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk);
 
   PairStage<DK, DV, CK> st;
   st.init(tid, a.dk_, a.dv_);
-  st.issue(kb_, sn2k, vb_, sn2v, 0, a.Lk);
+  if (W.nchunks > 0) st.issue(kb_, sn2k, vb_, sn2v, W.at(0));
 
   u32x4 qf[NP][KC], dof[NP][VC];
   float nlse[NP], del_n[NP];
-  int klim[NP];
+  int klim[NP], vlo[NP], vhi[NP];
 #pragma unroll
   for (int p = 0; p < NP; p++) {
-    const int xq = x0 + wave * 16 * NP + 16 * p + n;
-    const int64_t tq = xq < a.Lq ? (int64_t)xq : (int64_t)-1;
+    const int xq = wq0 + 16 * p + n;
+    const int64_t tq = xq < a.Lq ? (int64_t)(own_base + xq) : (int64_t)-1;
     klim[p] = CAUSAL ? dlt_imin(xq, a.Lk - 1) : a.Lk - 1;
+    vlo[p] = vhi[p] = 0;
+    if (TILE && wq0 + 16 * p < a.Lq) {
+      int rl, rh;
+      dlt_key_range(a.g, r_own, wq0 + 16 * p, rl, rh, vlo[p], vhi[p]);
+    }
     swa1_load_own<TIO, CT, DK>(qf[p], qb, a.qs[2], a.dk_, tq, g, no_rope, false);
     swa1_load_own<TIO, CT, DV>(dof[p], dob, a.dos[2], a.dv_, tq, g, no_rope, false);
     const int64_t off = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
@@ -363,54 +481,68 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
     for (int d = 0; d < KB; d++) dq_acc[p][d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float scale = a.scale_log2;
 
-  st.commit(sK, PK, sV, PV);
+  if (W.nchunks > 0) st.commit(sK, PK, sV, PV);
   __syncthreads();
 
-  for (int k0 = 0; k0 < k_end; k0 += CK) {
-    const bool has_next = k0 + CK < k_end;
-    if (has_next) st.issue(kb_, sn2k, vb_, sn2v, k0 + CK, a.Lk);
-    const bool tail = k0 + CK > a.Lk || (CAUSAL && k0 + CK - 1 > wq0);
+  for (int ci = 0; ci < W.nchunks; ci++) {
+    const FlashChunk c = W.at(ci);
+    const int k0 = c.x;
+    const bool has_next = ci + 1 < W.nchunks;
+    if (has_next) st.issue(kb_, sn2k, vb_, sn2v, W.at(ci + 1));
+    const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && k0 + CK - 1 > wq0));
     const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++) {
       if (!live) continue;
+      bool bv[NP], need = false;
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        bv[p] = !TILE || (k0 + 32 * kb + 32 > vlo[p] && k0 + 32 * kb < vhi[p]);
+        need = need || bv[p];
+      }
+      if (!need) continue;
       u32x4 ka[2][KC], va[2][VC];
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
 #pragma unroll
-        for (int c = 0; c < KC; c++) ka[mb][c] = lds_read16(sK + (32 * kb + 16 * mb + n) * PK + (32 * c + 8 * g) * 2);
+        for (int c_ = 0; c_ < KC; c_++) ka[mb][c_] = lds_read16(sK + (32 * kb + 16 * mb + n) * PK + (32 * c_ + 8 * g) * 2);
 #pragma unroll
-        for (int c = 0; c < VC; c++) va[mb][c] = lds_read16(sV + (32 * kb + 16 * mb + n) * PV + (32 * c + 8 * g) * 2);
+        for (int c_ = 0; c_ < VC; c_++) va[mb][c_] = lds_read16(sV + (32 * kb + 16 * mb + n) * PV + (32 * c_ + 8 * g) * 2);
       }
       u32x4 dsb[NP];
 #pragma unroll
       for (int p = 0; p < NP; p++) {
+        if (!bv[p]) continue;
         f32x4 s[2], dp[2];
 #pragma unroll
         for (int mb = 0; mb < 2; mb++) {
           s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
           dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int c = 0; c < KC; c++) s[mb] = Mma<CT>::mfma(ka[mb][c], qf[p][c], s[mb]);
+          for (int c_ = 0; c_ < KC; c_++) s[mb] = Mma<CT>::mfma(ka[mb][c_], qf[p][c_], s[mb]);
 #pragma unroll
-          for (int c = 0; c < VC; c++) dp[mb] = Mma<CT>::mfma(va[mb][c], dof[p][c], dp[mb]);
+          for (int c_ = 0; c_ < VC; c_++) dp[mb] = Mma<CT>::mfma(va[mb][c_], dof[p][c_], dp[mb]);
         }
         float ds[8];
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
+        for (int mb = 0; mb < 2; mb++) {
+          const bool hv = !TILE || (k0 + 32 * kb + 16 * mb >= vlo[p] && k0 + 32 * kb + 16 * mb < vhi[p]);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             float pv = fast_exp2(fmaf(s[mb][i], scale, nlse[p]));
             if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? pv : 0.f;
+            if (TILE) pv = hv ? pv : 0.f;
             ds[4 * mb + i] = pv * (dp[mb][i] - del_n[p]);
           }
+        }
         dsb[p] = pack8<CT>(ds);
       }
 #pragma unroll
       for (int d = 0; d < KB; d++) {
         const u32x4 kt = lds_read_tokens_as_k(sK, PK, 32 * kb, 16 * d, n, g);
 #pragma unroll
-        for (int p = 0; p < NP; p++) dq_acc[p][d] = Mma<CT>::mfma(kt, dsb[p], dq_acc[p][d]);
+        for (int p = 0; p < NP; p++)
+          if (bv[p]) dq_acc[p][d] = Mma<CT>::mfma(kt, dsb[p], dq_acc[p][d]);
       }
     }
     __syncthreads();
@@ -420,14 +552,15 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
     }
   }
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
-  flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, a.dqs[2], a.dqs[3], a.dk_, a.dq_vec != 0, x0, a.Lq, wave, n, g, tid);
+  flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, a.dqs[2], a.dqs[3], a.dk_, a.dq_vec != 0, own_base, x0, a.Lq, wave, n, g, tid);
 }
 
 // ---- dK / dV: own = keys, Q, dO, lse2 and delta stream
-template <typename TIO, int DK, int DV, int NP, int CK, bool CAUSAL>
+template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
 __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
+  constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
   constexpr int PQ = DK * 2 + 16, PD = DV * 2 + 16;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16, NQB = CK / 32;
   constexpr int OWN = 64 * NP;
@@ -441,8 +574,8 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
   float* sDel = sLse + CK;
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
-  const int bh = lin / a.nblk_k;
-  const int x0 = (lin - bh * a.nblk_k) * OWN;
+  int bh, r_own, x0;
+  flash_block(lin, a.nblk_k, TILE ? a.g.TR : 1, OWN, false, bh, r_own, x0);
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* kb_ = reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1];
   const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
@@ -452,30 +585,40 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
   const float* delb = a.delta + b * a.ls[0] + h * a.ls[1];
   const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
   RopeDev no_rope = RopeDev{};
+  const int own_base = TILE ? r_own * a.Lk : 0;
+
+  // causal: queries below the first own key see none of the own keys
+  FlashWalk<MODE, CK> W;
+  if (TILE) W.init_tile(a.g, r_own, x0, OWN, true);
+  else W.init_seq(CAUSAL ? (x0 / CK) * CK : 0, a.Lq);
+  const int wk0 = x0 + wave * 16 * NP;  // first own key of this wave
 
   PairStage<DK, DV, CK> st;
   st.init(tid, a.dk_, a.dv_);
-  // causal: queries below the first own key see none of the own keys
-  const int q_start = CAUSAL ? (x0 / CK) * CK : 0;
-  const int wk0 = x0 + wave * 16 * NP;  // first own key of this wave
-  st.issue(qb, sn2q, dob, sn2d, q_start, a.Lq);
+  if (W.nchunks > 0) st.issue(qb, sn2q, dob, sn2d, W.at(0));
   float r_lse = 0.f, r_del = 0.f;
-  auto issue_scalars = [&](int q0) {
+  auto issue_scalars = [&](const FlashChunk& c) {
     if (tid < CK) {
-      const int64_t tok = dlt_imin(q0 + tid, a.Lq - 1);
+      const int64_t tok = c.tok0 + dlt_imin(tid, c.nvalid - 1);
       r_lse = lseb[tok * a.ls[2]];
       r_del = delb[tok * a.ls[2]];
     }
   };
-  issue_scalars(q_start);
+  if (W.nchunks > 0) issue_scalars(W.at(0));
 
   u32x4 kf[NP][KC], vf[NP][VC];
-  int qmin[NP];  // first query that sees this lane's key
+  int qmin[NP];           // causal: first query that sees this lane's key
+  int vlo[NP], vhi[NP];   // tile mode: x interval of the queries that see this key block
 #pragma unroll
   for (int p = 0; p < NP; p++) {
-    const int xk = x0 + wave * 16 * NP + 16 * p + n;
-    const int64_t tk = xk < a.Lk ? (int64_t)xk : (int64_t)-1;
+    const int xk = wk0 + 16 * p + n;
+    const int64_t tk = xk < a.Lk ? (int64_t)(own_base + xk) : (int64_t)-1;
     qmin[p] = CAUSAL ? xk : 0;
+    vlo[p] = vhi[p] = 0;
+    if (TILE && wk0 + 16 * p < a.Lk) {
+      int rl, rh;
+      dlt_query_range(a.g, r_own, wk0 + 16 * p, rl, rh, vlo[p], vhi[p]);
+    }
     swa1_load_own<TIO, CT, DK>(kf[p], kb_, a.ks[2], a.dk_, tk, g, no_rope, false);
     swa1_load_own<TIO, CT, DV>(vf[p], vb_, a.vs[2], a.dv_, tk, g, no_rope, false);
   }
@@ -489,50 +632,64 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
   }
   const float scale = a.scale_log2;
 
-  st.commit(sQ, PQ, sDO, PD);
-  if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
+  if (W.nchunks > 0) {
+    st.commit(sQ, PQ, sDO, PD);
+    if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
+  }
   __syncthreads();
 
-  for (int q0 = q_start; q0 < a.Lq; q0 += CK) {
-    const bool has_next = q0 + CK < a.Lq;
+  for (int ci = 0; ci < W.nchunks; ci++) {
+    const FlashChunk c = W.at(ci);
+    const int q0 = c.x;
+    const bool has_next = ci + 1 < W.nchunks;
     if (has_next) {
-      st.issue(qb, sn2q, dob, sn2d, q0 + CK, a.Lq);
-      issue_scalars(q0 + CK);
+      const FlashChunk cn = W.at(ci + 1);
+      st.issue(qb, sn2q, dob, sn2d, cn);
+      issue_scalars(cn);
     }
-    // some queries of the chunk lie past Lq or (causal) below the wave's last own key
-    const bool tail = q0 + CK > a.Lq || (CAUSAL && q0 < wk0 + 16 * NP - 1);
+    // some queries of the chunk lie past the end or (causal) below the wave's last own key
+    const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && q0 < wk0 + 16 * NP - 1));
     // causal: every query of the chunk lies below every own key of this wave
     const bool live = !CAUSAL || q0 + CK - 1 >= wk0;
 #pragma unroll
     for (int qb_ = 0; qb_ < NQB; qb_++) {
       if (!live) continue;
+      bool bv[NP], need = false;
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        bv[p] = !TILE || (q0 + 32 * qb_ + 32 > vlo[p] && q0 + 32 * qb_ < vhi[p]);
+        need = need || bv[p];
+      }
+      if (!need) continue;
       u32x4 qa[2][KC], da[2][VC];
       f32x4 lq[2], dl[2];
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
 #pragma unroll
-        for (int c = 0; c < KC; c++) qa[mb][c] = lds_read16(sQ + (32 * qb_ + 16 * mb + n) * PQ + (32 * c + 8 * g) * 2);
+        for (int c_ = 0; c_ < KC; c_++) qa[mb][c_] = lds_read16(sQ + (32 * qb_ + 16 * mb + n) * PQ + (32 * c_ + 8 * g) * 2);
 #pragma unroll
-        for (int c = 0; c < VC; c++) da[mb][c] = lds_read16(sDO + (32 * qb_ + 16 * mb + n) * PD + (32 * c + 8 * g) * 2);
+        for (int c_ = 0; c_ < VC; c_++) da[mb][c_] = lds_read16(sDO + (32 * qb_ + 16 * mb + n) * PD + (32 * c_ + 8 * g) * 2);
         lq[mb] = *reinterpret_cast<const f32x4*>(sLse + 32 * qb_ + 16 * mb + 4 * g);
         dl[mb] = *reinterpret_cast<const f32x4*>(sDel + 32 * qb_ + 16 * mb + 4 * g);
       }
       u32x4 pb[NP], dsb[NP];
 #pragma unroll
       for (int p = 0; p < NP; p++) {
+        if (!bv[p]) continue;
         f32x4 s[2], dp[2];
 #pragma unroll
         for (int mb = 0; mb < 2; mb++) {
           s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
           dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-          for (int c = 0; c < KC; c++) s[mb] = Mma<CT>::mfma(qa[mb][c], kf[p][c], s[mb]);
+          for (int c_ = 0; c_ < KC; c_++) s[mb] = Mma<CT>::mfma(qa[mb][c_], kf[p][c_], s[mb]);
 #pragma unroll
-          for (int c = 0; c < VC; c++) dp[mb] = Mma<CT>::mfma(da[mb][c], vf[p][c], dp[mb]);
+          for (int c_ = 0; c_ < VC; c_++) dp[mb] = Mma<CT>::mfma(da[mb][c_], vf[p][c_], dp[mb]);
         }
         float pr[8], ds[8];
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
+        for (int mb = 0; mb < 2; mb++) {
+          const bool hv = !TILE || (q0 + 32 * qb_ + 16 * mb >= vlo[p] && q0 + 32 * qb_ + 16 * mb < vhi[p]);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             float pv = fast_exp2(fmaf(s[mb][i], scale, -lq[mb][i]));
@@ -540,9 +697,11 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
               const int qi = q0 + 32 * qb_ + 16 * mb + 4 * g + i;
               pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
             }
+            if (TILE) pv = hv ? pv : 0.f;
             pr[4 * mb + i] = pv;
             ds[4 * mb + i] = pv * (dp[mb][i] - dl[mb][i]);
           }
+        }
         pb[p] = pack8<CT>(pr);
         dsb[p] = pack8<CT>(ds);
       }
@@ -550,13 +709,15 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
       for (int d = 0; d < VB; d++) {
         const u32x4 dt = lds_read_tokens_as_k(sDO, PD, 32 * qb_, 16 * d, n, g);
 #pragma unroll
-        for (int p = 0; p < NP; p++) dv_acc[p][d] = Mma<CT>::mfma(dt, pb[p], dv_acc[p][d]);
+        for (int p = 0; p < NP; p++)
+          if (bv[p]) dv_acc[p][d] = Mma<CT>::mfma(dt, pb[p], dv_acc[p][d]);
       }
 #pragma unroll
       for (int d = 0; d < KB; d++) {
         const u32x4 qt = lds_read_tokens_as_k(sQ, PQ, 32 * qb_, 16 * d, n, g);
 #pragma unroll
-        for (int p = 0; p < NP; p++) dk_acc[p][d] = Mma<CT>::mfma(qt, dsb[p], dk_acc[p][d]);
+        for (int p = 0; p < NP; p++)
+          if (bv[p]) dk_acc[p][d] = Mma<CT>::mfma(qt, dsb[p], dk_acc[p][d]);
       }
     }
     __syncthreads();
@@ -568,6 +729,6 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
   }
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
-  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, a.dks[2], a.dks[3], a.dk_, a.dk_vec != 0, x0, a.Lk, wave, n, g, tid);
-  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.dv_, a.dv_vec != 0, x0, a.Lk, wave, n, g, tid);
+  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, a.dks[2], a.dks[3], a.dk_, a.dk_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
+  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.dv_, a.dv_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
 }
