@@ -392,8 +392,18 @@ def main():
         msd, _ = Timer.run(wd.step, max(K // 5, 3), 2)
         fd = wd.flops_fwd + wd.flops_bwd
         extra["ref_demo_b16"] = {"ms_per_step": msd, "eff_tflops": fd / (msd * 1e-3) / 1e12,
-                                 "workload": "B=4 H=8 16x16 tiles of 16 tokens, d=32, 3x3 window, fp16, fwd+bwd"}
+                                 "workload": "B=4 H=8 16x16 tiles of 16 tokens, d=32, 3x3 window, fp16, fwd+bwd (src/tiled_swa.py:736-750)"}
         del wd
+        # larger tiles: B=2, H=8, 16x16 tiles of 64 tokens (N = 16384), d=64, 3x3 tile window, bf16
+        wt = SwaWorkload("tiles_b64", 2, 8, 16, 16, 1, 64, fused_rope=False, nsets=1, b_size=64)
+        mst, _ = Timer.run(wt.step, max(K // 5, 3), 2)
+        kbt = kernel_breakdown(wt.step, 3)
+        ft = wt.flops_fwd + wt.flops_bwd
+        extra["tiles_b64_d64"] = {"ms_per_step": mst, "eff_tflops": ft / (mst * 1e-3) / 1e12,
+                                  "frac_mfma_peak": ft / (mst * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                                  "kernels_ms": {k_: v_["avg_ms"] for k_, v_ in kbt.items()},
+                                  "workload": "B=2 H=8 16x16 tiles of 64 tokens, d=64, 3x3 tile window, bf16, fwd+bwd"}
+        del wt
         # the shape the reference publishes flash numbers for (B=4, H=32, d=64, fp16, sm_scale 1.3,
         # src/flash_attn.py:548,580-586; its CSVs name no hardware), at N_CTX = 4096
         ref = {}
