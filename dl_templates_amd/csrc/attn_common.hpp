@@ -60,6 +60,24 @@ DLT_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 DLT_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 DLT_DEV float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
+// Values loaded from HBM before a streaming loop and first used inside it (own-token fragments,
+// per-token scalars).  Left alone, the compiler places the wait for them at the first use INSIDE
+// the loop as `s_waitcnt vmcnt(0)`, which on every iteration also waits for the chunk prefetch that
+// was issued just before, i.e. the prefetch never overlaps the products.  Consuming the values here
+// moves that wait in front of the loop (loads complete in order).
+DLT_DEV void pin_loaded(const u32x4& v) { asm volatile("" ::"v"(v)); }
+DLT_DEV void pin_loaded(float v) { asm volatile("" ::"v"(v)); }
+template <int N>
+DLT_DEV void pin_loaded(const u32x4 (&f)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; i++) pin_loaded(f[i]);
+}
+template <int M, int N>
+DLT_DEV void pin_loaded(const u32x4 (&f)[M][N]) {
+#pragma unroll
+  for (int i = 0; i < M; i++) pin_loaded(f[i]);
+}
+
 DLT_DEV u32x4 lds_read16(const char* p) { return *reinterpret_cast<const u32x4*>(p); }
 DLT_DEV void lds_write16(char* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 

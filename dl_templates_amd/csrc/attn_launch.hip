@@ -264,15 +264,21 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   d.o_vec = vec_ok(t.o, t.os, 4, p.dv, 2);
   d.do_vec = 1;
   d.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
-  int rc = dc.id == 0 ? dlt_launch_delta_64_64(d, stream) : dc.id == 1 ? dlt_launch_delta_128_128(d, stream)
-         : dc.id == 3 ? dlt_launch_delta_32_32(d, stream) : dlt_launch_delta_64_128(d, stream);
-  if (rc != DLT_OK) return rc;
+  // delta = rowsum(o * dO): folded into the dQ kernel when o can be read in 16-byte pieces
+  const bool fuse_delta = vec_ok(t.o, t.os, 4, p.dv, 2) && (int64_t)p.g.TR * p.g.XLq * t.os[2] * 2 < ((int64_t)1 << 31);
+  if (!fuse_delta) {
+    int rc = dc.id == 0 ? dlt_launch_delta_64_64(d, stream) : dc.id == 1 ? dlt_launch_delta_128_128(d, stream)
+           : dc.id == 3 ? dlt_launch_delta_32_32(d, stream) : dlt_launch_delta_64_128(d, stream);
+    if (rc != DLT_OK) return rc;
+  }
 
   FlashBwdArgs a;
-  a.q = t.q; a.k = t.k; a.v = t.v; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.o; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.delta_out = t.delta;
+  a.fuse_delta = fuse_delta ? 1 : 0;
   a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
   for (int i = 0; i < 4; i++) {
-    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.dos[i] = t.dos[i];
+    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; a.dos[i] = t.dos[i];
     a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
   }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];

@@ -37,15 +37,7 @@ int flash_set_lds(KernT kern, int bytes) {
 
 template <typename TIO, int MODE>
 int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
-  {
-    auto kern = flash_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, flash_np_kv(DLT_DK, DLT_DV), FLASH_CK, MODE>;
-    int rc = flash_set_lds(kern, a.lds_kv);
-    if (rc != DLT_OK) return rc;
-    dlt_timing_before(DLT_K_BWD_KV, stream);
-    hipLaunchKernelGGL(kern, dim3(grid_kv), dim3(256), a.lds_kv, stream, a);
-    dlt_timing_after(stream);
-    DLT_CHECK_LAUNCH("flash dK/dV launch");
-  }
+  // dQ first: with fuse_delta it produces the delta vector the dK/dV kernel consumes
   {
     auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK, MODE>;
     int rc = flash_set_lds(kern, a.lds_q);
@@ -54,6 +46,15 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
     hipLaunchKernelGGL(kern, dim3(grid_q), dim3(256), a.lds_q, stream, a);
     dlt_timing_after(stream);
     DLT_CHECK_LAUNCH("flash dQ launch");
+  }
+  {
+    auto kern = flash_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, flash_np_kv(DLT_DK, DLT_DV), FLASH_CK, MODE>;
+    int rc = flash_set_lds(kern, a.lds_kv);
+    if (rc != DLT_OK) return rc;
+    dlt_timing_before(DLT_K_BWD_KV, stream);
+    hipLaunchKernelGGL(kern, dim3(grid_kv), dim3(256), a.lds_kv, stream, a);
+    dlt_timing_after(stream);
+    DLT_CHECK_LAUNCH("flash dK/dV launch");
   }
   return DLT_OK;
 }

@@ -200,6 +200,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
 
   if (W.nchunks > 0) commit();
   __syncthreads();
+  pin_loaded(qf);
 
   for (int ci = 0; ci < W.nchunks; ci++) {
     const FlashChunk c = W.at(ci);
@@ -343,10 +344,12 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
 // (dK/dV pass over key blocks, dQ pass over query blocks) as two kernels; no host-side
 // pre-scaling pass over k (src/flash_attn.py:509-510), no atomics.
 struct FlashBwdArgs {
-  const void *q, *k, *v, *d_o;
+  const void *q, *k, *v, *o, *d_o;
   const float *lse, *delta;
+  float* delta_out;   // fuse_delta: the dQ kernel (launched first) stores delta = rowsum(o * dO) of its own queries
   void *dq, *dk, *dv;
-  int64_t qs[4], ks[4], vs[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int32_t fuse_delta;
   int32_t B, H, Lq, Lk, dk_, dv_;
   int32_t nblk_q, nblk_k;
   int32_t causal;
@@ -472,7 +475,25 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
     swa1_load_own<TIO, CT, DV>(dof[p], dob, a.dos[2], a.dv_, tq, g, no_rope, false);
     const int64_t off = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
     nlse[p] = tq >= 0 ? -a.lse[off] : 0.f;
-    del_n[p] = tq >= 0 ? a.delta[off] : 0.f;
+    if (a.fuse_delta != 0) {
+      // the reference's pre-pass (src/flash_attn.py:186-202) folded in: delta of the own queries
+      const TIO* ob = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1];
+      u32x4 of[VC];
+      swa1_load_own<TIO, CT, DV>(of, ob, a.os[2], a.dv_, tq, g, no_rope, false);
+      float part = 0.f;
+#pragma unroll
+      for (int c_ = 0; c_ < VC; c_++) {
+        float fo[8], fd[8];
+        unpack8<CT>(of[c_], fo);
+        unpack8<CT>(dof[p][c_], fd);
+#pragma unroll
+        for (int j = 0; j < 8; j++) part += fo[j] * fd[j];
+      }
+      del_n[p] = wave_sum4(part);
+      if (g == 0 && tq >= 0) a.delta_out[off] = del_n[p];
+    } else {
+      del_n[p] = tq >= 0 ? a.delta[off] : 0.f;
+    }
   }
   f32x4 dq_acc[NP][KB];
 #pragma unroll
@@ -483,6 +504,10 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
 
   if (W.nchunks > 0) st.commit(sK, PK, sV, PV);
   __syncthreads();
+  pin_loaded(qf);
+  pin_loaded(dof);
+#pragma unroll
+  for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
 
   for (int ci = 0; ci < W.nchunks; ci++) {
     const FlashChunk c = W.at(ci);
@@ -637,6 +662,8 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
     if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
   }
   __syncthreads();
+  pin_loaded(kf);
+  pin_loaded(vf);
 
   for (int ci = 0; ci < W.nchunks; ci++) {
     const FlashChunk c = W.at(ci);

@@ -45,13 +45,15 @@ DLT_DEV void swa1_issue_scalar(ScalarRegs<HCW, CR>& sr, const float* base, int64
       const int hr = idx / HCW, hc = idx - hr * HCW;
       const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + cr0 + hr, G.TR - 1));
       const int c = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));
-      sr.v[it] = base[(int64_t)(r * G.TC + c) * stride];
+      sr.v[it] = base[(uint32_t)((r * G.TC + c) * (int)stride)];
     }
   }
 }
 
 template <int HCW, int CR>
 DLT_DEV void swa1_commit_scalar(const ScalarRegs<HCW, CR>& sr, float* s, int tid) {
+#pragma unroll
+  for (int it = 0; it < (CR * HCW + 255) / 256; it++) pin_loaded(sr.v[it]);  // the wait, on every path
 #pragma unroll
   for (int it = 0; it < (CR * HCW + 255) / 256; it++) {
     const int idx = tid + 256 * it;
@@ -200,15 +202,12 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
   __syncthreads();
+  pin_loaded(kf);
+  pin_loaded(vf);
 
-  for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
+  // products of the chunk resident in LDS
+  auto consume = [&](const int ch) {
     const int cr0 = CR * ch;
-    if (ch < L.ch_last) {
-      swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, cr0 + CR, rope_idx);
-      swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, cr0 + CR, nullptr);
-      swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, cr0 + CR, tid);
-      swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, cr0 + CR, tid);
-    }
     float rbias[2];
 #pragma unroll
     for (int mb = 0; mb < 2; mb++) {
@@ -255,15 +254,24 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
         dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dk_acc[d]);
       }
     }
+  };
+  // the last chunk is peeled off: prefetch and commit are unconditional inside the loop (see the
+  // forward kernel)
+  for (int ch = L.ch_first; ch < L.ch_last; ch++) {
+    swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, CR * ch + CR, tid);
+    swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, CR * ch + CR, tid);
+    swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx);
+    swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr);
+    consume(ch);
     __syncthreads();
-    if (ch < L.ch_last) {
-      swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k);
-      swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
-      swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
-      swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
-      __syncthreads();
-    }
+    swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k);
+    swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
+    swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
+    swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
+    __syncthreads();
   }
+  consume(L.ch_last);
+  __syncthreads();
 
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
@@ -360,13 +368,14 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k);
   swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
   __syncthreads();
+  pin_loaded(qf);
+  pin_loaded(dof);
+  pin_loaded(lse_n);
+  pin_loaded(del_n);
 
-  for (int ch = L.ch_first; ch <= L.ch_last; ch++) {
+  // products of the chunk resident in LDS
+  auto consume = [&](const int ch) {
     const int cr0 = CR * ch;
-    if (ch < L.ch_last) {
-      swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
-      swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
-    }
     float rbias[2];
 #pragma unroll
     for (int mb = 0; mb < 2; mb++) {
@@ -406,13 +415,18 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
       for (int d = 0; d < DB; d++)
         dq_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sK, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dq_acc[d]);
     }
+  };
+  for (int ch = L.ch_first; ch < L.ch_last; ch++) {
+    swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx);
+    swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr);
+    consume(ch);
     __syncthreads();
-    if (ch < L.ch_last) {
-      swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k);
-      swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
-      __syncthreads();
-    }
+    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k);
+    swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
+    __syncthreads();
   }
+  consume(L.ch_last);
+  __syncthreads();
 
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
   if (a.dq_vec != 0) {

@@ -133,6 +133,15 @@ DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, con
 template <typename CT, int NI, bool BAL, int ROT>
 DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, int pbit, const RopeDev& rope, bool use_rope) {
   static_assert(ROT != 2 || BAL, "pair rotation needs the balanced mapping");
+  // wait for the staged loads HERE, on every path: a wait placed inside the per-thread `if` below
+  // would be skipped when no lane has an item, and the compiler would then treat the loads as
+  // possibly pending in the next iteration (a full wait in front of every new load)
+#pragma unroll
+  for (int it = 0; it < NI; it++) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) pin_loaded(sr.v[it][j]);
+    if (ROT != 0) asm volatile("" ::"v"(sr.id[it]));
+  }
 #pragma unroll
   for (int it = 0; it < NI; it++) {
     if (sp.loff[it] < 0) continue;

@@ -132,13 +132,11 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k);
   swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
   __syncthreads();
+  pin_loaded(qf);
 
-  for (int ch = ch_first; ch <= ch_last; ch++) {
+  // products and softmax update of the chunk resident in LDS
+  auto consume = [&](const int ch) {
     const int cr0 = CR * ch;
-    if (ch < ch_last) {  // next chunk: HBM -> registers while this one is consumed
-      swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, cr0 + CR, rope_idx);
-      swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, cr0 + CR, nullptr);
-    }
 
     // block kb, half mb -> (row offset inside the chunk, column group)
     float t[NKB][8];
@@ -219,13 +217,22 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
         if (ONES) acc_l = Mma<CT>::mfma(ones, pb[kb], acc_l);
       }
     }
+  };
+  // The last chunk is peeled off so that inside the loop the prefetch and the commit are
+  // unconditional: with `if (has_next)` around each, the compiler sees a path on which loads stay
+  // pending across the back edge and guards every later load with a full vmcnt(0) wait.
+  for (int ch = ch_first; ch < ch_last; ch++) {
+    // next chunk: HBM -> registers while this one is consumed
+    swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx);
+    swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr);
+    consume(ch);
     __syncthreads();  // every wave is done with this chunk
-    if (ch < ch_last) {
-      swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k);
-      swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
-      __syncthreads();
-    }
+    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k);
+    swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
+    __syncthreads();
   }
+  consume(ch_last);
+  __syncthreads();
 
   // ---- epilogue
   typedef typename TileOf<TIO>::type TL;
