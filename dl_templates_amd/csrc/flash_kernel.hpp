@@ -29,6 +29,9 @@ constexpr int FLASH_NP = FLASH_NP_DEF;  // 16-query blocks per wave (forward and
 constexpr int FLASH_CK = FLASH_CK_DEF;  // streamed tokens per LDS chunk
 // key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
 constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 128 ? 1 : 2; }
+// resident workgroups per CU the register allocation aims for (spill-free at these settings)
+constexpr int flash_occ_fwd(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 3 : 2); }
+constexpr int flash_occ_bwd(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 192 ? 3 : 2); }
 
 // One chunk of streamed tokens: first token (index inside the [N, D] slab), its x inside the grid
 // row (tile mode) or the sequence, and how many of the CK staged tokens exist.
@@ -101,7 +104,7 @@ struct FlashArgs {
 };
 
 template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
-__global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
+__global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(const FlashArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef typename TileOf<TIO>::type TL;
   extern __shared__ __align__(16) char smem[];
@@ -160,6 +163,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
     }
   };
   auto commit = [&]() {
+    pin_loaded(rk);
+    pin_loaded(rv);
 #pragma unroll
     for (int it = 0; it < NKI; it++) lds_write16(sK + (kkey0 + it * (256 / KCH)) * PK + 16 * kc_, rk[it]);
 #pragma unroll
@@ -202,11 +207,10 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
   __syncthreads();
   pin_loaded(qf);
 
-  for (int ci = 0; ci < W.nchunks; ci++) {
+  // products and softmax update of the chunk resident in LDS
+  auto consume = [&](const int ci) {
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
-    const bool has_next = ci + 1 < W.nchunks;
-    if (has_next) issue(W.at(ci + 1));
     // dense / causal: some keys of this chunk lie past the end or (causal) above the wave's first query
     const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && k0 + CK - 1 > wq0));
     // causal: every key of the chunk lies above every query of this wave (wave-uniform)
@@ -313,12 +317,19 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_kernel(const FlashArgs a) {
           if (bv[p][kb]) acc_l[p] = Mma<CT>::mfma(ones, pb[p][kb], acc_l[p]);
       }
     }
+  };
+  // The last chunk is peeled off so that prefetch and commit are unconditional inside the loop:
+  // with `if (has_next)` around each, the compiler sees a path on which loads stay pending across
+  // the back edge and guards every later load with a full vmcnt(0) wait.
+  for (int ci = 0; ci + 1 < W.nchunks; ci++) {
+    issue(W.at(ci + 1));
+    consume(ci);
     __syncthreads();
-    if (has_next) {
-      commit();
-      __syncthreads();
-    }
+    commit();
+    __syncthreads();
   }
+  if (W.nchunks > 0) consume(W.nchunks - 1);
+  __syncthreads();
 
   // ---- epilogue: normalise, O^T fragments -> LDS tile -> coalesced rows
 #pragma unroll
@@ -393,6 +404,8 @@ struct PairStage {
     }
   }
   DLT_DEV void commit(char* sa, int pa, char* sb, int pb) const {
+    pin_loaded(ra);
+    pin_loaded(rb);
 #pragma unroll
     for (int it = 0; it < NAI; it++) lds_write16(sa + (akey0 + it * (256 / ACH)) * pa + 16 * ac, ra[it]);
 #pragma unroll
@@ -423,7 +436,7 @@ DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO
 
 // ---- dQ: own = queries, K and V stream
 template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
-__global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs a) {
+__global__ __launch_bounds__(256, flash_occ_bwd(DK, DV)) void flash_bwd_q_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
@@ -509,11 +522,9 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
 #pragma unroll
   for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
 
-  for (int ci = 0; ci < W.nchunks; ci++) {
+  auto consume = [&](const int ci) {
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
-    const bool has_next = ci + 1 < W.nchunks;
-    if (has_next) st.issue(kb_, sn2k, vb_, sn2v, W.at(ci + 1));
     const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && k0 + CK - 1 > wq0));
     const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
 #pragma unroll
@@ -570,19 +581,24 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_q_kernel(const FlashBwdArgs 
           if (bv[p]) dq_acc[p][d] = Mma<CT>::mfma(kt, dsb[p], dq_acc[p][d]);
       }
     }
+  };
+  // last chunk peeled off: unconditional prefetch and commit inside the loop (see the forward kernel)
+  for (int ci = 0; ci + 1 < W.nchunks; ci++) {
+    st.issue(kb_, sn2k, vb_, sn2v, W.at(ci + 1));
+    consume(ci);
     __syncthreads();
-    if (has_next) {
-      st.commit(sK, PK, sV, PV);
-      __syncthreads();
-    }
+    st.commit(sK, PK, sV, PV);
+    __syncthreads();
   }
+  if (W.nchunks > 0) consume(W.nchunks - 1);
+  __syncthreads();
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
   flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, a.dqs[2], a.dqs[3], a.dk_, a.dq_vec != 0, own_base, x0, a.Lq, wave, n, g, tid);
 }
 
 // ---- dK / dV: own = keys, Q, dO, lse2 and delta stream
 template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
-__global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
+__global__ __launch_bounds__(256, flash_occ_bwd(DK, DV)) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
@@ -665,15 +681,9 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
   pin_loaded(kf);
   pin_loaded(vf);
 
-  for (int ci = 0; ci < W.nchunks; ci++) {
+  auto consume = [&](const int ci) {
     const FlashChunk c = W.at(ci);
     const int q0 = c.x;
-    const bool has_next = ci + 1 < W.nchunks;
-    if (has_next) {
-      const FlashChunk cn = W.at(ci + 1);
-      st.issue(qb, sn2q, dob, sn2d, cn);
-      issue_scalars(cn);
-    }
     // some queries of the chunk lie past the end or (causal) below the wave's last own key
     const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && q0 < wk0 + 16 * NP - 1));
     // causal: every query of the chunk lies below every own key of this wave
@@ -747,13 +757,21 @@ __global__ __launch_bounds__(256, 2) void flash_bwd_kv_kernel(const FlashBwdArgs
           if (bv[p]) dk_acc[p][d] = Mma<CT>::mfma(qt, dsb[p], dk_acc[p][d]);
       }
     }
+  };
+  for (int ci = 0; ci + 1 < W.nchunks; ci++) {
+    const FlashChunk cn = W.at(ci + 1);
+    st.issue(qb, sn2q, dob, sn2d, cn);
+    issue_scalars(cn);
+    consume(ci);
     __syncthreads();
-    if (has_next) {
-      st.commit(sQ, PQ, sDO, PD);
-      if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
-      __syncthreads();
-    }
+    st.commit(sQ, PQ, sDO, PD);
+    pin_loaded(r_lse);
+    pin_loaded(r_del);
+    if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
+    __syncthreads();
   }
+  if (W.nchunks > 0) consume(W.nchunks - 1);
+  __syncthreads();
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
   flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, a.dks[2], a.dks[3], a.dk_, a.dk_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
