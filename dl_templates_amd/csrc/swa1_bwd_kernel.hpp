@@ -177,6 +177,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
   StageRegs<NI> srq, srd;
   swa1_regs_zero(srq);
+  TabRegs<NI> tr_srq;
   swa1_regs_zero(srd);
   swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx);
   swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr);
@@ -197,7 +198,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   for (int d = 0; d < DB; d++) { dk_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; dv_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
   const float scale = a.scale_log2;
 
-  swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k);
+  if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
+  swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq);
   swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
   swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
@@ -263,8 +265,9 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
     swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx);
     swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr);
     consume(ch);
+    if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k);
+    swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq);
     swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
     swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
     swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
@@ -328,6 +331,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
+  TabRegs<NI> tr_srk;
   swa1_regs_zero(srv);
   swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx);
   swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr);
@@ -365,7 +369,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   for (int d = 0; d < DB; d++) dq_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float scale = a.scale_log2;
 
-  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k);
+  if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
+  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk);
   swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
   __syncthreads();
   pin_loaded(qf);
@@ -420,8 +425,9 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
     swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx);
     swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr);
     consume(ch);
+    if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k);
+    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk);
     swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
     __syncthreads();
   }

@@ -127,11 +127,36 @@ DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, con
   }
 }
 
+// Table values of the rotary pair each staged item of the balanced map needs, fetched ahead of
+// the commit: the load depends on the token index that arrived with the chunk, and issuing it before
+// the workgroup barrier lets its latency overlap the wait for the other waves.
+template <int NI>
+struct TabRegs {
+  f32x4 t[NI][4];   // (cos, sin) of the 8 pair elements
+  bool rot[NI];     // the token has this axis rotated
+};
+
+template <int NI>
+DLT_DEV void swa1_tab_issue(TabRegs<NI>& tr, const StageRegs<NI>& sr, const StagePlan<NI>& sp, const RopeDev& rope) {
+#pragma unroll
+  for (int it = 0; it < NI; it++) {
+    bool rotated;
+    const float* tab = rope_table_row(rope, sp.axis, sr.id[it], rotated) + sp.tab_off;
+    tr.rot[it] = rotated;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const float* tj = tab + 4 * j;
+      tr.t[it][j] = f32x4{tj[0], tj[1], tj[2], tj[3]};
+    }
+  }
+}
+
 // Rotate (K / Q side only) and write the staged registers into an LDS chunk.
 // ROT: 0 no rotation, 1 rotation with the plain chunk mapping, 2 rotation of the balanced
 // mapping's pair (chunks 0 and 1).  pbit: chunk distance between rotary partners (1 or 2).
 template <typename CT, int NI, bool BAL, int ROT>
-DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, int pbit, const RopeDev& rope, bool use_rope) {
+DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, int pbit, const RopeDev& rope, bool use_rope,
+                         const TabRegs<NI>* tr = nullptr) {
   static_assert(ROT != 2 || BAL, "pair rotation needs the balanced mapping");
   // wait for the staged loads HERE, on every path: a wait placed inside the per-thread `if` below
   // would be skipped when no lane has an item, and the compiler would then treat the loads as
@@ -141,20 +166,22 @@ DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, in
 #pragma unroll
     for (int j = 0; j < 4; j++) pin_loaded(sr.v[it][j]);
     if (ROT != 0) asm volatile("" ::"v"(sr.id[it]));
+    if (ROT == 2) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) asm volatile("" ::"v"(tr->t[it][j]));
+    }
   }
 #pragma unroll
   for (int it = 0; it < NI; it++) {
     if (sp.loff[it] < 0) continue;
     if (ROT == 2 && use_rope) {
-      bool rotated;
-      const float* tab = rope_table_row(rope, sp.axis, sr.id[it], rotated) + sp.tab_off;
-      if (rotated) {
+      if (tr->rot[it]) {
         float x0[8], x1[8];
         unpack8<CT>(sr.v[it][0], x0);
         unpack8<CT>(sr.v[it][1], x1);
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-          const float cs = tab[2 * j], sn = tab[2 * j + 1];
+          const float cs = tr->t[it][j >> 1][2 * (j & 1)], sn = tr->t[it][j >> 1][2 * (j & 1) + 1];
           const float y0 = rope_mix(x0[j], x1[j], cs, sn, true);
           const float y1 = rope_mix(x1[j], x0[j], cs, sn, false);
           x0[j] = y0; x1[j] = y1;
@@ -267,26 +294,65 @@ DLT_DEV void swa1_store_own(char* sW, const f32x4 (&acc)[D / 16], float mul, TIO
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  constexpr int NIT = 16 * CH / 64;
+  int tok[NIT];
+  bool ok[NIT];
 #pragma unroll
-  for (int it = 0; it < 16 * CH / 64; it++) {
+  for (int it = 0; it < NIT; it++) {
     const int p = lane + 64 * it;
     const int row = p / CH, c = p % CH;
     const int r = G.r0 + (row >> 2), col = G.c0 + 4 * wave + (row & 3);
-    if (r < G.TR && col < G.TC && 8 * c < dact) {
-      const int tok = r * G.TC + col;
+    ok[it] = r < G.TR && col < G.TC && 8 * c < dact;
+    tok[it] = ok[it] ? r * G.TC + col : 0;
+  }
+  if (use_rope) {
+    // The rotation needs two dependent global loads per piece (token index, then its table row).
+    // They are issued in phases over all pieces of the lane, with clamped addresses instead of
+    // branches, so that their latencies overlap instead of adding up.
+    int32_t id[NIT];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) id[it] = rope.idx[tok[it]];
+    RopeChunk rc[NIT];
+    bool rot[NIT];
+    f32x4 tv[NIT][4];
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      const int c = (lane + 64 * it) % CH;
+      rc[it] = rope_chunk_setup(rope, c, true);
+      bool rotated;
+      const float* tab = rope_table_row(rope, rc[it].axis, id[it], rotated) + rc[it].tab_off;
+      rot[it] = ok[it] && rc[it].mode == 1 && rotated;
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const float* tj = tab + 4 * j;
+        tv[it][j] = f32x4{tj[0], tj[1], tj[2], tj[3]};
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      const int p = lane + 64 * it;
+      const int row = p / CH, c = p % CH;
       const char* lrow = sW + row * PT;
       u32x4 v = lds_read16(lrow + 16 * c);
-      if (use_rope) {
-        const RopeChunk rc = rope_chunk_setup(rope, c, true);
-        if (rc.mode == 1) {
-          float self[8], partner[8];
-          unpack8<CT>(v, self);
-          unpack8<CT>(lds_read16(lrow + 16 * rc.partner_c), partner);
-          rope_apply8(rope, rc, c, rope.idx[tok], self, partner, [](int) { return 0.f; });
-          v = pack8<CT>(self);
+      if (rot[it]) {
+        float self[8], partner[8];
+        unpack8<CT>(v, self);
+        unpack8<CT>(lds_read16(lrow + 16 * rc[it].partner_c), partner);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+          const float cs = tv[it][j >> 1][2 * (j & 1)], sn_ = tv[it][j >> 1][2 * (j & 1) + 1];
+          self[j] = rope_mix(self[j], partner[j], cs, rope.inverse ? -sn_ : sn_, rc[it].is_x0);
         }
+        v = pack8<CT>(self);
       }
-      *reinterpret_cast<u32x4*>(base + (int64_t)tok * sn + 8 * c) = v;
+      if (ok[it]) *reinterpret_cast<u32x4*>(base + (int64_t)tok[it] * sn + 8 * c) = v;
+    }
+  } else {
+#pragma unroll
+    for (int it = 0; it < NIT; it++) {
+      const int p = lane + 64 * it;
+      const int row = p / CH, c = p % CH;
+      if (ok[it]) *reinterpret_cast<u32x4*>(base + (int64_t)tok[it] * sn + 8 * c) = lds_read16(sW + row * PT + 16 * c);
     }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -92,6 +92,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
+  TabRegs<NI> tr_srk;
   swa1_regs_zero(srv);
   swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx);
   swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr);
@@ -129,7 +130,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const unsigned one2 = pack2<CT>(1.f, 1.f);
   const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
 
-  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k);
+  if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, a.p.rope);
+  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk);
   swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
   __syncthreads();
   pin_loaded(qf);
@@ -226,8 +228,9 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
     swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx);
     swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr);
     consume(ch);
+    if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, a.p.rope);  // table rows of the next chunk's tokens, ahead of the barrier
     __syncthreads();  // every wave is done with this chunk
-    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k);
+    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk);
     swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
     __syncthreads();
   }
