@@ -170,17 +170,18 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  constexpr int NI = swa1_items(D, HCW, CR);
+  constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
+  constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR, BAL>(sp, G, PITCH, tid, a.rope_pbit);
+  swa1_plan_init<D, HCW, CR, BAL, TAIL>(sp, G, PITCH, tid, a.rope_pbit);
   const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
   StageRegs<NI> srq, srd;
   swa1_regs_zero(srq);
   TabRegs<NI> tr_srq;
   swa1_regs_zero(srd);
-  swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx);
-  swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr);
+  swa1_issue<NI, BAL, TAIL>(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
+  swa1_issue<NI, BAL, TAIL>(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
   ScalarRegs<HCW, CR> r_lse, r_del;
   swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, CR * L.ch_first, tid);
   swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, CR * L.ch_first, tid);
@@ -199,8 +200,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   const float scale = a.scale_log2;
 
   if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
-  swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq);
-  swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
+  swa1_commit<CT, NI, BAL, ROPE, TAIL>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
+  swa1_commit<CT, NI, BAL, 0, TAIL>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
   __syncthreads();
@@ -262,13 +263,13 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   for (int ch = L.ch_first; ch < L.ch_last; ch++) {
     swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, CR * ch + CR, tid);
     swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, CR * ch + CR, tid);
-    swa1_issue<NI, BAL>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx);
-    swa1_issue<NI, BAL>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr);
+    swa1_issue<NI, BAL, TAIL>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
+    swa1_issue<NI, BAL, TAIL>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
     if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq);
-    swa1_commit<CT, NI, BAL, 0>(srd, sp, sDO, 1, no_rope, false);
+    swa1_commit<CT, NI, BAL, ROPE, TAIL>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, 0, TAIL>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
     swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
     __syncthreads();
@@ -324,17 +325,18 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  constexpr int NI = swa1_items(D, HCW, CR);
+  constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
+  constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR, BAL>(sp, G, PITCH, tid, a.rope_pbit);
+  swa1_plan_init<D, HCW, CR, BAL, TAIL>(sp, G, PITCH, tid, a.rope_pbit);
   const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   TabRegs<NI> tr_srk;
   swa1_regs_zero(srv);
-  swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx);
-  swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr);
+  swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
+  swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
 
   // own queries / output gradients straight into B-operand fragments
   u32x4 qf[KC], dof[KC];
@@ -370,8 +372,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   const float scale = a.scale_log2;
 
   if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
-  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk);
-  swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
+  swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+  swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   __syncthreads();
   pin_loaded(qf);
   pin_loaded(dof);
@@ -422,13 +424,13 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
     }
   };
   for (int ch = L.ch_first; ch < L.ch_last; ch++) {
-    swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx);
-    swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr);
+    swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
+    swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
     if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk);
-    swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, no_rope, false);
+    swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     __syncthreads();
   }
   consume(L.ch_last);

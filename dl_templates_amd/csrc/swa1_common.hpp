@@ -28,6 +28,14 @@ constexpr int swa1_hcw(int ncgmax) { return 12 + 4 * ncgmax; }
 
 // 64-byte items (4 chunks of 8 dims of one token) a thread stages per 8-row chunk of one tensor
 constexpr int swa1_items(int d, int hcw, int cr = 8) { return (cr * hcw * (d / 32) + 255) / 256; }
+// Tail staging: when the 64-byte items of a chunk do not divide evenly over the 256 threads and the
+// remainder is at most 256 16-byte chunks, the remainder is staged one 16-byte chunk per thread
+// instead of one more (mostly idle) 64-byte item: 4 staging registers per tensor instead of 16.
+// Only without rotation (a rotary pair must sit in one thread).
+constexpr bool swa1_use_tail(int d, int hcw, int cr) {
+  return (cr * hcw * (d / 32)) / 256 >= 1 && (cr * hcw * (d / 32)) % 256 != 0 && ((cr * hcw * (d / 32)) % 256) * 4 <= 256;
+}
+constexpr int swa1_items_t(int d, int hcw, int cr, bool tail) { return tail ? (cr * hcw * (d / 32)) / 256 : swa1_items(d, hcw, cr); }
 
 struct Swa1Geom {
   int r0, c0;      // first grid row / column of the workgroup's band
@@ -52,15 +60,30 @@ struct StagePlan {
   int cc[NI];    // grid column, clamped
   int loff[NI];  // byte offset of the token row inside the LDS chunk, -1: no such item
   int coff[4];   // byte offsets of the thread's four 16-byte chunks inside a token row
+  int t_hr, t_cc;  // tail chunk: halo row and clamped grid column of its token
+  int t_loff;      // tail chunk: byte offset inside the LDS chunk, -1: this thread has none
+  int t_off;       // tail chunk: byte offset inside the token row
   int bal;       // balanced mapping: chunks 0 and 1 are a rotary pair
   int axis;      // balanced: 0 row angle, 1 column angle
   int tab_off;   // balanced: float offset of the pair's (cos, sin) values inside a table row
 };
 
-template <int D, int HCW, int CR, bool BAL>
-DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW, CR)>& sp, const Swa1Geom& G, int pitch, int tid, int bal_r8) {
+template <int D, int HCW, int CR, bool BAL, bool TAIL = false>
+DLT_DEV void swa1_plan_init(StagePlan<swa1_items_t(D, HCW, CR, TAIL)>& sp, const Swa1Geom& G, int pitch, int tid, int bal_r8) {
   constexpr int QUADS = D / 32;
   const int qd = tid % QUADS, key0 = tid / QUADS;
+  sp.t_hr = 0; sp.t_cc = dlt_imax(0, dlt_imin(G.c0 - G.WC, G.TC - 1)); sp.t_loff = -1; sp.t_off = 0;
+  if (TAIL) {
+    constexpr int FULL = (CR * HCW * QUADS) / 256, REM = (CR * HCW * QUADS) % 256;
+    if (tid < REM * 4) {
+      const int ti = FULL * 256 + (tid >> 2);
+      const int key = ti / QUADS;
+      sp.t_off = 64 * (ti % QUADS) + 16 * (tid & 3);
+      sp.t_hr = key / HCW;
+      sp.t_cc = dlt_imax(0, dlt_imin(G.c0 - G.WC + (key - sp.t_hr * HCW), G.TC - 1));
+      sp.t_loff = key * pitch + sp.t_off;
+    }
+  }
   sp.bal = BAL;
   if (BAL) {
     const int region2 = qd / bal_r8, ci = qd - region2 * bal_r8;
@@ -78,7 +101,7 @@ DLT_DEV void swa1_plan_init(StagePlan<swa1_items(D, HCW, CR)>& sp, const Swa1Geo
     sp.tab_off = 0;
   }
 #pragma unroll
-  for (int it = 0; it < swa1_items(D, HCW, CR); it++) {
+  for (int it = 0; it < swa1_items_t(D, HCW, CR, TAIL); it++) {
     const int key = key0 + it * (256 / QUADS);
     const bool live = key < CR * HCW;
     const int k = live ? key : 0;
@@ -95,6 +118,7 @@ template <int NI>
 struct StageRegs {
   u32x4 v[NI][4];
   int32_t id[NI];  // packed rotary index of the token
+  u32x4 tv;        // tail chunk
 };
 
 template <int NI>
@@ -105,15 +129,22 @@ DLT_DEV void swa1_regs_zero(StageRegs<NI>& sr) {
     for (int j = 0; j < 4; j++) sr.v[it][j] = u32x4{0u, 0u, 0u, 0u};
     sr.id[it] = -1;
   }
+  sr.tv = u32x4{0u, 0u, 0u, 0u};
 }
 
 // Issue the global loads of halo rows [cr0, cr0 + 8) into registers.  `sn2` is the token stride
 // in BYTES; offsets are 32-bit (the host checks that a [N, D] slab stays below 2 GiB).  `on`:
 // the thread's 64-byte piece lies below the actual head dim (pieces above it stay zero).
-template <int NI, bool BAL>
+template <int NI, bool BAL, bool TAIL = false>
 DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, const void* base, int sn2, const Swa1Geom& G,
-                        int cr0, const int32_t* rope_idx) {
+                        int cr0, const int32_t* rope_idx, bool tail_on = false) {
   const int rbase = G.r0 - G.WR + cr0;
+  if (TAIL) {
+    // always a valid address (threads without a tail chunk re-read a token of the chunk)
+    const int r = dlt_imax(0, dlt_imin(rbase + sp.t_hr, G.TR - 1));
+    const char* p = reinterpret_cast<const char*>(base) + (uint32_t)((r * G.TC + sp.t_cc) * sn2 + (tail_on ? sp.t_off : 0));
+    sr.tv = *reinterpret_cast<const u32x4*>(p);
+  }
 #pragma unroll
   for (int it = 0; it < NI; it++) {
     const int r = dlt_imax(0, dlt_imin(rbase + sp.hr[it], G.TR - 1));
@@ -154,10 +185,15 @@ DLT_DEV void swa1_tab_issue(TabRegs<NI>& tr, const StageRegs<NI>& sr, const Stag
 // Rotate (K / Q side only) and write the staged registers into an LDS chunk.
 // ROT: 0 no rotation, 1 rotation with the plain chunk mapping, 2 rotation of the balanced
 // mapping's pair (chunks 0 and 1).  pbit: chunk distance between rotary partners (1 or 2).
-template <typename CT, int NI, bool BAL, int ROT>
+template <typename CT, int NI, bool BAL, int ROT, bool TAIL = false>
 DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, int pbit, const RopeDev& rope, bool use_rope,
-                         const TabRegs<NI>* tr = nullptr) {
+                         const TabRegs<NI>* tr = nullptr, bool tail_on = false) {
   static_assert(ROT != 2 || BAL, "pair rotation needs the balanced mapping");
+  static_assert(!TAIL || ROT == 0, "tail staging splits rotary pairs");
+  if (TAIL) {
+    pin_loaded(sr.tv);
+    if (sp.t_loff >= 0) lds_write16(s + sp.t_loff, tail_on ? sr.tv : u32x4{0u, 0u, 0u, 0u});
+  }
   // wait for the staged loads HERE, on every path: a wait placed inside the per-thread `if` below
   // would be skipped when no lane has an item, and the compiler would then treat the loads as
   // possibly pending in the next iteration (a full wait in front of every new load)

@@ -85,17 +85,18 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const int wrow_lo = dlt_imax(0, G.WR - G.r0), wrow_hi = dlt_imin(3 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
   const int ch_first = wrow_lo / CR, ch_last = wrow_hi / CR;
 
-  constexpr int NI = swa1_items(D, HCW, CR);
+  constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
+  constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR, BAL>(sp, G, PITCH, tid, a.rope_pbit);
+  swa1_plan_init<D, HCW, CR, BAL, TAIL>(sp, G, PITCH, tid, a.rope_pbit);
   const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   TabRegs<NI> tr_srk;
   swa1_regs_zero(srv);
-  swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx);
-  swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr);
+  swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
+  swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
 
   // own queries straight into B-operand fragments (rotated on the way when fused)
   u32x4 qf[KC];
@@ -131,8 +132,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
 
   if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, a.p.rope);
-  swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk);
-  swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
+  swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+  swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, a.p.rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   __syncthreads();
   pin_loaded(qf);
 
@@ -225,13 +226,13 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   // pending across the back edge and guards every later load with a full vmcnt(0) wait.
   for (int ch = ch_first; ch < ch_last; ch++) {
     // next chunk: HBM -> registers while this one is consumed
-    swa1_issue<NI, BAL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx);
-    swa1_issue<NI, BAL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr);
+    swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
+    swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
     if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, a.p.rope);  // table rows of the next chunk's tokens, ahead of the barrier
     __syncthreads();  // every wave is done with this chunk
-    swa1_commit<CT, NI, BAL, ROPE>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk);
-    swa1_commit<CT, NI, BAL, 0>(srv, sp, sV, 1, a.p.rope, false);
+    swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, a.p.rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     __syncthreads();
   }
   consume(ch_last);
