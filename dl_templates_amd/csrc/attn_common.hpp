@@ -65,6 +65,11 @@ DLT_DEV float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 // the loop as `s_waitcnt vmcnt(0)`, which on every iteration also waits for the chunk prefetch that
 // was issued just before, i.e. the prefetch never overlaps the products.  Consuming the values here
 // moves that wait in front of the loop (loads complete in order).
+// Placed at the top of a wave-uniform `if` body whose work is rarely needed (edge masks, the
+// accumulator rescale of the online softmax): the compiler otherwise turns the body into
+// unconditional select / multiply instructions that every iteration pays for.
+DLT_DEV void keep_branch() { asm volatile(""); }
+
 DLT_DEV void pin_loaded(const u32x4& v) { asm volatile("" ::"v"(v)); }
 DLT_DEV void pin_loaded(float v) { asm volatile("" ::"v"(v)); }
 template <int N>

@@ -292,6 +292,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
           pb[p][kb] = pack8<CT>(t[p][kb]);
         }
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+          keep_branch();
 #pragma unroll
           for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
           acc_l[p] *= alpha;
