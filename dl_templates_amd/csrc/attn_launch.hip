@@ -283,7 +283,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
   a.B = p.B; a.H = p.H; a.Lq = p.g.XLq; a.Lk = p.g.XLk; a.dk_ = p.dk; a.dv_ = p.dv;
-  const int own = 64 * FLASH_NP, own_kv = 64 * flash_np_kv(dc.DK, dc.DV);
+  const int own = 64 * flash_np_q(dc.DK, dc.DV), own_kv = 64 * flash_np_kv(dc.DK, dc.DV);
   a.nblk_q = (a.Lq + own - 1) / own;
   a.nblk_k = (a.Lk + own_kv - 1) / own_kv;
   a.causal = p.g.mode == DLT_GEOM_CAUSAL;

@@ -39,7 +39,7 @@ template <typename TIO, int MODE>
 int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
   // dQ first: with fuse_delta it produces the delta vector the dK/dV kernel consumes
   {
-    auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK, MODE>;
+    auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, flash_np_q(DLT_DK, DLT_DV), FLASH_CK, MODE>;
     int rc = flash_set_lds(kern, a.lds_q);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_Q, stream);

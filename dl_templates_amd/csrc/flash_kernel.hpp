@@ -29,9 +29,14 @@ constexpr int FLASH_NP = FLASH_NP_DEF;  // 16-query blocks per wave (forward and
 constexpr int FLASH_CK = FLASH_CK_DEF;  // streamed tokens per LDS chunk
 // key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
 constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 128 ? 1 : 2; }
+// query blocks per wave in the dQ kernel: one at 128/128 (accumulators, q and dO fragments of two blocks do not fit 256 registers)
+constexpr int flash_np_q(int dk, int dv) { return dk + dv > 192 ? 1 : FLASH_NP_DEF; }
 // resident workgroups per CU the register allocation aims for (spill-free at these settings)
 constexpr int flash_occ_fwd(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 3 : 2); }
-constexpr int flash_occ_bwd(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 192 ? 3 : 2); }
+constexpr int flash_occ_q(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 3 : 2); }
+constexpr int flash_occ_kv(int dk, int dv, int mode) {
+  return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 2 : (dk + dv <= 192 && mode != 2 ? 3 : 2));
+}
 
 // One chunk of streamed tokens: first token (index inside the [N, D] slab), its x inside the grid
 // row (tile mode) or the sequence, and how many of the CK staged tokens exist.
@@ -437,7 +442,7 @@ DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO
 
 // ---- dQ: own = queries, K and V stream
 template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
-__global__ __launch_bounds__(256, flash_occ_bwd(DK, DV)) void flash_bwd_q_kernel(const FlashBwdArgs a) {
+__global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
@@ -599,7 +604,7 @@ __global__ __launch_bounds__(256, flash_occ_bwd(DK, DV)) void flash_bwd_q_kernel
 
 // ---- dK / dV: own = keys, Q, dO, lse2 and delta stream
 template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
-__global__ __launch_bounds__(256, flash_occ_bwd(DK, DV)) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
+__global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
