@@ -34,19 +34,29 @@ struct Swa1BwdArgs {
 template <int HCW, int CR>
 struct ScalarRegs { float v[(CR * HCW + 255) / 256]; };
 
+// lse2 and delta share their indexing: the offsets are computed once and BEFORE the first load (an
+// address computation placed between two loads can end up waiting for the first one: the compiler
+// forms 32-bit multiply-adds with a 64-bit instruction whose unused upper addend half may be the
+// register the pending load writes).
 template <int HCW, int CR>
-DLT_DEV void swa1_issue_scalar(ScalarRegs<HCW, CR>& sr, const float* base, int64_t stride, const Swa1Geom& G, int cr0, int tid) {
+DLT_DEV void swa1_issue_scalar2(ScalarRegs<HCW, CR>& sa, ScalarRegs<HCW, CR>& sb, const float* base_a, const float* base_b,
+                                int64_t stride, const Swa1Geom& G, int cr0, int tid) {
+  constexpr int NS = (CR * HCW + 255) / 256;
+  uint32_t off[NS];
 #pragma unroll
-  for (int it = 0; it < (CR * HCW + 255) / 256; it++) {
-    const int idx = tid + 256 * it;
-    sr.v[it] = 0.f;
-    if (idx < CR * HCW) {
-      // clamped like the tile staging: out-of-grid halo positions are masked by the window bias
-      const int hr = idx / HCW, hc = idx - hr * HCW;
-      const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + cr0 + hr, G.TR - 1));
-      const int c = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));
-      sr.v[it] = base[(uint32_t)((r * G.TC + c) * (int)stride)];
-    }
+  for (int it = 0; it < NS; it++) {
+    // clamped like the tile staging: out-of-grid halo positions are masked by the window bias;
+    // threads past the end of the chunk re-read its first token (the value is not stored)
+    const int idx = dlt_imin(tid + 256 * it, CR * HCW - 1);
+    const int hr = idx / HCW, hc = idx - hr * HCW;
+    const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + cr0 + hr, G.TR - 1));
+    const int c = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));
+    off[it] = (uint32_t)((r * G.TC + c) * (int)stride);
+  }
+#pragma unroll
+  for (int it = 0; it < NS; it++) {
+    sa.v[it] = base_a[off[it]];
+    sb.v[it] = base_b[off[it]];
   }
 }
 
@@ -183,15 +193,14 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   swa1_issue<NI, BAL, TAIL>(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
   swa1_issue<NI, BAL, TAIL>(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
   ScalarRegs<HCW, CR> r_lse, r_del;
-  swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, CR * L.ch_first, tid);
-  swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, CR * L.ch_first, tid);
+  swa1_issue_scalar2<HCW, CR>(r_lse, r_del, lseb, delb, a.ls[2], G, CR * L.ch_first, tid);
 
   // own keys / values straight into B-operand fragments
   u32x4 kf[KC], vf[KC];
   {
     const int64_t tk = L.own_token(16 * wave + n);
-    swa1_load_own<TIO, CT, D>(kf, kb_, a.ks[2], a.p.dk, tk, g, fwd_rope, use_rope);
     swa1_load_own<TIO, CT, D>(vf, vb_, a.vs[2], a.p.dv, tk, g, no_rope, false);
+    swa1_load_own<TIO, CT, D>(kf, kb_, a.ks[2], a.p.dk, tk, g, fwd_rope, use_rope);
   }
 
   f32x4 dk_acc[DB], dv_acc[DB];
@@ -261,8 +270,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   // the last chunk is peeled off: prefetch and commit are unconditional inside the loop (see the
   // forward kernel)
   for (int ch = L.ch_first; ch < L.ch_last; ch++) {
-    swa1_issue_scalar<HCW, CR>(r_lse, lseb, a.ls[2], G, CR * ch + CR, tid);
-    swa1_issue_scalar<HCW, CR>(r_del, delb, a.ls[2], G, CR * ch + CR, tid);
+    swa1_issue_scalar2<HCW, CR>(r_lse, r_del, lseb, delb, a.ls[2], G, CR * ch + CR, tid);
     swa1_issue<NI, BAL, TAIL>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
     swa1_issue<NI, BAL, TAIL>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
@@ -338,19 +346,24 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
   swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
 
-  // own queries / output gradients straight into B-operand fragments
-  u32x4 qf[KC], dof[KC];
+  // own output gradients, outputs and queries straight into B-operand fragments.  Everything that
+  // needs no rotation is requested first; the rotated query fragments wait for their table rows last.
+  u32x4 qf[KC], dof[KC], of[KC];
   const int64_t tq = L.own_token(16 * wave + n);
-  swa1_load_own<TIO, CT, D>(qf, qb, a.qs[2], a.p.dk, tq, g, fwd_rope, use_rope);
-  swa1_load_own<TIO, CT, D>(dof, dob, a.dos[2], a.p.dv, tq, g, no_rope, false);
   const int64_t loff = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
-  const float lse_n = tq >= 0 ? a.lse[loff] : 0.f;
+  const float lse_ld = a.lse[loff];
+  const float del_ld = a.fuse_delta != 0 ? 0.f : a.delta[loff];
+  swa1_load_own<TIO, CT, D>(dof, dob, a.dos[2], a.p.dv, tq, g, no_rope, false);
+  {
+    // o is only needed when delta is computed here; otherwise dO is re-read (a valid address, unused)
+    const TIO* ob = a.fuse_delta != 0 ? reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1] : dob;
+    swa1_load_own<TIO, CT, D>(of, ob, a.fuse_delta != 0 ? a.os[2] : a.dos[2], a.p.dv, tq, g, no_rope, false);
+  }
+  swa1_load_own<TIO, CT, D>(qf, qb, a.qs[2], a.p.dk, tq, g, fwd_rope, use_rope);
+  const float lse_n = tq >= 0 ? lse_ld : 0.f;
   float del_n;
   if (a.fuse_delta != 0) {
     // delta of the own tokens, computed here and published for the dK/dV kernel that runs next
-    const TIO* ob = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1];
-    u32x4 of[KC];
-    swa1_load_own<TIO, CT, D>(of, ob, a.os[2], a.p.dv, tq, g, no_rope, false);
     float part = 0.f;
 #pragma unroll
     for (int c = 0; c < KC; c++) {
@@ -363,7 +376,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
     del_n = wave_sum4(part);
     if (g == 0 && tq >= 0) a.delta_out[loff] = del_n;
   } else {
-    del_n = tq >= 0 ? a.delta[loff] : 0.f;
+    del_n = tq >= 0 ? del_ld : 0.f;
   }
 
   f32x4 dq_acc[DB];

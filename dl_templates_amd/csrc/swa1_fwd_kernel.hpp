@@ -91,6 +91,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   swa1_plan_init<D, HCW, CR, BAL, TAIL>(sp, G, PITCH, tid, a.rope_pbit);
   const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
+  const int64_t tq_own = own_token(16 * wave + n);
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   TabRegs<NI> tr_srk;
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
 
   // own queries straight into B-operand fragments (rotated on the way when fused)
   u32x4 qf[KC];
-  swa1_load_own<TIO, CT, D>(qf, qb, a.qs[2], a.p.dk, own_token(16 * wave + n), g, a.p.rope, use_rope);
+  swa1_load_own<TIO, CT, D>(qf, qb, a.qs[2], a.p.dk, tq_own, g, a.p.rope, use_rope);
 
   // ---- window of this lane's query in halo coordinates -> additive biases
   const int qr_l = n >> 2, qc_l = n & 3;
