@@ -125,13 +125,15 @@ bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streame
 }
 
 // n_regions: [8 rows x HCW tokens] LDS regions the kernel keeps resident
-void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int extra_bytes, Swa1Plan& plan, int cr = 8) {
+void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int extra_bytes, Swa1Plan& plan, int cr = 8, bool kv = false) {
   plan.ncg = (4 + 2 * p.g.WC + 3) / 4;
   const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
   plan.HRP = roundup(4 + 2 * p.g.WR, cr);
   plan.nblk_r = (p.g.TR + 3) / 4;
   plan.nblk_c = (p.g.TC + 15) / 16;
-  plan.lds_bytes = n_regions * cr * hcw * (c.D * 2 + SWA1_PAD) + extra_bytes;
+  const int ncgmax = c.wclass == 0 ? 4 : 6;
+  const bool wide = c.rope_mode == 0;  // must match WIDE in the kernels
+  plan.lds_bytes = cr * hcw * (swa1_pitch(c.D, ncgmax, 0, wide, kv) + swa1_pitch(c.D, ncgmax, 1, wide, kv)) + extra_bytes;
   const int own_tile = 64 * (c.D * 2 + 16);  // output tile of the epilogue
   if (plan.lds_bytes < own_tile) plan.lds_bytes = own_tile;
 }
@@ -167,7 +169,7 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
   Swa1Plan plan_q;
   swa1_make_plan(p, c, 2, 0, plan_q, SWA1_FWD_CR);
   const int hcw = swa1_hcw(c.wclass == 0 ? 4 : 6);
-  swa1_make_plan(p, c, 2, 2 * SWA1_KV_CR * hcw * 4, a.plan, SWA1_KV_CR);
+  swa1_make_plan(p, c, 2, 2 * SWA1_KV_CR * hcw * 4, a.plan, SWA1_KV_CR, true);
   const int lds_q = plan_q.lds_bytes, lds_kv = a.plan.lds_bytes;
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.o; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
   a.delta_out = t.delta;

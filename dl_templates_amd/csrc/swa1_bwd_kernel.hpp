@@ -145,10 +145,11 @@ template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr int PITCH = D * 2 + SWA1_PAD;
+  constexpr bool WIDE = ROPE == 0;
+  constexpr int PA = swa1_pitch(D, NCGMAX, 0, WIDE, true), PB = swa1_pitch(D, NCGMAX, 1, WIDE, true);  // Q rows, dO rows
   constexpr int KC = D / 32, DB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
-  constexpr int REGION = CR * HCW * PITCH;
+  constexpr int REGION = CR * HCW * PA;
   constexpr int NKB = CR == 8 ? NCGMAX : NCGMAX / 2;
   constexpr int MB_STEP = CR == 8 ? 4 * HCW : 4;
 
@@ -158,7 +159,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   const Swa1Plan& P = a.plan;
   char* sQ = smem;
   char* sDO = smem + REGION;
-  float* sLse = reinterpret_cast<float*>(smem + 2 * REGION);
+  float* sLse = reinterpret_cast<float*>(smem + REGION + CR * HCW * PB);
   float* sDel = sLse + CR * HCW;
 
   Swa1Lane<NCGMAX> L;
@@ -183,15 +184,15 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
   constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR, BAL, TAIL>(sp, G, PITCH, tid, a.rope_pbit);
+  swa1_plan_init<D, HCW, CR, BAL, TAIL, WIDE, PA, PB>(sp, G, tid, a.rope_pbit);
   const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
   StageRegs<NI> srq, srd;
   swa1_regs_zero(srq);
   TabRegs<NI> tr_srq;
   swa1_regs_zero(srd);
-  swa1_issue<NI, BAL, TAIL>(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
-  swa1_issue<NI, BAL, TAIL>(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
+  swa1_issue<NI, BAL, TAIL, 0>(srq, sp, on_k, qb, sn2q, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
+  swa1_issue<NI, BAL, TAIL, 1>(srd, sp, on_v, dob, sn2d, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
   ScalarRegs<HCW, CR> r_lse, r_del;
   swa1_issue_scalar2<HCW, CR>(r_lse, r_del, lseb, delb, a.ls[2], G, CR * L.ch_first, tid);
 
@@ -209,8 +210,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   const float scale = a.scale_log2;
 
   if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
-  swa1_commit<CT, NI, BAL, ROPE, TAIL>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
-  swa1_commit<CT, NI, BAL, 0, TAIL>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
+  swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
+  swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
   __syncthreads();
@@ -239,8 +240,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
         dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KC; c++) {
-          s[mb] = Mma<CT>::mfma(lds_read16(sQ + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), kf[c], s[mb]);
-          dp[mb] = Mma<CT>::mfma(lds_read16(sDO + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), vf[c], dp[mb]);
+          s[mb] = Mma<CT>::mfma(lds_read16(sQ + (key0 + mb * MB_STEP) * PA + (32 * c + 8 * g) * 2), kf[c], s[mb]);
+          dp[mb] = Mma<CT>::mfma(lds_read16(sDO + (key0 + mb * MB_STEP) * PB + (32 * c + 8 * g) * 2), vf[c], dp[mb]);
         }
       }
       float pr[8], ds[8];
@@ -262,8 +263,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
       const int kt0 = 4 * wave + 4 * cg0;
 #pragma unroll
       for (int d = 0; d < DB; d++) {
-        dv_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sDO, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), pb, dv_acc[d]);
-        dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dk_acc[d]);
+        dv_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sDO, PB, HCW, kt0, 16 * d, n, g, MB_STEP), pb, dv_acc[d]);
+        dk_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sQ, PA, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dk_acc[d]);
       }
     }
   };
@@ -271,13 +272,13 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   // forward kernel)
   for (int ch = L.ch_first; ch < L.ch_last; ch++) {
     swa1_issue_scalar2<HCW, CR>(r_lse, r_del, lseb, delb, a.ls[2], G, CR * ch + CR, tid);
-    swa1_issue<NI, BAL, TAIL>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
-    swa1_issue<NI, BAL, TAIL>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
+    swa1_issue<NI, BAL, TAIL, 0>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
+    swa1_issue<NI, BAL, TAIL, 1>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
     if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE, TAIL>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
-    swa1_commit<CT, NI, BAL, 0, TAIL>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
+    swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
     swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
     __syncthreads();
@@ -302,10 +303,11 @@ template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr int PITCH = D * 2 + SWA1_PAD;
+  constexpr bool WIDE = ROPE == 0;
+  constexpr int PA = swa1_pitch(D, NCGMAX, 0, WIDE), PB = swa1_pitch(D, NCGMAX, 1, WIDE);  // K rows, V rows
   constexpr int KC = D / 32, DB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
-  constexpr int REGION = CR * HCW * PITCH;
+  constexpr int REGION = CR * HCW * PA;
   constexpr int NKB = CR == 8 ? NCGMAX : NCGMAX / 2;
   constexpr int MB_STEP = CR == 8 ? 4 * HCW : 4;
 
@@ -336,15 +338,15 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
   constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR, BAL, TAIL>(sp, G, PITCH, tid, a.rope_pbit);
+  swa1_plan_init<D, HCW, CR, BAL, TAIL, WIDE, PA, PB>(sp, G, tid, a.rope_pbit);
   const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   StageRegs<NI> srk, srv;
   swa1_regs_zero(srk);
   TabRegs<NI> tr_srk;
   swa1_regs_zero(srv);
-  swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
-  swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
+  swa1_issue<NI, BAL, TAIL, 0>(srk, sp, on_k, kb_, sn2k, G, CR * L.ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
+  swa1_issue<NI, BAL, TAIL, 1>(srv, sp, on_v, vb_, sn2v, G, CR * L.ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
 
   // own output gradients, outputs and queries straight into B-operand fragments.  Everything that
   // needs no rotation is requested first; the rotated query fragments wait for their table rows last.
@@ -385,8 +387,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   const float scale = a.scale_log2;
 
   if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
-  swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
-  swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
+  swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+  swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   __syncthreads();
   pin_loaded(qf);
   pin_loaded(dof);
@@ -414,8 +416,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
         dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KC; c++) {
-          s[mb] = Mma<CT>::mfma(lds_read16(sK + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), qf[c], s[mb]);
-          dp[mb] = Mma<CT>::mfma(lds_read16(sV + (key0 + mb * MB_STEP) * PITCH + (32 * c + 8 * g) * 2), dof[c], dp[mb]);
+          s[mb] = Mma<CT>::mfma(lds_read16(sK + (key0 + mb * MB_STEP) * PA + (32 * c + 8 * g) * 2), qf[c], s[mb]);
+          dp[mb] = Mma<CT>::mfma(lds_read16(sV + (key0 + mb * MB_STEP) * PB + (32 * c + 8 * g) * 2), dof[c], dp[mb]);
         }
       }
       float ds[8];
@@ -433,17 +435,17 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
       const int kt0 = 4 * wave + 4 * cg0;
 #pragma unroll
       for (int d = 0; d < DB; d++)
-        dq_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sK, PITCH, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dq_acc[d]);
+        dq_acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sK, PA, HCW, kt0, 16 * d, n, g, MB_STEP), dsb, dq_acc[d]);
     }
   };
   for (int ch = L.ch_first; ch < L.ch_last; ch++) {
-    swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
-    swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
+    swa1_issue<NI, BAL, TAIL, 0>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
+    swa1_issue<NI, BAL, TAIL, 1>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
     if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
-    swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
+    swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     __syncthreads();
   }
   consume(L.ch_last);

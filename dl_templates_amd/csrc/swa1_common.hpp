@@ -11,9 +11,17 @@
 #pragma once
 #include "attn_common.hpp"
 
-#ifndef SWA1_PAD
-#define SWA1_PAD 16  // bytes of padding after each token row of an LDS chunk
-#endif
+// LDS row pitch of a staged chunk.  16-byte LDS accesses of a wave are served 16 lanes at a time,
+// lanes {0-7, 16-23}, {8-15, 24-31}, ... together (measured with a probe); with 64 banks of 4 bytes
+// a pitch of 16 k bytes keeps the reads of such a group on distinct banks iff k = 2 (mod 4):
+// 32 bytes of padding for head dims 64 and 128, where 16 bytes make every read a 2-way conflict.
+// `wide`: the layout with 32 bytes of padding and the bank-spreading write map (kernels without
+// rotation).  At D = 128 the wide window class cannot afford it for both regions within two
+// workgroups per CU: its second region keeps 16 bytes (and the dK/dV kernel, which also stages
+// lse2 / delta, keeps 16 bytes for both).
+constexpr int swa1_pitch(int d, int ncgmax, int region, bool wide, bool kv = false) {
+  return d * 2 + ((!wide || (d == 128 && ncgmax > 4 && (region == 1 || kv))) ? 16 : 32);
+}
 
 struct Swa1Plan {
   int32_t HRP;      // halo rows, padded to a multiple of 8 (chunks hold 8 halo rows)
@@ -58,30 +66,40 @@ template <int NI>
 struct StagePlan {
   int hr[NI];    // halo row inside the chunk (0..7)
   int cc[NI];    // grid column, clamped
-  int loff[NI];  // byte offset of the token row inside the LDS chunk, -1: no such item
+  int lkey[NI];  // token row inside the LDS chunk, -1: no such item
   int coff[4];   // byte offsets of the thread's four 16-byte chunks inside a token row
   int t_hr, t_cc;  // tail chunk: halo row and clamped grid column of its token
-  int t_loff;      // tail chunk: byte offset inside the LDS chunk, -1: this thread has none
+  int t_key;       // tail chunk: token row inside the LDS chunk, -1: this thread has none
   int t_off;       // tail chunk: byte offset inside the token row
+  int jx16[2];   // wide layout, per region: register j holds chunk j ^ (jx16 / 16) of the piece (0: in order)
   int bal;       // balanced mapping: chunks 0 and 1 are a rotary pair
   int axis;      // balanced: 0 row angle, 1 column angle
   int tab_off;   // balanced: float offset of the pair's (cos, sin) values inside a table row
 };
 
-template <int D, int HCW, int CR, bool BAL, bool TAIL = false>
-DLT_DEV void swa1_plan_init(StagePlan<swa1_items_t(D, HCW, CR, TAIL)>& sp, const Swa1Geom& G, int pitch, int tid, int bal_r8) {
+// WIDE: thread -> token map with lane bits 3 and 4 swapped, and for a region of pitch 2 D + 32 the
+// chunk order of a piece flipped on every other thread (D = 64) or token pair (D = 128): the 16 writes
+// of a lane group then land on 16 distinct bank quads (PA / PB: the pitches of the two regions).
+template <int D, int HCW, int CR, bool BAL, bool TAIL = false, bool WIDE = false, int PA = 0, int PB = 0>
+DLT_DEV void swa1_plan_init(StagePlan<swa1_items_t(D, HCW, CR, TAIL)>& sp, const Swa1Geom& G, int tid_, int bal_r8) {
   constexpr int QUADS = D / 32;
+  const int tid = WIDE ? ((tid_ & ~0x18) | ((tid_ & 8) << 1) | ((tid_ & 16) >> 1)) : tid_;
   const int qd = tid % QUADS, key0 = tid / QUADS;
-  sp.t_hr = 0; sp.t_cc = dlt_imax(0, dlt_imin(G.c0 - G.WC, G.TC - 1)); sp.t_loff = -1; sp.t_off = 0;
+  {
+    const int jx = WIDE ? 16 * (QUADS == 2 ? (qd & 1) : ((key0 >> 1) & 1)) : 0;
+    sp.jx16[0] = PA == 2 * D + 32 ? jx : 0;
+    sp.jx16[1] = PB == 2 * D + 32 ? jx : 0;
+  }
+  sp.t_hr = 0; sp.t_cc = dlt_imax(0, dlt_imin(G.c0 - G.WC, G.TC - 1)); sp.t_key = -1; sp.t_off = 0;
   if (TAIL) {
     constexpr int FULL = (CR * HCW * QUADS) / 256, REM = (CR * HCW * QUADS) % 256;
-    if (tid < REM * 4) {
-      const int ti = FULL * 256 + (tid >> 2);
+    if (tid_ < REM * 4) {
+      const int ti = FULL * 256 + (tid_ >> 2);
       const int key = ti / QUADS;
-      sp.t_off = 64 * (ti % QUADS) + 16 * (tid & 3);
+      sp.t_off = 64 * (ti % QUADS) + 16 * (tid_ & 3);
       sp.t_hr = key / HCW;
       sp.t_cc = dlt_imax(0, dlt_imin(G.c0 - G.WC + (key - sp.t_hr * HCW), G.TC - 1));
-      sp.t_loff = key * pitch + sp.t_off;
+      sp.t_key = key;
     }
   }
   sp.bal = BAL;
@@ -108,7 +126,7 @@ DLT_DEV void swa1_plan_init(StagePlan<swa1_items_t(D, HCW, CR, TAIL)>& sp, const
     const int hr = k / HCW, hc = k - hr * HCW;
     sp.hr[it] = hr;
     sp.cc[it] = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));
-    sp.loff[it] = live ? k * pitch : -1;
+    sp.lkey[it] = live ? k : -1;
   }
 }
 
@@ -135,7 +153,7 @@ DLT_DEV void swa1_regs_zero(StageRegs<NI>& sr) {
 // Issue the global loads of halo rows [cr0, cr0 + 8) into registers.  `sn2` is the token stride
 // in BYTES; offsets are 32-bit (the host checks that a [N, D] slab stays below 2 GiB).  `on`:
 // the thread's 64-byte piece lies below the actual head dim (pieces above it stay zero).
-template <int NI, bool BAL, bool TAIL = false>
+template <int NI, bool BAL, bool TAIL = false, int REG = 0>
 DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, const void* base, int sn2, const Swa1Geom& G,
                         int cr0, const int32_t* rope_idx, bool tail_on = false) {
   const int rbase = G.r0 - G.WR + cr0;
@@ -152,7 +170,7 @@ DLT_DEV void swa1_issue(StageRegs<NI>& sr, const StagePlan<NI>& sp, bool on, con
     if (on) {
       const char* p = reinterpret_cast<const char*>(base) + (uint32_t)(tok * sn2);
 #pragma unroll
-      for (int j = 0; j < 4; j++) sr.v[it][j] = *reinterpret_cast<const u32x4*>(p + (BAL ? sp.coff[j] : sp.coff[0] + 16 * j));
+      for (int j = 0; j < 4; j++) sr.v[it][j] = *reinterpret_cast<const u32x4*>(p + (BAL ? sp.coff[j] : sp.coff[0] + ((16 * j) ^ sp.jx16[REG])));
     }
     if (rope_idx != nullptr) sr.id[it] = rope_idx[tok];
   }
@@ -185,14 +203,14 @@ DLT_DEV void swa1_tab_issue(TabRegs<NI>& tr, const StageRegs<NI>& sr, const Stag
 // Rotate (K / Q side only) and write the staged registers into an LDS chunk.
 // ROT: 0 no rotation, 1 rotation with the plain chunk mapping, 2 rotation of the balanced
 // mapping's pair (chunks 0 and 1).  pbit: chunk distance between rotary partners (1 or 2).
-template <typename CT, int NI, bool BAL, int ROT, bool TAIL = false>
+template <typename CT, int NI, bool BAL, int ROT, bool TAIL, int REG, int PITCH>
 DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, int pbit, const RopeDev& rope, bool use_rope,
                          const TabRegs<NI>* tr = nullptr, bool tail_on = false) {
   static_assert(ROT != 2 || BAL, "pair rotation needs the balanced mapping");
   static_assert(!TAIL || ROT == 0, "tail staging splits rotary pairs");
   if (TAIL) {
     pin_loaded(sr.tv);
-    if (sp.t_loff >= 0) lds_write16(s + sp.t_loff, tail_on ? sr.tv : u32x4{0u, 0u, 0u, 0u});
+    if (sp.t_key >= 0) lds_write16(s + sp.t_key * PITCH + sp.t_off, tail_on ? sr.tv : u32x4{0u, 0u, 0u, 0u});
   }
   // wait for the staged loads HERE, on every path: a wait placed inside the per-thread `if` below
   // would be skipped when no lane has an item, and the compiler would then treat the loads as
@@ -209,7 +227,7 @@ DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, in
   }
 #pragma unroll
   for (int it = 0; it < NI; it++) {
-    if (sp.loff[it] < 0) continue;
+    if (sp.lkey[it] < 0) continue;
     if (ROT == 2 && use_rope) {
       if (tr->rot[it]) {
         float x0[8], x1[8];
@@ -261,9 +279,9 @@ DLT_DEV void swa1_commit(StageRegs<NI>& sr, const StagePlan<NI>& sp, char* s, in
         }
       }
     }
-    char* row = s + sp.loff[it];
+    char* row = s + sp.lkey[it] * PITCH;
 #pragma unroll
-    for (int j = 0; j < 4; j++) lds_write16(row + (BAL ? sp.coff[j] : sp.coff[0] + 16 * j), sr.v[it][j]);
+    for (int j = 0; j < 4; j++) lds_write16(row + (BAL ? sp.coff[j] : sp.coff[0] + ((16 * j) ^ sp.jx16[REG])), sr.v[it][j]);
   }
 }
 

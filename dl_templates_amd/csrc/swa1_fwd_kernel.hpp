@@ -37,10 +37,11 @@ template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 2) : (CR == 4 ? 2 : 1))) void swa1_fwd_kernel(const Swa1FwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr int PITCH = D * 2 + SWA1_PAD;
+  constexpr bool WIDE = ROPE == 0;  // padded-by-32 layout: kernels without rotation
+  constexpr int PA = swa1_pitch(D, NCGMAX, 0, WIDE), PB = swa1_pitch(D, NCGMAX, 1, WIDE);  // K rows, V rows
   constexpr int KC = D / 32, VB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
-  constexpr int REGION = CR * HCW * PITCH;
+  constexpr int REGION = CR * HCW * PA;
   constexpr int NKB = CR == 8 ? NCGMAX : NCGMAX / 2;      // 32-token blocks per wave and chunk
   constexpr int MB_STEP = CR == 8 ? 4 * HCW : 4;          // token distance between the halves of a block
   static_assert(CR == 8 || NCGMAX % 2 == 0, "4-row chunks pair column groups");
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
   constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
-  swa1_plan_init<D, HCW, CR, BAL, TAIL>(sp, G, PITCH, tid, a.rope_pbit);
+  swa1_plan_init<D, HCW, CR, BAL, TAIL, WIDE, PA, PB>(sp, G, tid, a.rope_pbit);
   const bool on_k = (sp.coff[0] >> 1) < a.p.dk, on_v = (sp.coff[0] >> 1) < a.p.dv;
   const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
   const int64_t tq_own = own_token(16 * wave + n);
@@ -96,8 +97,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   swa1_regs_zero(srk);
   TabRegs<NI> tr_srk;
   swa1_regs_zero(srv);
-  swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
-  swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
+  swa1_issue<NI, BAL, TAIL, 0>(srk, sp, on_k, kb_, sn2k, G, CR * ch_first, rope_idx, (sp.t_off >> 1) < a.p.dk);
+  swa1_issue<NI, BAL, TAIL, 1>(srv, sp, on_v, vb_, sn2v, G, CR * ch_first, nullptr, (sp.t_off >> 1) < a.p.dv);
 
   // own queries straight into B-operand fragments (rotated on the way when fused)
   u32x4 qf[KC];
@@ -133,8 +134,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
 
   if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, a.p.rope);
-  swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
-  swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, a.p.rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
+  swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+  swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srv, sp, sV, 1, a.p.rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   __syncthreads();
   pin_loaded(qf);
 
@@ -162,8 +163,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int c = 0; c < KC; c++) {
-          const u32x4 k0 = lds_read16(sK + key0 * PITCH + (32 * c + 8 * g) * 2);
-          const u32x4 k1 = lds_read16(sK + (key0 + MB_STEP) * PITCH + (32 * c + 8 * g) * 2);
+          const u32x4 k0 = lds_read16(sK + key0 * PA + (32 * c + 8 * g) * 2);
+          const u32x4 k1 = lds_read16(sK + (key0 + MB_STEP) * PA + (32 * c + 8 * g) * 2);
           s0 = Mma<CT>::mfma(k0, qf[c], s0);
           s1 = Mma<CT>::mfma(k1, qf[c], s1);
         }
@@ -217,7 +218,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
         const int key0 = 4 * wave + 4 * (CR == 8 ? kb : 2 * kb);
 #pragma unroll
         for (int d = 0; d < VB; d++)
-          acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PITCH, HCW, key0, 16 * d, n, g, MB_STEP), pb[kb], acc[d]);
+          acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PB, HCW, key0, 16 * d, n, g, MB_STEP), pb[kb], acc[d]);
         if (ONES) acc_l = Mma<CT>::mfma(ones, pb[kb], acc_l);
       }
     }
@@ -227,13 +228,13 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   // pending across the back edge and guards every later load with a full vmcnt(0) wait.
   for (int ch = ch_first; ch < ch_last; ch++) {
     // next chunk: HBM -> registers while this one is consumed
-    swa1_issue<NI, BAL, TAIL>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
-    swa1_issue<NI, BAL, TAIL>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
+    swa1_issue<NI, BAL, TAIL, 0>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
+    swa1_issue<NI, BAL, TAIL, 1>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
     if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, a.p.rope);  // table rows of the next chunk's tokens, ahead of the barrier
     __syncthreads();  // every wave is done with this chunk
-    swa1_commit<CT, NI, BAL, ROPE, TAIL>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
-    swa1_commit<CT, NI, BAL, 0, TAIL>(srv, sp, sV, 1, a.p.rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
+    swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, a.p.rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srv, sp, sV, 1, a.p.rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     __syncthreads();
   }
   consume(ch_last);
