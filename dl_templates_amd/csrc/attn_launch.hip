@@ -244,7 +244,7 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
   a.tile = p.g.mode == DLT_GEOM_SWA;
   a.g = p.g;
   a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, 2);
-  const int chunk = FLASH_CK * (dc.DK * 2 + 16 + dc.DV * 2 + 16), tile = own * (dc.DV * 2 + 16);
+  const int chunk = FLASH_CK * (dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD), tile = own * (dc.DV * 2 + 16);
   a.lds_bytes = chunk > tile ? chunk : tile;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   const int64_t grid = (int64_t)p.B * p.H * p.g.TR * a.nblk;
@@ -294,7 +294,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, 2);
   a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, 2);
   a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, 2);
-  const int chunk = FLASH_CK * (dc.DK * 2 + 16 + dc.DV * 2 + 16);
+  const int chunk = FLASH_CK * (dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD);
   const int tile_q = own * (dc.DK * 2 + 16);
   const int tile_k = own_kv * (dc.DK * 2 + 16), tile_v = own_kv * (dc.DV * 2 + 16);
   a.lds_q = chunk > tile_q ? chunk : tile_q;

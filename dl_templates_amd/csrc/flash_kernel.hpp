@@ -19,6 +19,23 @@
 #pragma once
 #include "swa1_common.hpp"
 
+// Streamed chunks in LDS: rows of 2 D + 32 bytes.  16-byte LDS accesses of a wave are served 16
+// lanes at a time, lanes {0-7, 16-23}, {8-15, 24-31}, ... together; with 64 banks a pitch of 16 k
+// bytes keeps the operand reads (16 rows x 16 bytes, and the transposing 8-byte reads) of such a group
+// on distinct banks iff k = 2 (mod 4).  The staging writes (thread -> 16-byte vector t % CH of token
+// t / CH) then need the tokens of a lane group a quarter or half of the bank space apart: one pair
+// of thread-index bits is swapped per row length.
+#ifndef FLASH_PAD
+#define FLASH_PAD 32
+#endif
+template <int CH>
+DLT_DEV int flash_stage_tid(int tid) {
+  constexpr int A = CH == 4 ? 2 : 4, B = CH == 4 ? 3 : (CH == 8 ? 5 : 6);  // bits to swap
+  if (FLASH_PAD != 32) return tid;
+  const int x = ((tid >> A) ^ (tid >> B)) & 1;
+  return tid ^ ((x << A) | (x << B));
+}
+
 #ifndef FLASH_NP_DEF
 #define FLASH_NP_DEF 2
 #endif
@@ -114,7 +131,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   typedef typename TileOf<TIO>::type TL;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
-  constexpr int PK = DK * 2 + 16, PV = DV * 2 + 16, PO = DV * (int)sizeof(TL) + 16;
+  constexpr int PK = DK * 2 + FLASH_PAD, PV = DV * 2 + FLASH_PAD, PO = DV * (int)sizeof(TL) + 16;
   constexpr int KC = DK / 32, VB = DV / 16, NKB = CK / 32;
   constexpr int OWN = 64 * NP;
   constexpr int KCH = DK / 8, VCH = DV / 8;                    // 16-byte vectors per token
@@ -146,8 +163,9 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   else W.init_seq(0, CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk);   // causal: keys up to the last own query
 
   // ---- staging plan (chunk invariant): vector `it` of this thread = chunk ck*/vc* of key kkey/vkey + it * step
-  const int kc_ = tid % KCH, kkey0 = tid / KCH;
-  const int vc_ = tid % VCH, vkey0 = tid / VCH;
+  const int tk = flash_stage_tid<KCH>(tid), tv = flash_stage_tid<VCH>(tid);
+  const int kc_ = tk % KCH, kkey0 = tk / KCH;
+  const int vc_ = tv % VCH, vkey0 = tv / VCH;
   const bool on_k = 8 * kc_ < a.dk, on_v = 8 * vc_ < a.dv;
   u32x4 rk[NKI], rv[NVI];
 #pragma unroll
@@ -388,8 +406,9 @@ struct PairStage {
   bool on_a, on_b;
 
   DLT_DEV void init(int tid, int dact_a, int dact_b) {
-    ac = tid % ACH; akey0 = tid / ACH;
-    bc = tid % BCH; bkey0 = tid / BCH;
+    const int ta = flash_stage_tid<ACH>(tid), tb = flash_stage_tid<BCH>(tid);
+    ac = ta % ACH; akey0 = ta / ACH;
+    bc = tb % BCH; bkey0 = tb / BCH;
     on_a = 8 * ac < dact_a; on_b = 8 * bc < dact_b;
 #pragma unroll
     for (int it = 0; it < NAI; it++) ra[it] = u32x4{0u, 0u, 0u, 0u};
@@ -446,7 +465,7 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
-  constexpr int PK = DK * 2 + 16, PV = DV * 2 + 16;
+  constexpr int PK = DK * 2 + FLASH_PAD, PV = DV * 2 + FLASH_PAD;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, NKB = CK / 32;
   constexpr int OWN = 64 * NP;
 
@@ -608,7 +627,7 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
-  constexpr int PQ = DK * 2 + 16, PD = DV * 2 + 16;
+  constexpr int PQ = DK * 2 + FLASH_PAD, PD = DV * 2 + FLASH_PAD;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16, NQB = CK / 32;
   constexpr int OWN = 64 * NP;
 
