@@ -328,6 +328,37 @@ def recorded_traffic(kernel):
         return None
 
 
+def image_layout_demo(steps):
+    from dl_templates_amd import tiled_swa
+    B, H, th, tw, bh, bw, d = 4, 8, 64, 64, 4, 4, 32   # the demo's tiles and head dim on a 256 x 256 image
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(3)
+    img = [torch.randn((B, th * bh, tw * bw, H, d), generator=g).to(torch.float16).to(dev) for _ in range(4)]
+    qi, ki, vi, doi = img
+
+    def to_tokens(x):   # [B, IH, IW, H, D] -> [B, H, N, D], a real copy
+        return x.reshape(B, th, bh, tw, bw, H, d).permute(0, 5, 1, 3, 2, 4, 6).reshape(B, H, th * tw * bh * bw, d)
+
+    def to_image(x):
+        return x.reshape(B, H, th, tw, bh, bw, d).permute(0, 2, 4, 3, 5, 1, 6).reshape(B, th * bh, tw * bw, H, d)
+
+    def direct():
+        q, k, v = (t.detach().requires_grad_(True) for t in (qi, ki, vi))
+        tiled_swa.TiledSwaImage.apply(q, k, v, bh, bw, 1, 1, 0.25).backward(doi)
+        return q.grad, k.grad, v.grad
+
+    def converted():
+        q, k, v = (to_tokens(t).requires_grad_(True) for t in (qi, ki, vi))
+        o = tiled_swa.TiledSwa.apply(q, k, v, bh * bw, th, tw, 1, 1, 0.25)
+        o.backward(to_tokens(doi))
+        return to_image(o), to_image(q.grad), to_image(k.grad), to_image(v.grad)
+
+    ms_direct, _ = Timer.run(direct, steps, 3)
+    ms_conv, _ = Timer.run(converted, steps, 3)
+    return {"ms_image_entry_points": ms_direct, "ms_convert_run_convert_back": ms_conv,
+            "workload": "B=4 H=8, 256x256 pixel image, 4x4-pixel tiles, d=32, 3x3 tile window, fp16, fwd+bwd"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -394,6 +425,10 @@ def main():
         extra["ref_demo_b16"] = {"ms_per_step": msd, "eff_tflops": fd / (msd * 1e-3) / 1e12,
                                  "workload": "B=4 H=8 16x16 tiles of 16 tokens, d=32, 3x3 window, fp16, fwd+bwd (src/tiled_swa.py:736-750)"}
         del wd
+        # the demo's tiles with q, k, v, dO kept as images [B, IH, IW, heads, D] (4 x 4 pixel tiles):
+        # the image entry points against converting to the token layout and back around the operator
+        # (src/tiled_swa.py:753-755), both through the autograd functions of the package
+        extra["ref_demo_image_layout"] = image_layout_demo(max(K // 5, 3))
         # larger tiles: B=2, H=8, 16x16 tiles of 64 tokens (N = 16384), d=64, 3x3 tile window, bf16
         wt = SwaWorkload("tiles_b64", 2, 8, 16, 16, 1, 64, fused_rope=False, nsets=1, b_size=64)
         mst, _ = Timer.run(wt.step, max(K // 5, 3), 2)

@@ -26,6 +26,7 @@ EXPORTS = (
     "dlt_last_error", "dlt_version", "dlt_rope2d", "dlt_rope2d_pair", "dlt_rope_pe_mask",
     "dlt_swa_fwd", "dlt_swa_bwd", "dlt_swa_neighbors", "dlt_flash_fwd", "dlt_flash_bwd",
     "dlt_timing_enable", "dlt_timing_collect", "dlt_debug_copy",
+    "dlt_swa_fwd_image", "dlt_swa_bwd_image", "dlt_swa_image_offsets",
 )
 KERNEL_NAMES = ("rope2d", "attn_fwd", "attn_delta", "attn_bwd_kv", "attn_bwd_q")
 
@@ -56,6 +57,10 @@ class SwaShape(Structure):
         ("row_size", c_int32), ("col_size", c_int32), ("dk", c_int32), ("dv", c_int32),
         ("sm_scale", c_float), ("dtype", c_int32),
     ]
+
+
+class SwaTile(Structure):
+    _fields_ = [("bh", c_int32), ("bw", c_int32)]
 
 
 class FlashShape(Structure):
@@ -101,6 +106,12 @@ def _declare(lib) -> None:
     lib.dlt_swa_fwd.argtypes = fwd + [POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
     lib.dlt_swa_bwd.restype = c_int
     lib.dlt_swa_bwd.argtypes = bwd + [POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
+    lib.dlt_swa_fwd_image.restype = c_int
+    lib.dlt_swa_fwd_image.argtypes = fwd + [POINTER(SwaShape), POINTER(SwaTile), POINTER(RopeDesc), c_void_p]
+    lib.dlt_swa_bwd_image.restype = c_int
+    lib.dlt_swa_bwd_image.argtypes = bwd + [POINTER(SwaShape), POINTER(SwaTile), POINTER(RopeDesc), c_void_p]
+    lib.dlt_swa_image_offsets.restype = c_int
+    lib.dlt_swa_image_offsets.argtypes = [c_int32, c_int32, c_int32, c_int32, c_int64, c_int64, c_void_p, c_void_p]
     lib.dlt_flash_fwd.restype = c_int
     lib.dlt_flash_fwd.argtypes = fwd + [POINTER(FlashShape), c_void_p]
     lib.dlt_flash_bwd.restype = c_int

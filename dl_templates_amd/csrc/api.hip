@@ -92,6 +92,15 @@ __global__ void swa_neighbors_kernel(DltGeom g, uint8_t* mask) {
   mask[id] = (uint8_t)((kr >= rlo && kr <= rhi && kx >= xlo && kx < xhi) ? 1 : 0);
 }
 
+__global__ void swa_image_offsets_kernel(DltTokMap tm, int64_t sy, int64_t sx, int64_t n_tokens, int64_t* out) {
+  // one thread per token: the same dlt_token_pixel the attention kernels address image tensors with
+  const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= n_tokens) return;
+  uint32_t y, x;
+  dlt_token_pixel(tm, (uint32_t)n, y, x);
+  out[n] = (int64_t)y * sy + (int64_t)x * sx;
+}
+
 bool is_dtype(int d) { return d == DLT_BF16 || d == DLT_FP16 || d == DLT_FP32; }
 
 int check_ptrs(const char* who, const void* const* ptrs, const int64_t* const* strides, int n) {
@@ -124,6 +133,7 @@ int swa_problem(const char* who, const dlt_swa_shape_t* s, const dlt_rope_t* rop
     if (rc != DLT_OK) return rc;
   }
   p.rope = dlt_make_rope_dev(rope, 0);
+  p.tm = dlt_tokmap_none();
   return DLT_OK;
 }
 
@@ -138,6 +148,7 @@ int flash_problem(const char* who, const dlt_flash_shape_t* s, AttnProblem& p) {
   p.g.XLq = s->Lq; p.g.XLk = s->Lk;
   p.B = s->B; p.H = s->H; p.dk = s->dk; p.dv = s->dv; p.sm_scale = s->sm_scale; p.dtype = s->dtype;
   p.rope = dlt_make_rope_dev(nullptr, 0);
+  p.tm = dlt_tokmap_none();
   return DLT_OK;
 }
 
@@ -170,6 +181,34 @@ int fill_bwd(const char* who, AttnTensors& t, const void* q, const int64_t* qs, 
   cp4(t.qs, qs); cp4(t.ks, ks); cp4(t.vs, vs); cp4(t.os, os); cp4(t.dos, dos);
   cp4(t.dqs, dqs); cp4(t.dks, dks); cp4(t.dvs, dvs); cp3(t.ls, ls);
   return DLT_OK;
+}
+
+// ---- image layout: [B, IH, IW, heads, D] strides -> internal [B, heads, pixel x, D, pixel y] -------
+int image_tile(const char* who, const dlt_swa_shape_t* s, const dlt_swa_tile_t* tile) {
+  DLT_REQUIRE(s != nullptr && tile != nullptr, "%s: shape / tile is NULL", who);
+  DLT_REQUIRE(tile->bh > 0 && tile->bw > 0, "%s: tile of %d x %d pixels", who, tile->bh, tile->bw);
+  DLT_REQUIRE((int64_t)tile->bh * tile->bw == s->b_size, "%s: b_size=%d is not the tile of %d x %d pixels", who,
+              s->b_size, tile->bh, tile->bw);
+  return DLT_OK;
+}
+
+int image_strides(const char* who, int which, const int64_t* in, int64_t* out) {
+  DLT_REQUIRE(in != nullptr, "%s: stride argument %d is NULL", who, which);
+  for (int i = 0; i < 5; i++) DLT_REQUIRE(in[i] >= 0, "%s: image tensor %d has a negative stride", who, which);
+  out[0] = in[0]; out[1] = in[3]; out[2] = in[2]; out[3] = in[4]; out[4] = in[1];
+  return DLT_OK;
+}
+
+// Every tensor of a call whose pixel rows are TC * bw pixel columns apart with single-pixel tiles is
+// a plain [B, H, N, D] view: the token map is dropped and every kernel family stays available.
+void image_finish(AttnProblem& p, const dlt_swa_tile_t* tile, int64_t* const* st, int n) {
+  bool linear = tile->bh == 1 && tile->bw == 1;
+  for (int i = 0; i < n && linear; i++) linear = st[i][4] == (int64_t)p.g.TC * st[i][2];
+  if (linear) {
+    for (int i = 0; i < n; i++) st[i][4] = 0;
+    return;
+  }
+  p.tm = dlt_tokmap_image((uint32_t)tile->bh, (uint32_t)tile->bw, (uint32_t)p.g.TC);
 }
 
 }  // namespace
@@ -268,5 +307,78 @@ extern "C" int dlt_flash_bwd(const void* q, const int64_t q_strides[4], const vo
   rc = fill_bwd("flash_bwd", t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, d_o, do_strides, lse2, delta,
                 lse_strides, dq, dq_strides, dk, dk_strides, dv, dv_strides);
   if (rc != DLT_OK) return rc;
+  return dlt_attn_backward(p, t, (hipStream_t)stream);
+}
+
+// ---- image-layout entry points ------------------------------------------------------------------
+extern "C" int dlt_swa_image_offsets(int32_t t_height, int32_t t_width, int32_t bh, int32_t bw, int64_t stride_y,
+                                     int64_t stride_x, int64_t* offsets, void* stream) {
+  DLT_REQUIRE(t_height > 0 && t_width > 0 && bh > 0 && bw > 0, "swa_image_offsets: bad grid / tile");
+  DLT_REQUIRE(offsets != nullptr, "swa_image_offsets: offsets is NULL");
+  const int64_t n = (int64_t)t_height * t_width * bh * bw;
+  DLT_REQUIRE(n <= 0x3fffffff, "swa_image_offsets: too many tokens");
+  const DltTokMap tm = dlt_tokmap_image((uint32_t)bh, (uint32_t)bw, (uint32_t)t_width);
+  hipLaunchKernelGGL(swa_image_offsets_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, tm,
+                     stride_y, stride_x, n, offsets);
+  DLT_CHECK_LAUNCH("swa_image_offsets launch");
+  return DLT_OK;
+}
+
+extern "C" int dlt_swa_fwd_image(const void* q, const int64_t q_strides[5], const void* k, const int64_t k_strides[5],
+                                 const void* v, const int64_t v_strides[5], void* o, const int64_t o_strides[5],
+                                 float* lse2, const int64_t lse_strides[3], const dlt_swa_shape_t* shape,
+                                 const dlt_swa_tile_t* tile, const dlt_rope_t* rope, void* stream) {
+  const char* who = "swa_fwd_image";
+  int rc = image_tile(who, shape, tile);
+  if (rc != DLT_OK) return rc;
+  AttnProblem p;
+  rc = swa_problem(who, shape, rope, p);
+  if (rc != DLT_OK) return rc;
+  const void* const ptrs[] = {q, k, v, o, lse2};
+  const int64_t* const st[] = {q_strides, k_strides, v_strides, o_strides, lse_strides};
+  rc = check_ptrs(who, ptrs, st, 5);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  memset(&t, 0, sizeof(t));
+  t.q = q; t.k = k; t.v = v; t.out_o = o; t.lse = lse2;
+  cp3(t.ls, lse_strides);
+  int64_t* const mine[] = {t.qs, t.ks, t.vs, t.os};
+  for (int i = 0; i < 4; i++) {
+    rc = image_strides(who, i, st[i], mine[i]);
+    if (rc != DLT_OK) return rc;
+  }
+  image_finish(p, tile, mine, 4);
+  return dlt_attn_forward(p, t, (hipStream_t)stream);
+}
+
+extern "C" int dlt_swa_bwd_image(const void* q, const int64_t q_strides[5], const void* k, const int64_t k_strides[5],
+                                 const void* v, const int64_t v_strides[5], const void* o, const int64_t o_strides[5],
+                                 const void* d_o, const int64_t do_strides[5],
+                                 const float* lse2, float* delta, const int64_t lse_strides[3],
+                                 void* dq, const int64_t dq_strides[5], void* dk, const int64_t dk_strides[5],
+                                 void* dv, const int64_t dv_strides[5], const dlt_swa_shape_t* shape,
+                                 const dlt_swa_tile_t* tile, const dlt_rope_t* rope, void* stream) {
+  const char* who = "swa_bwd_image";
+  int rc = image_tile(who, shape, tile);
+  if (rc != DLT_OK) return rc;
+  AttnProblem p;
+  rc = swa_problem(who, shape, rope, p);
+  if (rc != DLT_OK) return rc;
+  const void* const ptrs[] = {q, k, v, o, d_o, dq, dk, dv, lse2, delta};
+  const int64_t* const st[] = {q_strides, k_strides, v_strides, o_strides, do_strides, dq_strides, dk_strides, dv_strides,
+                               lse_strides, lse_strides};
+  rc = check_ptrs(who, ptrs, st, 10);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  memset(&t, 0, sizeof(t));
+  t.q = q; t.k = k; t.v = v; t.o = o; t.d_o = d_o; t.lse = const_cast<float*>(lse2); t.delta = delta;
+  t.dq = dq; t.dk = dk; t.dv = dv;
+  cp3(t.ls, lse_strides);
+  int64_t* const mine[] = {t.qs, t.ks, t.vs, t.os, t.dos, t.dqs, t.dks, t.dvs};
+  for (int i = 0; i < 8; i++) {
+    rc = image_strides(who, i, st[i], mine[i]);
+    if (rc != DLT_OK) return rc;
+  }
+  image_finish(p, tile, mine, 8);
   return dlt_attn_backward(p, t, (hipStream_t)stream);
 }

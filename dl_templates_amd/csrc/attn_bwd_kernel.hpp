@@ -23,7 +23,7 @@ struct BwdArgs {
   const float* lse;
   float* delta;
   void *dq, *dk, *dv;
-  int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int64_t qs[5], ks[5], vs[5], os[5], dos[5], dqs[5], dks[5], dvs[5], ls[3];
   int32_t q_vec, k_vec, v_vec, o_vec, do_vec, dq_vec, dk_vec, dv_vec;
   float scale_log2;
   int64_t n_tokens_q;  // tokens per (batch, head) on the query side
@@ -46,8 +46,8 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
     const int b = (int)(bh / a.p.H), h = (int)(bh - (int64_t)b * a.p.H);
     const int nvalid = dlt_imin(8, a.p.dv - 8 * c);
     if (nvalid > 0) {
-      const TIO* po = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1] + nn * a.os[2] + (int64_t)8 * c * a.os[3];
-      const TIO* pd = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1] + nn * a.dos[2] + (int64_t)8 * c * a.dos[3];
+      const TIO* po = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1] + tok_addr(a.os, a.p.tm)(nn) + (int64_t)8 * c * a.os[3];
+      const TIO* pd = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1] + tok_addr(a.dos, a.p.tm)(nn) + (int64_t)8 * c * a.dos[3];
       if (sizeof(TIO) == 4) {
 #pragma unroll
         for (int j = 0; j < 8; j++) if (j < nvalid) part += (float)po[j * a.os[3]] * (float)pd[j * a.dos[3]];
@@ -78,8 +78,8 @@ DLT_DEV void stage_scalars(float* s, const float* base, int64_t stride, int n, T
 }
 
 // accumulators (C layout, [dim][own token]) -> LDS tile [own token][dim] -> HBM rows
-template <typename TIO, int D, int NP, typename Ctx>
-DLT_DEV void write_grad_tile(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO* base, int64_t sn, int64_t sd, int dact,
+template <typename TIO, int D, int NP, typename Ctx, typename SN>
+DLT_DEV void write_grad_tile(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO* base, const SN& sn, int64_t sd, int dact,
                              bool vec, const Ctx& T, const RopeDev& rope, int wave, int n, int g, int tid) {
   typedef typename TileOf<TIO>::type TL;
   constexpr int PT = D * (int)sizeof(TL) + 16;
@@ -134,9 +134,9 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
 
   // ---- own keys / values -> B-operand fragments (head dim along k)
-  stage_tile<TIO, CT, DK>(sOwnK, PQ, kb_, a.ks[2], a.ks[3], a.p.dk, a.k_vec != 0, OWN,
+  stage_tile<TIO, CT, DK>(sOwnK, PQ, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, fwd_rope, tid);
-  stage_tile<TIO, CT, DV>(sOwnV, PV, vb_, a.vs[2], a.vs[3], a.p.dv, a.v_vec != 0, OWN,
+  stage_tile<TIO, CT, DV>(sOwnV, PV, vb_, tok_addr(a.vs, a.p.tm), a.vs[3], a.p.dv, a.v_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, no_rope, tid);
   __syncthreads();
   u32x4 kf[NP][KC], vf[NP][VC];
@@ -172,8 +172,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
       for (int ri = 0; ri < nr; ri++) {
         const int64_t row_tok0 = (int64_t)(kr0 + ri) * G.XLq + cx0;
         auto tok = [&](int xi) { return cx0 + xi < G.XLq ? row_tok0 + xi : (int64_t)-1; };
-        stage_tile<TIO, CT, DK>(sQ + ri * CX * PQ, PQ, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, stage_w, tok, fwd_rope, tid);
-        stage_tile<TIO, CT, DV>(sDO + ri * CX * PV, PV, dob, a.dos[2], a.dos[3], a.p.dv, a.do_vec != 0, stage_w, tok, no_rope, tid);
+        stage_tile<TIO, CT, DK>(sQ + ri * CX * PQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, stage_w, tok, fwd_rope, tid);
+        stage_tile<TIO, CT, DV>(sDO + ri * CX * PV, PV, dob, tok_addr(a.dos, a.p.tm), a.dos[3], a.p.dv, a.do_vec != 0, stage_w, tok, no_rope, tid);
         stage_scalars(sLse + ri * CX, lseb, a.ls[2], stage_w, tok, tid);
         stage_scalars(sDel + ri * CX, delb, a.ls[2], stage_w, tok, tid);
       }
@@ -240,8 +240,8 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
   __syncthreads();
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
-  write_grad_tile<TIO, DK, NP>(smem, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.dks[3], a.p.dk, a.dk_vec != 0, T, inv_rope, wave, n, g, tid);
-  write_grad_tile<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.p.dv, a.dv_vec != 0, T, no_rope, wave, n, g, tid);
+  write_grad_tile<TIO, DK, NP>(smem, dk_acc, a.p.sm_scale, dkb, tok_addr(a.dks, a.p.tm), a.dks[3], a.p.dk, a.dk_vec != 0, T, inv_rope, wave, n, g, tid);
+  write_grad_tile<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, tok_addr(a.dvs, a.p.tm), a.dvs[3], a.p.dv, a.dv_vec != 0, T, no_rope, wave, n, g, tid);
 }
 
 // =============================================================================================
@@ -277,9 +277,9 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
 
-  stage_tile<TIO, CT, DK>(sOwnQ, PQ, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, OWN,
+  stage_tile<TIO, CT, DK>(sOwnQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, fwd_rope, tid);
-  stage_tile<TIO, CT, DV>(sOwnDO, PV, dob, a.dos[2], a.dos[3], a.p.dv, a.do_vec != 0, OWN,
+  stage_tile<TIO, CT, DV>(sOwnDO, PV, dob, tok_addr(a.dos, a.p.tm), a.dos[3], a.p.dv, a.do_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, no_rope, tid);
   __syncthreads();
   u32x4 qf[NP][KC], dof[NP][VC];
@@ -317,8 +317,8 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
       for (int ri = 0; ri < nr; ri++) {
         const int64_t row_tok0 = (int64_t)(kr0 + ri) * G.XLk + cx0;
         auto tok = [&](int xi) { return cx0 + xi < G.XLk ? row_tok0 + xi : (int64_t)-1; };
-        stage_tile<TIO, CT, DK>(sK + ri * CX * PQ, PQ, kb_, a.ks[2], a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, fwd_rope, tid);
-        stage_tile<TIO, CT, DV>(sV + ri * CX * PV, PV, vb_, a.vs[2], a.vs[3], a.p.dv, a.v_vec != 0, stage_w, tok, no_rope, tid);
+        stage_tile<TIO, CT, DK>(sK + ri * CX * PQ, PQ, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, fwd_rope, tid);
+        stage_tile<TIO, CT, DV>(sV + ri * CX * PV, PV, vb_, tok_addr(a.vs, a.p.tm), a.vs[3], a.p.dv, a.v_vec != 0, stage_w, tok, no_rope, tid);
       }
       __syncthreads();
 
@@ -372,5 +372,5 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
 
   __syncthreads();
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
-  write_grad_tile<TIO, DK, NP>(smem, dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.dqs[3], a.p.dk, a.dq_vec != 0, T, inv_rope, wave, n, g, tid);
+  write_grad_tile<TIO, DK, NP>(smem, dq_acc, a.p.sm_scale, dqb, tok_addr(a.dqs, a.p.tm), a.dqs[3], a.p.dk, a.dq_vec != 0, T, inv_rope, wave, n, g, tid);
 }

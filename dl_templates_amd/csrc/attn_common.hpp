@@ -251,12 +251,28 @@ DLT_DEV void rope_apply8(const RopeDev& r, const RopeChunk& rc, int c, int32_t i
   }
 }
 
+// ---- token -> element offset inside one (batch, head) slab --------------------------------------
+// A plain stride (tokens n * sn apart) or, for image-layout tensors, the pixel map of DltTokMap.
+struct TokAddr {
+  int64_t sn, sy;
+  const DltTokMap* tm;
+  DLT_DEV int64_t operator()(int64_t t) const {
+    if (!tm->img) return t * sn;
+    uint32_t y, x;
+    dlt_token_pixel(*tm, (uint32_t)t, y, x);
+    return (int64_t)y * sy + (int64_t)x * sn;
+  }
+};
+DLT_DEV TokAddr tok_addr(const int64_t (&s)[5], const DltTokMap& tm) { return TokAddr{s[2], s[4], &tm}; }
+DLT_DEV int64_t tok_offset(int64_t sn, int64_t t) { return t * sn; }
+DLT_DEV int64_t tok_offset(const TokAddr& a, int64_t t) { return a(t); }
+
 // ---- HBM -> LDS staging of `nrows` token rows of D head dims -------------------------------
 // LDS tile: row-major, `pitch` bytes per row, compute-type elements.  tok(row) gives the token
 // index inside the [N, D] slab at `base` (or -1: the row is zero-filled).  Dims >= dact are
 // zero-filled.  With `rope.enabled` rows are rotated on the way in (q and k of the fused call).
-template <typename TIO, typename CT, int D, typename TokFn>
-DLT_DEV void stage_tile(char* s, int pitch, const TIO* base, int64_t sn, int64_t sd, int dact, bool vec, int nrows,
+template <typename TIO, typename CT, int D, typename TokFn, typename SN>
+DLT_DEV void stage_tile(char* s, int pitch, const TIO* base, const SN& sn, int64_t sd, int dact, bool vec, int nrows,
                         TokFn tok, const RopeDev& rope, int tid) {
   constexpr int CH = D / 8;
   constexpr int RSTEP = 256 / CH;
@@ -267,7 +283,7 @@ DLT_DEV void stage_tile(char* s, int pitch, const TIO* base, int64_t sn, int64_t
     const int64_t t = tok(row);
     u32x4 val = {0u, 0u, 0u, 0u};
     if (t >= 0 && nvalid > 0) {
-      const TIO* p = base + t * sn;
+      const TIO* p = base + tok_offset(sn, t);
       val = Io<TIO, CT>::load8(p + (int64_t)8 * c * sd, vec, sd, nvalid);
       if (rc.mode != 0) {
         float self[8], partner8[8];
@@ -288,8 +304,8 @@ DLT_DEV void stage_tile(char* s, int pitch, const TIO* base, int64_t sn, int64_t
 
 // ---- LDS -> HBM store of an output tile ------------------------------------------------------
 // TL: element type of the LDS tile (the output type, or float for fp32 outputs).
-template <typename TO, typename TL, int D, typename TokFn>
-DLT_DEV void store_tile(const char* s, int pitch, TO* base, int64_t sn, int64_t sd, int dact, bool vec, int nrows,
+template <typename TO, typename TL, int D, typename TokFn, typename SN>
+DLT_DEV void store_tile(const char* s, int pitch, TO* base, const SN& sn, int64_t sd, int dact, bool vec, int nrows,
                         TokFn tok, const RopeDev& rope, int tid) {
   constexpr int CH = D / 8;
   constexpr int RSTEP = 256 / CH;
@@ -312,7 +328,7 @@ DLT_DEV void store_tile(const char* s, int pitch, TO* base, int64_t sn, int64_t 
       }
       rope_apply8(rope, rc, c, rope.idx[t], v, partner8, [&](int d) { return (float)lrow[d]; });
     }
-    Io<TO, CT>::store8(base + t * sn + (int64_t)8 * c * sd, v, vec, sd, nvalid);
+    Io<TO, CT>::store8(base + tok_offset(sn, t) + (int64_t)8 * c * sd, v, vec, sd, nvalid);
   }
 }
 

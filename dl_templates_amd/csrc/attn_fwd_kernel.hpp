@@ -19,7 +19,7 @@ struct FwdArgs {
   const void *q, *k, *v;
   void* o;
   float* lse;
-  int64_t qs[4], ks[4], vs[4], os[4], ls[3];
+  int64_t qs[5], ks[5], vs[5], os[5], ls[3];
   int32_t q_vec, k_vec, v_vec, o_vec;
   float scale_log2;
 };
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   no_rope.enabled = 0;
 
   // ---- own queries -> LDS -> B-operand fragments
-  stage_tile<TIO, CT, DK>(sQ, PQ, qb, a.qs[2], a.qs[3], a.p.dk, a.q_vec != 0, OWN,
+  stage_tile<TIO, CT, DK>(sQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, a.p.rope, tid);
   __syncthreads();
   u32x4 qf[NP][KC];
@@ -89,8 +89,8 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
       for (int ri = 0; ri < nr; ri++) {
         const int64_t row_tok0 = (int64_t)(kr0 + ri) * G.XLk + cx0;
         auto tok = [&](int xi) { return cx0 + xi < G.XLk ? row_tok0 + xi : (int64_t)-1; };
-        stage_tile<TIO, CT, DK>(sK + ri * CX * PK, PK, kb_, a.ks[2], a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, a.p.rope, tid);
-        stage_tile<TIO, CT, DV>(sV + ri * CX * PV, PV, vb_, a.vs[2], a.vs[3], a.p.dv, a.v_vec != 0, stage_w, tok, no_rope, tid);
+        stage_tile<TIO, CT, DK>(sK + ri * CX * PK, PK, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, a.p.rope, tid);
+        stage_tile<TIO, CT, DV>(sV + ri * CX * PV, PV, vb_, tok_addr(a.vs, a.p.tm), a.vs[3], a.p.dv, a.v_vec != 0, stage_w, tok, no_rope, tid);
       }
       __syncthreads();
 
@@ -170,6 +170,6 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
       a.lse[b * a.ls[0] + h * a.ls[1] + ((int64_t)r_own * G.XLq + xq) * a.ls[2]] = m_run[p] + fast_log2(lt);
   }
   __syncthreads();
-  store_tile<TIO, TL, DV>(sO, PO, ob, a.os[2], a.os[3], a.p.dv, a.o_vec != 0, OWN,
+  store_tile<TIO, TL, DV>(sO, PO, ob, tok_addr(a.os, a.p.tm), a.os[3], a.p.dv, a.o_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, no_rope, tid);
 }

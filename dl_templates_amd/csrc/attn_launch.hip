@@ -60,6 +60,17 @@ bool vec_ok(const void* ptr, const int64_t* st, int nd, int d, int elem) {
   return true;
 }
 
+// [B, H, N, D] tensor (entry 4 of the strides: pixel-row stride of an image-layout tensor, else 0)
+bool tvec_ok(const void* ptr, const int64_t* st, int d, int elem) {
+  return vec_ok(ptr, st, 4, d, elem) && (st[4] * elem) % 16 == 0;
+}
+
+// elements between the first and one past the last token of a (batch, head) slab
+int64_t slab_span(const AttnProblem& p, const int64_t* st, int64_t ntok) {
+  if (!p.tm.img) return ntok * st[2];
+  return ((int64_t)p.g.TR * p.tm.bh - 1) * st[4] + ((int64_t)p.g.TC * p.tm.bw - 1) * st[2] + 1;
+}
+
 // chunking plan for a kernel whose halo buffers need `per_tok` bytes per staged token and
 // whose own-tile region needs `own_bytes`
 int make_plan(const AttnProblem& p, int own, int own_bytes, int per_tok, int XL_own, int XL_halo, AttnPlan& plan) {
@@ -98,7 +109,7 @@ struct Swa1Class { int D, wclass, pbit, rope_mode; };
 // streamed tensors, both head dims in one padded class, a window of at most 21 columns and,
 // with rotation, rotary partners a power-of-two number of 8-dim chunks apart.
 bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streamed, Swa1Class& c) {
-  if (p.g.mode != DLT_GEOM_SWA || p.g.S != 1) return false;
+  if (p.g.mode != DLT_GEOM_SWA || p.g.S != 1 || p.tm.img) return false;
   if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
   if (p.dk % 32 != 0 || p.dv % 32 != 0) return false;  // 64-byte staging pieces
   if (p.dk <= 64 && p.dv <= 64) c.D = 64;
@@ -148,14 +159,14 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
   const int es = dlt_elem_size(p.dtype);
   // delta = rowsum(o * dO): folded into the dQ kernel when o can be read in 16-byte pieces like the
   // other operands, else the pre-pass kernel shared with the generic path
-  const bool fuse_delta = vec_ok(t.o, t.os, 4, p.dv, es) && t.os[2] < ((int64_t)1 << 20);
+  const bool fuse_delta = tvec_ok(t.o, t.os, p.dv, es) && t.os[2] < ((int64_t)1 << 20);
   BwdArgs d;
   d.p = p;
   d.o = t.o; d.d_o = t.d_o; d.delta = t.delta;
-  for (int i = 0; i < 4; i++) { d.os[i] = t.os[i]; d.dos[i] = t.dos[i]; }
+  for (int i = 0; i < 5; i++) { d.os[i] = t.os[i]; d.dos[i] = t.dos[i]; }
   for (int i = 0; i < 3; i++) d.ls[i] = t.ls[i];
-  d.o_vec = vec_ok(t.o, t.os, 4, p.dv, es);
-  d.do_vec = vec_ok(t.d_o, t.dos, 4, p.dv, es);
+  d.o_vec = tvec_ok(t.o, t.os, p.dv, es);
+  d.do_vec = tvec_ok(t.d_o, t.dos, p.dv, es);
   d.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
   if (!fuse_delta) {
     int rc = c.D == 64 ? dlt_launch_delta_64_64(d, stream) : dlt_launch_delta_128_128(d, stream);
@@ -181,9 +192,9 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
   }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
   a.q_vec = 1; a.k_vec = 1; a.v_vec = 1; a.do_vec = 1;
-  a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, es);
-  a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, es);
-  a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, es);
+  a.dq_vec = tvec_ok(t.dq, t.dqs, p.dk, es);
+  a.dk_vec = tvec_ok(t.dk, t.dks, p.dk, es);
+  a.dv_vec = tvec_ok(t.dv, t.dvs, p.dv, es);
   a.rope_pbit = c.pbit;
   a.rope_mode = c.rope_mode;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
@@ -201,8 +212,8 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
   for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
-  a.q_vec = vec_ok(t.q, t.qs, 4, p.dk, es);
-  a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, es);
+  a.q_vec = tvec_ok(t.q, t.qs, p.dk, es);
+  a.o_vec = tvec_ok(t.out_o, t.os, p.dv, es);
   a.rope_pbit = c.pbit;
   a.rope_mode = c.rope_mode;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
@@ -222,28 +233,29 @@ bool flash_eligible(const AttnProblem& p, const AttnTensors& t, bool with_do) {
   }
   if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
   const int es = 2;
-  if (!vec_ok(t.q, t.qs, 4, p.dk, es) || !vec_ok(t.k, t.ks, 4, p.dk, es) || !vec_ok(t.v, t.vs, 4, p.dv, es)) return false;
-  if (with_do && !vec_ok(t.d_o, t.dos, 4, p.dv, es)) return false;
+  if (!tvec_ok(t.q, t.qs, p.dk, es) || !tvec_ok(t.k, t.ks, p.dk, es) || !tvec_ok(t.v, t.vs, p.dv, es)) return false;
+  if (with_do && !tvec_ok(t.d_o, t.dos, p.dv, es)) return false;
   const int64_t lim = ((int64_t)1 << 31) - 1;
   const int64_t nq = (int64_t)p.g.TR * p.g.XLq, nk = (int64_t)p.g.TR * p.g.XLk;  // tokens of one (batch, head)
-  if (nk * t.ks[2] * es > lim || nk * t.vs[2] * es > lim) return false;
-  if (nq * t.qs[2] * es > lim) return false;
-  if (with_do && nq * t.dos[2] * es > lim) return false;
+  if (slab_span(p, t.ks, nk) * es > lim || slab_span(p, t.vs, nk) * es > lim) return false;
+  if (slab_span(p, t.qs, nq) * es > lim) return false;
+  if (with_do && slab_span(p, t.dos, nq) * es > lim) return false;
   return true;
 }
 
 int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc, hipStream_t stream) {
   FlashArgs a;
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
-  for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
+  for (int i = 0; i < 5; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.tm = p.tm;
   a.B = p.B; a.H = p.H; a.Lq = p.g.XLq; a.Lk = p.g.XLk; a.dk = p.dk; a.dv = p.dv;
   const int own = 64 * FLASH_NP;
   a.nblk = (a.Lq + own - 1) / own;
   a.causal = p.g.mode == DLT_GEOM_CAUSAL;
   a.tile = p.g.mode == DLT_GEOM_SWA;
   a.g = p.g;
-  a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, 2);
+  a.o_vec = tvec_ok(t.out_o, t.os, p.dv, 2);
   const int chunk = FLASH_CK * (dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD), tile = own * (dc.DV * 2 + 16);
   a.lds_bytes = chunk > tile ? chunk : tile;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
@@ -261,13 +273,13 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   BwdArgs d;
   d.p = p;
   d.o = t.o; d.d_o = t.d_o; d.delta = t.delta;
-  for (int i = 0; i < 4; i++) { d.os[i] = t.os[i]; d.dos[i] = t.dos[i]; }
+  for (int i = 0; i < 5; i++) { d.os[i] = t.os[i]; d.dos[i] = t.dos[i]; }
   for (int i = 0; i < 3; i++) d.ls[i] = t.ls[i];
-  d.o_vec = vec_ok(t.o, t.os, 4, p.dv, 2);
+  d.o_vec = tvec_ok(t.o, t.os, p.dv, 2);
   d.do_vec = 1;
   d.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
   // delta = rowsum(o * dO): folded into the dQ kernel when o can be read in 16-byte pieces
-  const bool fuse_delta = vec_ok(t.o, t.os, 4, p.dv, 2) && (int64_t)p.g.TR * p.g.XLq * t.os[2] * 2 < ((int64_t)1 << 31);
+  const bool fuse_delta = tvec_ok(t.o, t.os, p.dv, 2) && slab_span(p, t.os, (int64_t)p.g.TR * p.g.XLq) * 2 < ((int64_t)1 << 31);
   if (!fuse_delta) {
     int rc = dc.id == 0 ? dlt_launch_delta_64_64(d, stream) : dc.id == 1 ? dlt_launch_delta_128_128(d, stream)
            : dc.id == 3 ? dlt_launch_delta_32_32(d, stream) : dlt_launch_delta_64_128(d, stream);
@@ -279,11 +291,12 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   a.delta_out = t.delta;
   a.fuse_delta = fuse_delta ? 1 : 0;
   a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < 5; i++) {
     a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; a.dos[i] = t.dos[i];
     a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
   }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.tm = p.tm;
   a.B = p.B; a.H = p.H; a.Lq = p.g.XLq; a.Lk = p.g.XLk; a.dk_ = p.dk; a.dv_ = p.dv;
   const int own = 64 * flash_np_q(dc.DK, dc.DV), own_kv = 64 * flash_np_kv(dc.DK, dc.DV);
   a.nblk_q = (a.Lq + own - 1) / own;
@@ -291,9 +304,9 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   a.causal = p.g.mode == DLT_GEOM_CAUSAL;
   a.tile = p.g.mode == DLT_GEOM_SWA;
   a.g = p.g;
-  a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, 2);
-  a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, 2);
-  a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, 2);
+  a.dq_vec = tvec_ok(t.dq, t.dqs, p.dk, 2);
+  a.dk_vec = tvec_ok(t.dk, t.dks, p.dk, 2);
+  a.dv_vec = tvec_ok(t.dv, t.dvs, p.dv, 2);
   const int chunk = FLASH_CK * (dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD);
   const int tile_q = own * (dc.DK * 2 + 16);
   const int tile_k = own_kv * (dc.DK * 2 + 16), tile_v = own_kv * (dc.DV * 2 + 16);
@@ -321,7 +334,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
   if (rc != DLT_OK) return rc;
   const int es = dlt_elem_size(p.dtype);
   {
-    const bool streamed[2] = {vec_ok(t.k, t.ks, 4, p.dk, es), vec_ok(t.v, t.vs, 4, p.dv, es)};
+    const bool streamed[2] = {tvec_ok(t.k, t.ks, p.dk, es), tvec_ok(t.v, t.vs, p.dv, es)};
     Swa1Class c;
     if (swa1_eligible(p, streamed, 2, c) && swa1_strides_fit(t)) {
       rc = swa1_forward(p, t, c, stream);
@@ -339,12 +352,12 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
   a.plan.off_b = a.plan.off_a + a.plan.chunk_rows * a.plan.chunk_x * PK;
   a.plan.off_c = a.plan.off_d = 0;
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
-  for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
+  for (int i = 0; i < 5; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
-  a.q_vec = vec_ok(t.q, t.qs, 4, p.dk, es);
-  a.k_vec = vec_ok(t.k, t.ks, 4, p.dk, es);
-  a.v_vec = vec_ok(t.v, t.vs, 4, p.dv, es);
-  a.o_vec = vec_ok(t.out_o, t.os, 4, p.dv, es);
+  a.q_vec = tvec_ok(t.q, t.qs, p.dk, es);
+  a.k_vec = tvec_ok(t.k, t.ks, p.dk, es);
+  a.v_vec = tvec_ok(t.v, t.vs, p.dv, es);
+  a.o_vec = tvec_ok(t.out_o, t.os, p.dv, es);
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   const int64_t grid = (int64_t)p.B * p.H * p.g.TR * a.plan.nblk_x;
   if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: grid too large");
@@ -362,8 +375,8 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
   if (rc != DLT_OK) return rc;
   const int es = dlt_elem_size(p.dtype);
   {
-    const bool streamed[4] = {vec_ok(t.q, t.qs, 4, p.dk, es), vec_ok(t.k, t.ks, 4, p.dk, es),
-                              vec_ok(t.v, t.vs, 4, p.dv, es), vec_ok(t.d_o, t.dos, 4, p.dv, es)};
+    const bool streamed[4] = {tvec_ok(t.q, t.qs, p.dk, es), tvec_ok(t.k, t.ks, p.dk, es),
+                              tvec_ok(t.v, t.vs, p.dv, es), tvec_ok(t.d_o, t.dos, p.dv, es)};
     Swa1Class c;
     if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(t)) return swa1_backward(p, t, c, stream);
   }
@@ -380,19 +393,19 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
   a.p = p;
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.o; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
   a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
-  for (int i = 0; i < 4; i++) {
+  for (int i = 0; i < 5; i++) {
     a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; a.dos[i] = t.dos[i];
     a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
   }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
-  a.q_vec = vec_ok(t.q, t.qs, 4, p.dk, es);
-  a.k_vec = vec_ok(t.k, t.ks, 4, p.dk, es);
-  a.v_vec = vec_ok(t.v, t.vs, 4, p.dv, es);
-  a.o_vec = vec_ok(t.o, t.os, 4, p.dv, es);
-  a.do_vec = vec_ok(t.d_o, t.dos, 4, p.dv, es);
-  a.dq_vec = vec_ok(t.dq, t.dqs, 4, p.dk, es);
-  a.dk_vec = vec_ok(t.dk, t.dks, 4, p.dk, es);
-  a.dv_vec = vec_ok(t.dv, t.dvs, 4, p.dv, es);
+  a.q_vec = tvec_ok(t.q, t.qs, p.dk, es);
+  a.k_vec = tvec_ok(t.k, t.ks, p.dk, es);
+  a.v_vec = tvec_ok(t.v, t.vs, p.dv, es);
+  a.o_vec = tvec_ok(t.o, t.os, p.dv, es);
+  a.do_vec = tvec_ok(t.d_o, t.dos, p.dv, es);
+  a.dq_vec = tvec_ok(t.dq, t.dqs, p.dk, es);
+  a.dk_vec = tvec_ok(t.dk, t.dks, p.dk, es);
+  a.dv_vec = tvec_ok(t.dv, t.dvs, p.dv, es);
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   a.n_tokens_q = (int64_t)p.g.TR * p.g.XLq;
 

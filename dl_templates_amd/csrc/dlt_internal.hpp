@@ -49,7 +49,9 @@ struct AttnTensors {
   void *out_o, *dq, *dk, *dv;
   float* lse;        // written by forward, read by backward
   float* delta;      // scratch written by the backward pre-pass
-  int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  // element strides [B, H, N, D]; entry 4 is only used with an image token map (AttnProblem::tm):
+  // then [2] is the stride of a pixel column and [4] the stride of a pixel row
+  int64_t qs[5], ks[5], vs[5], os[5], dos[5], dqs[5], dks[5], dvs[5], ls[3];
 };
 
 struct AttnProblem {
@@ -58,6 +60,7 @@ struct AttnProblem {
   float sm_scale;
   int32_t dtype;
   RopeDev rope;
+  DltTokMap tm;  // token -> element offset map of q, k, v, o and the gradients (lse2 / delta stay [B, H, N])
 };
 
 int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream);

@@ -22,7 +22,7 @@ int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
 
 template <typename TIO>
 int flash_launch_fwd_t(const FlashArgs& a, int grid, hipStream_t stream) {
-  if (a.tile) return flash_launch_fwd_c<TIO, 2>(a, grid, stream);
+  if (a.tile) return a.tm.img ? flash_launch_fwd_c<TIO, 3>(a, grid, stream) : flash_launch_fwd_c<TIO, 2>(a, grid, stream);
   return a.causal ? flash_launch_fwd_c<TIO, 1>(a, grid, stream) : flash_launch_fwd_c<TIO, 0>(a, grid, stream);
 }
 
@@ -61,7 +61,7 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
 
 template <typename TIO>
 int flash_launch_bwd_t(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
-  if (a.tile) return flash_launch_bwd_c<TIO, 2>(a, grid_kv, grid_q, stream);
+  if (a.tile) return a.tm.img ? flash_launch_bwd_c<TIO, 3>(a, grid_kv, grid_q, stream) : flash_launch_bwd_c<TIO, 2>(a, grid_kv, grid_q, stream);
   return a.causal ? flash_launch_bwd_c<TIO, 1>(a, grid_kv, grid_q, stream) : flash_launch_bwd_c<TIO, 0>(a, grid_kv, grid_q, stream);
 }
 }  // namespace

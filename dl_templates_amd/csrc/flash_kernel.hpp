@@ -1,6 +1,7 @@
 // Dense, causal and tile-window flash attention forward for gfx950 with separate qk / vo head dims.
 //
-// MODE 0 dense, 1 causal, 2 tiled 2D sliding window with b_size a multiple of 16 (the regime
+// MODE 0 dense, 1 causal, 2 and 3 tiled 2D sliding window with b_size a multiple of 16 (3: the tensors are
+// images, tokens are addressed through the pixel map of DltTokMap; the regime
 // tiled_swa_fwd_large_kernel was written for, src/tiled_swa.py:142-244): a block of 16 own tokens
 // lies inside one tile and every 16-token half of a streamed block lies inside one tile, so the
 // window test is wave-uniform per half: no per-element mask exists, invisible blocks are skipped.
@@ -52,12 +53,12 @@ constexpr int flash_np_q(int dk, int dv) { return dk + dv > 192 ? 1 : FLASH_NP_D
 constexpr int flash_occ_fwd(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 3 : 2); }
 constexpr int flash_occ_q(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 3 : 2); }
 constexpr int flash_occ_kv(int dk, int dv, int mode) {
-  return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 2 : (dk + dv <= 192 && mode != 2 ? 3 : 2));
+  return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 2 : (dk + dv <= 192 && mode < 2 ? 3 : 2));
 }
 
 // One chunk of streamed tokens: first token (index inside the [N, D] slab), its x inside the grid
 // row (tile mode) or the sequence, and how many of the CK staged tokens exist.
-struct FlashChunk { int tok0, x, nvalid; };
+struct FlashChunk { int tok0, x, nvalid, row; };
 
 // Streamed tokens a workgroup visits.  Dense / causal: [first, len) of the sequence.  Tile mode:
 // for every grid row in [rlo, rhi] the x range [X0, X1) that some own token can see, CK at a time.
@@ -86,19 +87,59 @@ struct FlashWalk {
   }
   DLT_DEV FlashChunk at(int i) const {
     FlashChunk c;
-    if (MODE == 2) {
+    if (MODE >= 2) {
       const int ri = i / nxc;
       c.x = X0 + (i - ri * nxc) * CK;
-      c.tok0 = (rlo + ri) * XL + c.x;
+      c.row = rlo + ri;
+      c.tok0 = c.row * XL + c.x;
       c.nvalid = dlt_imin(CK, X1 - c.x);
     } else {
       c.x = first + i * CK;
+      c.row = 0;
       c.tok0 = c.x;
       c.nvalid = dlt_imin(CK, len - c.x);
     }
     return c;
   }
 };
+
+// Byte offset of streamed token j of chunk c inside its (batch, head) slab: a plain token stride, or
+// (IMG) the pixel map applied to the token's slot inside its grid row (two exact divisions; the
+// row part is wave-uniform).
+template <bool IMG>
+struct FlashAddr;
+template <>
+struct FlashAddr<false> {
+  int sn2;  // bytes between tokens
+  DLT_DEV uint32_t operator()(const FlashChunk& c, int j) const { return (uint32_t)((c.tok0 + j) * sn2); }
+};
+template <>
+struct FlashAddr<true> {
+  int sn2, sy2;  // bytes between pixel columns and between pixel rows
+  const DltTokMap* tm;
+  DLT_DEV uint32_t operator()(const FlashChunk& c, int j) const {
+    uint32_t i, x;
+    dlt_slot_pixel(*tm, (uint32_t)(c.x + j), i, x);
+    return (uint32_t)(((uint32_t)c.row * tm->bh + i) * (uint32_t)sy2 + x * (uint32_t)sn2);
+  }
+};
+template <bool IMG>
+DLT_DEV FlashAddr<IMG> flash_addr(const int64_t (&st)[5], const DltTokMap& tm) {
+  if constexpr (IMG) return FlashAddr<true>{(int)st[2] * 2, (int)st[4] * 2, &tm};
+  else return FlashAddr<false>{(int)st[2] * 2};
+}
+// what the tile writers take as the token stride: the plain stride, or (IMG) the pixel map
+template <bool IMG>
+DLT_DEV auto flash_tok(const int64_t (&st)[5], const DltTokMap& tm) {
+  if constexpr (IMG) return tok_addr(st, tm);
+  else return st[2];
+}
+// element offset of own token t (-1: none) for the loaders that take (base, stride, token)
+template <bool IMG>
+DLT_DEV int64_t flash_own_off(const int64_t (&st)[5], const DltTokMap& tm, int64_t t) {
+  if (t < 0) return t;
+  return IMG ? tok_addr(st, tm)(t) : t * st[2];
+}
 
 // workgroup -> (batch * head, grid row, first own x).  `rev`: heavy blocks first (causal).
 DLT_DEV void flash_block(int lin, int nblk, int TR, int own, bool rev, int& bh, int& r, int& x0) {
@@ -114,7 +155,8 @@ struct FlashArgs {
   const void *q, *k, *v;
   void* o;
   float* lse;
-  int64_t qs[4], ks[4], vs[4], os[4], ls[3];
+  int64_t qs[5], ks[5], vs[5], os[5], ls[3];
+  DltTokMap tm;
   int32_t B, H, Lq, Lk, dk, dv;
   int32_t nblk;       // workgroups per (batch, head) and grid row
   int32_t causal;
@@ -130,7 +172,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   typedef typename ComputeOf<TIO>::type CT;
   typedef typename TileOf<TIO>::type TL;
   extern __shared__ __align__(16) char smem[];
-  constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
+  constexpr bool CAUSAL = MODE == 1, TILE = MODE >= 2, IMG = MODE == 3;
   constexpr int PK = DK * 2 + FLASH_PAD, PV = DV * 2 + FLASH_PAD, PO = DV * (int)sizeof(TL) + 16;
   constexpr int KC = DK / 32, VB = DV / 16, NKB = CK / 32;
   constexpr int OWN = 64 * NP;
@@ -154,7 +196,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   const char* kb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1]);
   const char* vb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1]);
   TIO* ob = reinterpret_cast<TIO*>(a.o) + b * a.os[0] + h * a.os[1];
-  const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
+  const FlashAddr<IMG> ak = flash_addr<IMG>(a.ks, a.tm), av = flash_addr<IMG>(a.vs, a.tm);
   RopeDev no_rope = RopeDev{};
   const int own_base = TILE ? r_own * a.Lq : 0;                   // token index of own x = 0
 
@@ -176,13 +218,13 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   auto issue = [&](const FlashChunk& c) {
 #pragma unroll
     for (int it = 0; it < NKI; it++) {
-      const int key = c.tok0 + dlt_imin(kkey0 + it * (256 / KCH), c.nvalid - 1);
-      if (on_k) rk[it] = *reinterpret_cast<const u32x4*>(kb_ + (uint32_t)(key * sn2k + 16 * kc_));
+      const uint32_t off = ak(c, dlt_imin(kkey0 + it * (256 / KCH), c.nvalid - 1));
+      if (on_k) rk[it] = *reinterpret_cast<const u32x4*>(kb_ + (off + 16 * kc_));
     }
 #pragma unroll
     for (int it = 0; it < NVI; it++) {
-      const int key = c.tok0 + dlt_imin(vkey0 + it * (256 / VCH), c.nvalid - 1);
-      if (on_v) rv[it] = *reinterpret_cast<const u32x4*>(vb_ + (uint32_t)(key * sn2v + 16 * vc_));
+      const uint32_t off = av(c, dlt_imin(vkey0 + it * (256 / VCH), c.nvalid - 1));
+      if (on_v) rv[it] = *reinterpret_cast<const u32x4*>(vb_ + (off + 16 * vc_));
     }
   };
   auto commit = [&]() {
@@ -210,7 +252,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
       int rl, rh;
       dlt_key_range(a.g, r_own, wq0 + 16 * p, rl, rh, vlo[p], vhi[p]);
     }
-    swa1_load_own<TIO, CT, DK>(qf[p], qb, a.qs[2], a.dk, tq[p], g, no_rope, false);
+    swa1_load_own<TIO, CT, DK>(qf[p], qb, 1, a.dk, flash_own_off<IMG>(a.qs, a.tm, tq[p]), g, no_rope, false);
   }
 
   float m_run[NP];
@@ -368,7 +410,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
     if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
   }
   __syncthreads();
-  store_tile<TIO, TL, DV>(smem, PO, ob, a.os[2], a.os[3], a.dv, a.o_vec != 0, OWN,
+  store_tile<TIO, TL, DV>(smem, PO, ob, flash_tok<IMG>(a.os, a.tm), a.os[3], a.dv, a.o_vec != 0, OWN,
                           [&](int row) { return x0 + row < a.Lq ? (int64_t)(own_base + x0 + row) : (int64_t)-1; }, no_rope, tid);
 }
 
@@ -383,7 +425,8 @@ struct FlashBwdArgs {
   const float *lse, *delta;
   float* delta_out;   // fuse_delta: the dQ kernel (launched first) stores delta = rowsum(o * dO) of its own queries
   void *dq, *dk, *dv;
-  int64_t qs[4], ks[4], vs[4], os[4], dos[4], dqs[4], dks[4], dvs[4], ls[3];
+  int64_t qs[5], ks[5], vs[5], os[5], dos[5], dqs[5], dks[5], dvs[5], ls[3];
+  DltTokMap tm;
   int32_t fuse_delta;
   int32_t B, H, Lq, Lk, dk_, dv_;
   int32_t nblk_q, nblk_k;
@@ -416,16 +459,17 @@ struct PairStage {
     for (int it = 0; it < NBI; it++) rb[it] = u32x4{0u, 0u, 0u, 0u};
   }
   // tokens past the end of the chunk are clamped onto its last token (the caller masks them)
-  DLT_DEV void issue(const char* a, int sn2a, const char* b, int sn2b, const FlashChunk& c) {
+  template <typename AD>
+  DLT_DEV void issue(const char* a, const AD& ada, const char* b, const AD& adb, const FlashChunk& c) {
 #pragma unroll
     for (int it = 0; it < NAI; it++) {
-      const int tok = c.tok0 + dlt_imin(akey0 + it * (256 / ACH), c.nvalid - 1);
-      if (on_a) ra[it] = *reinterpret_cast<const u32x4*>(a + (uint32_t)(tok * sn2a + 16 * ac));
+      const uint32_t off = ada(c, dlt_imin(akey0 + it * (256 / ACH), c.nvalid - 1));
+      if (on_a) ra[it] = *reinterpret_cast<const u32x4*>(a + (off + 16 * ac));
     }
 #pragma unroll
     for (int it = 0; it < NBI; it++) {
-      const int tok = c.tok0 + dlt_imin(bkey0 + it * (256 / BCH), c.nvalid - 1);
-      if (on_b) rb[it] = *reinterpret_cast<const u32x4*>(b + (uint32_t)(tok * sn2b + 16 * bc));
+      const uint32_t off = adb(c, dlt_imin(bkey0 + it * (256 / BCH), c.nvalid - 1));
+      if (on_b) rb[it] = *reinterpret_cast<const u32x4*>(b + (off + 16 * bc));
     }
   }
   DLT_DEV void commit(char* sa, int pa, char* sb, int pb) const {
@@ -439,8 +483,8 @@ struct PairStage {
 };
 
 // accumulators (C layout, [dim][own token]) of NP blocks -> LDS tile -> HBM rows
-template <typename TIO, int D, int NP>
-DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO* base, int64_t sn, int64_t sd, int dact,
+template <typename TIO, int D, int NP, typename SN>
+DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO* base, const SN& sn, int64_t sd, int dact,
                               bool vec, int own_base, int x0, int len, int wave, int n, int g, int tid) {
   typedef typename TileOf<TIO>::type TL;
   constexpr int PT = D * (int)sizeof(TL) + 16;
@@ -464,7 +508,7 @@ template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
 __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
+  constexpr bool CAUSAL = MODE == 1, TILE = MODE >= 2, IMG = MODE == 3;
   constexpr int PK = DK * 2 + FLASH_PAD, PV = DV * 2 + FLASH_PAD;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, NKB = CK / 32;
   constexpr int OWN = 64 * NP;
@@ -484,7 +528,7 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
   const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
   const char* kb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1]);
   const char* vb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1]);
-  const int sn2k = (int)a.ks[2] * 2, sn2v = (int)a.vs[2] * 2;
+  const FlashAddr<IMG> ak = flash_addr<IMG>(a.ks, a.tm), av = flash_addr<IMG>(a.vs, a.tm);
   RopeDev no_rope = RopeDev{};
   const int own_base = TILE ? r_own * a.Lq : 0;
 
@@ -494,7 +538,7 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
 
   PairStage<DK, DV, CK> st;
   st.init(tid, a.dk_, a.dv_);
-  if (W.nchunks > 0) st.issue(kb_, sn2k, vb_, sn2v, W.at(0));
+  if (W.nchunks > 0) st.issue(kb_, ak, vb_, av, W.at(0));
 
   u32x4 qf[NP][KC], dof[NP][VC];
   float nlse[NP], del_n[NP];
@@ -509,15 +553,15 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
       int rl, rh;
       dlt_key_range(a.g, r_own, wq0 + 16 * p, rl, rh, vlo[p], vhi[p]);
     }
-    swa1_load_own<TIO, CT, DK>(qf[p], qb, a.qs[2], a.dk_, tq, g, no_rope, false);
-    swa1_load_own<TIO, CT, DV>(dof[p], dob, a.dos[2], a.dv_, tq, g, no_rope, false);
+    swa1_load_own<TIO, CT, DK>(qf[p], qb, 1, a.dk_, flash_own_off<IMG>(a.qs, a.tm, tq), g, no_rope, false);
+    swa1_load_own<TIO, CT, DV>(dof[p], dob, 1, a.dv_, flash_own_off<IMG>(a.dos, a.tm, tq), g, no_rope, false);
     const int64_t off = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
     nlse[p] = tq >= 0 ? -a.lse[off] : 0.f;
     if (a.fuse_delta != 0) {
       // the reference's pre-pass (src/flash_attn.py:186-202) folded in: delta of the own queries
       const TIO* ob = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1];
       u32x4 of[VC];
-      swa1_load_own<TIO, CT, DV>(of, ob, a.os[2], a.dv_, tq, g, no_rope, false);
+      swa1_load_own<TIO, CT, DV>(of, ob, 1, a.dv_, flash_own_off<IMG>(a.os, a.tm, tq), g, no_rope, false);
       float part = 0.f;
 #pragma unroll
       for (int c_ = 0; c_ < VC; c_++) {
@@ -609,7 +653,7 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
   };
   // last chunk peeled off: unconditional prefetch and commit inside the loop (see the forward kernel)
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
-    st.issue(kb_, sn2k, vb_, sn2v, W.at(ci + 1));
+    st.issue(kb_, ak, vb_, av, W.at(ci + 1));
     consume(ci);
     __syncthreads();
     st.commit(sK, PK, sV, PV);
@@ -618,7 +662,7 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
   if (W.nchunks > 0) consume(W.nchunks - 1);
   __syncthreads();
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
-  flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, a.dqs[2], a.dqs[3], a.dk_, a.dq_vec != 0, own_base, x0, a.Lq, wave, n, g, tid);
+  flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, flash_tok<IMG>(a.dqs, a.tm), a.dqs[3], a.dk_, a.dq_vec != 0, own_base, x0, a.Lq, wave, n, g, tid);
 }
 
 // ---- dK / dV: own = keys, Q, dO, lse2 and delta stream
@@ -626,7 +670,7 @@ template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
 __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr bool CAUSAL = MODE == 1, TILE = MODE == 2;
+  constexpr bool CAUSAL = MODE == 1, TILE = MODE >= 2, IMG = MODE == 3;
   constexpr int PQ = DK * 2 + FLASH_PAD, PD = DV * 2 + FLASH_PAD;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16, NQB = CK / 32;
   constexpr int OWN = 64 * NP;
@@ -649,7 +693,7 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
   const char* dob = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1]);
   const float* lseb = a.lse + b * a.ls[0] + h * a.ls[1];
   const float* delb = a.delta + b * a.ls[0] + h * a.ls[1];
-  const int sn2q = (int)a.qs[2] * 2, sn2d = (int)a.dos[2] * 2;
+  const FlashAddr<IMG> aq = flash_addr<IMG>(a.qs, a.tm), ad = flash_addr<IMG>(a.dos, a.tm);
   RopeDev no_rope = RopeDev{};
   const int own_base = TILE ? r_own * a.Lk : 0;
 
@@ -661,7 +705,7 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
 
   PairStage<DK, DV, CK> st;
   st.init(tid, a.dk_, a.dv_);
-  if (W.nchunks > 0) st.issue(qb, sn2q, dob, sn2d, W.at(0));
+  if (W.nchunks > 0) st.issue(qb, aq, dob, ad, W.at(0));
   float r_lse = 0.f, r_del = 0.f;
   auto issue_scalars = [&](const FlashChunk& c) {
     if (tid < CK) {
@@ -685,8 +729,8 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
       int rl, rh;
       dlt_query_range(a.g, r_own, wk0 + 16 * p, rl, rh, vlo[p], vhi[p]);
     }
-    swa1_load_own<TIO, CT, DK>(kf[p], kb_, a.ks[2], a.dk_, tk, g, no_rope, false);
-    swa1_load_own<TIO, CT, DV>(vf[p], vb_, a.vs[2], a.dv_, tk, g, no_rope, false);
+    swa1_load_own<TIO, CT, DK>(kf[p], kb_, 1, a.dk_, flash_own_off<IMG>(a.ks, a.tm, tk), g, no_rope, false);
+    swa1_load_own<TIO, CT, DV>(vf[p], vb_, 1, a.dv_, flash_own_off<IMG>(a.vs, a.tm, tk), g, no_rope, false);
   }
   f32x4 dk_acc[NP][KB], dv_acc[NP][VB];
 #pragma unroll
@@ -785,7 +829,7 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
   };
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
     const FlashChunk cn = W.at(ci + 1);
-    st.issue(qb, sn2q, dob, sn2d, cn);
+    st.issue(qb, aq, dob, ad, cn);
     issue_scalars(cn);
     consume(ci);
     __syncthreads();
@@ -799,6 +843,6 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
   __syncthreads();
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
-  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, a.dks[2], a.dks[3], a.dk_, a.dk_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
-  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.dv_, a.dv_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
+  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, flash_tok<IMG>(a.dks, a.tm), a.dks[3], a.dk_, a.dk_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
+  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, flash_tok<IMG>(a.dvs, a.tm), a.dvs[3], a.dv_, a.dv_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
 }

@@ -11,6 +11,10 @@ backward (the reference raises, :660-661).
 ``TiledSwaRope`` is the fused RoPE-2D + attention op: it equals ``RotaryPE2D`` applied to
 q and k followed by ``TiledSwa`` (the composition of README.md:11) without writing the
 rotated q / k to HBM; its backward returns gradients for the un-rotated q and k.
+
+``TiledSwaImage`` takes q, k, v as images ``[B, IH, IW, heads, D]`` (the layout the reference's
+demo converts from with reshape / permute / reshape, src/tiled_swa.py:753-755) and returns o in
+the same layout; the kernels address pixels themselves, so no permuted copy is made on either side.
 """
 from __future__ import annotations
 
@@ -111,6 +115,66 @@ class TiledSwaRope(torch.autograd.Function):
         shape = _shape(q, k, v, *ctx.scalars)
         dq, dk, dv = _backward(q, k, v, o, m, do, shape, (idx, row_cs_buffer, col_cs_buffer))
         return (dq, dk, dv) + (None,) * 9
+
+
+def _image_shape(q, k, v, bh, bw, row_size, col_size, sm_scale):
+    B, IH, IW, H, KEY_DIM = q.shape
+    assert IH % bh == 0 and IW % bw == 0, "image size should be a multiple of the tile size"
+    assert k.shape == q.shape and v.shape[:4] == q.shape[:4]
+    assert q.dtype == k.dtype == v.dtype
+    shape = _lib.SwaShape(B, H, bh * bw, IH // bh, IW // bw, row_size, col_size, KEY_DIM, v.shape[-1], float(sm_scale),
+                          _lib.dtype_code(q))
+    return shape, _lib.SwaTile(bh, bw)
+
+
+class TiledSwaImage(torch.autograd.Function):
+    """``TiledSwa`` on image-layout tensors: q, k ``[B, IH, IW, heads, dk]``, v and o ``[B, IH, IW, heads, dv]``.
+
+    A tile is a block of ``bh x bw`` pixels (``b_size = bh * bw``); the window is ``row_size`` / ``col_size``
+    tiles to each side as in ``TiledSwa``.  Equals the reference's conversion to ``[B, heads, N, D]``
+    (src/tiled_swa.py:753-755, inverted), ``TiledSwa`` and the conversion back, without the copies.
+    """
+
+    @staticmethod
+    def forward(ctx, q, k, v, bh: int, bw: int, row_size: int, col_size: int, sm_scale: float):
+        shape, tile = _image_shape(q, k, v, bh, bw, row_size, col_size, sm_scale)
+        _lib.require_cuda(q, k, v)
+        B, IH, IW, H, _ = q.shape
+        o = torch.empty((B, IH, IW, H, v.shape[-1]), dtype=q.dtype, device=q.device)
+        lse = torch.empty((B, H, IH * IW), dtype=torch.float32, device=q.device)
+        with torch.cuda.device(q.device):
+            _lib.check(_lib.load().dlt_swa_fwd_image(
+                _lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v), _lib.strides(v),
+                _lib.ptr(o), _lib.strides(o), _lib.ptr(lse), _lib.strides(lse), shape, tile, None, _lib.stream_of(q)))
+        ctx.save_for_backward(q, k, v, lse, o)
+        ctx.scalars = (bh, bw, row_size, col_size, sm_scale)
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, lse, o = ctx.saved_tensors
+        shape, tile = _image_shape(q, k, v, *ctx.scalars)
+        _lib.require_cuda(q, k, v, o, lse, do)
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        delta = torch.empty_like(lse)
+        with torch.cuda.device(q.device):
+            _lib.check(_lib.load().dlt_swa_bwd_image(
+                _lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v), _lib.strides(v),
+                _lib.ptr(o), _lib.strides(o), _lib.ptr(do), _lib.strides(do),
+                _lib.ptr(lse), _lib.ptr(delta), _lib.strides(lse),
+                _lib.ptr(dq), _lib.strides(dq), _lib.ptr(dk), _lib.strides(dk), _lib.ptr(dv), _lib.strides(dv),
+                shape, tile, None, _lib.stream_of(q)))
+        return (dq, dk, dv) + (None,) * 5
+
+
+def swa_image_offsets(t_height: int, t_width: int, bh: int, bw: int, stride_y: int, stride_x: int,
+                      device="cuda") -> torch.Tensor:
+    """int64 [N]: element offset of every token's pixel, computed by the kernels' own token -> pixel routine."""
+    out = torch.empty((t_height * t_width * bh * bw,), dtype=torch.int64, device=device)
+    with torch.cuda.device(out.device):
+        _lib.check(_lib.load().dlt_swa_image_offsets(t_height, t_width, bh, bw, stride_y, stride_x, _lib.ptr(out),
+                                                     _lib.stream_of(out)))
+    return out
 
 
 def swa_neighbors(t_height: int, t_width: int, row_size: int, col_size: int, device="cuda") -> torch.Tensor:

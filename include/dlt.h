@@ -115,6 +115,41 @@ int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void* k, const 
 int dlt_swa_neighbors(int32_t t_height, int32_t t_width, int32_t row_size, int32_t col_size,
                       uint8_t* mask, void* stream);
 
+/* ---- the same operator on image-layout tensors ----------------------------------------------
+ * q, k, v, o and the gradients are images [B, IH, IW, heads, D] (five element strides each, all
+ * non-negative) with IH = t_height * bh and IW = t_width * bw; a tile is a block of bh x bw pixels,
+ * shape->b_size must equal bh * bw, and pixel (y, x) is token
+ *     n = ((y / bh * t_width + x / bw) * bh + y % bh) * bw + x % bw
+ * of the tile-major order dlt_swa_fwd uses: exactly the permutation the reference's demo applies
+ * around the operator to move between the two layouts (reshape -> permute(0, 2, 4, 3, 5, 1, 6) ->
+ * reshape, src/tiled_swa.py:753-755).  The kernels address pixels directly, so that pass over
+ * q, k, v (and over o and the three gradients) disappears.  lse2 / delta stay fp32 [B, heads, N] in
+ * tile-major token order, and `rope->idx` is indexed by that token number as well.  A call whose
+ * tiles are single pixels and whose pixel rows lie t_width pixel columns apart is run as the plain
+ * [B, H, N, D] view it is. */
+typedef struct {
+  int32_t bh, bw; /* pixels per tile, vertically and horizontally */
+} dlt_swa_tile_t;
+
+int dlt_swa_fwd_image(const void* q, const int64_t q_strides[5], const void* k, const int64_t k_strides[5],
+                      const void* v, const int64_t v_strides[5], void* o, const int64_t o_strides[5],
+                      float* lse2, const int64_t lse_strides[3], const dlt_swa_shape_t* shape,
+                      const dlt_swa_tile_t* tile, const dlt_rope_t* rope, void* stream);
+
+int dlt_swa_bwd_image(const void* q, const int64_t q_strides[5], const void* k, const int64_t k_strides[5],
+                      const void* v, const int64_t v_strides[5], const void* o, const int64_t o_strides[5],
+                      const void* d_o, const int64_t do_strides[5],
+                      const float* lse2, float* delta, const int64_t lse_strides[3],
+                      void* dq, const int64_t dq_strides[5], void* dk, const int64_t dk_strides[5],
+                      void* dv, const int64_t dv_strides[5], const dlt_swa_shape_t* shape,
+                      const dlt_swa_tile_t* tile, const dlt_rope_t* rope, void* stream);
+
+/* Debug export: offsets[n] = y * stride_y + x * stride_x for the pixel (y, x) of token n, n in
+ * [0, t_height * t_width * bh * bw), computed on the device by the SAME token -> pixel routine the
+ * attention kernels use (the inverse of the permutation of src/tiled_swa.py:753-755). */
+int dlt_swa_image_offsets(int32_t t_height, int32_t t_width, int32_t bh, int32_t bw, int64_t stride_y,
+                          int64_t stride_x, int64_t* offsets, void* stream);
+
 /* ---- flash attention with separate qk / vo head dims -----------------------------------
  * q [B,H,Lq,dk], k [B,H,Lk,dk], v [B,H,Lk,dv], o [B,H,Lq,dv], lse2 fp32 [B,H,Lq].
  * Replaces _attn_fwd (src/flash_attn.py:81-172) and _attention.forward (:455-490); unlike

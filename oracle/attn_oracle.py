@@ -21,6 +21,9 @@ of one reference function, cited as ``file:line`` relative to the reference tree
                              cos then sin).  PARITY UNPINNED for the frequency formula: the
                              file that defines it (src/rope2d.py) is absent from the reference.
 * ``swa_pairs``/``attn_flops`` - src/flash_attn.py:608-614 FLOP convention.
+* ``tokens_to_image``/``image_to_tokens`` - src/tiled_swa.py:753-755 (tile-major [B, H, N, D] to the
+                             image layout [B, IH, IW, H, D] and back); ``image_token_index`` is the
+                             same map as a closed form, pinned against it and against loops.
 
 Pinning status: the reference holds no golden vectors for this path.  Each
 function above is pinned in ``tests/test_oracle.py`` by closed forms (neighbour
@@ -37,6 +40,43 @@ import torch
 import torch.nn.functional as F
 
 MASK_VALUE = -1e6  # src/tiled_swa.py:712 uses an additive -1e6, not -inf
+
+
+# ------------------------------------------------------------------ layout adapters
+def tokens_to_image(x: torch.Tensor, t_height: int, t_width: int, bh: int, bw: int) -> torch.Tensor:
+    """[B, H, N, D] in tile-major token order -> image [B, t_height*bh, t_width*bw, H, D].
+
+    src/tiled_swa.py:753-755: reshape to (B, H, TH, TW, BH, BW, D), permute (0, 2, 4, 3, 5, 1, 6),
+    reshape to (B, TH*BH, TW*BW, H, D).
+    """
+    B, H, N, D = x.shape
+    assert N == t_height * t_width * bh * bw
+    return (x.reshape(B, H, t_height, t_width, bh, bw, D).permute(0, 2, 4, 3, 5, 1, 6)
+            .reshape(B, t_height * bh, t_width * bw, H, D))
+
+
+def image_to_tokens(x: torch.Tensor, t_height: int, t_width: int, bh: int, bw: int) -> torch.Tensor:
+    """Inverse of ``tokens_to_image``: image [B, IH, IW, H, D] -> [B, H, N, D]."""
+    B, IH, IW, H, D = x.shape
+    assert IH == t_height * bh and IW == t_width * bw
+    return (x.reshape(B, t_height, bh, t_width, bw, H, D).permute(0, 5, 1, 3, 2, 4, 6)
+            .reshape(B, H, t_height * t_width * bh * bw, D))
+
+
+def image_token_index(t_height: int, t_width: int, bh: int, bw: int) -> np.ndarray:
+    """int64 [IH, IW]: token number of every pixel, n = ((y//bh * TW + x//bw) * bh + y%bh) * bw + x%bw."""
+    y = np.arange(t_height * bh, dtype=np.int64)[:, None]
+    x = np.arange(t_width * bw, dtype=np.int64)[None, :]
+    return ((y // bh * t_width + x // bw) * bh + y % bh) * bw + x % bw
+
+
+def image_token_offsets(t_height: int, t_width: int, bh: int, bw: int, stride_y: int, stride_x: int) -> np.ndarray:
+    """int64 [N]: offset y * stride_y + x * stride_x of the pixel (y, x) that holds token n."""
+    idx = image_token_index(t_height, t_width, bh, bw)
+    out = np.empty(idx.size, dtype=np.int64)
+    yy, xx = np.meshgrid(np.arange(idx.shape[0], dtype=np.int64), np.arange(idx.shape[1], dtype=np.int64), indexing="ij")
+    out[idx.reshape(-1)] = (yy * stride_y + xx * stride_x).reshape(-1)
+    return out
 
 
 # --------------------------------------------------------------------------- a1

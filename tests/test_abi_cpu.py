@@ -44,6 +44,12 @@ def test_argument_validation_happens_before_any_launch():
     shape = L.SwaShape(1, 1, 1, 4, 4, 1, 1, 512, 64, 1.0, 0)
     rc = lib.dlt_swa_fwd(one, st4, one, st4, one, st4, one, st4, one, st3, shape, None, None)
     assert rc == 2 and b"head dims" in lib.dlt_last_error()
+    st5 = (ctypes.c_int64 * 5)(1, 1, 1, 1, 1)
+    shape = L.SwaShape(1, 1, 6, 4, 4, 1, 1, 64, 64, 1.0, 0)  # tile of 2 x 2 pixels is not 6 tokens
+    rc = lib.dlt_swa_fwd_image(one, st5, one, st5, one, st5, one, st5, one, st3, shape, L.SwaTile(2, 2), None, None)
+    assert rc == 1 and b"b_size" in lib.dlt_last_error()
+    rc = lib.dlt_swa_image_offsets(0, 4, 2, 2, 8, 1, one, None)
+    assert rc == 1 and b"grid" in lib.dlt_last_error()
     fshape = L.FlashShape(1, 1, 8, 16, 64, 64, 1.0, 1, 0)  # causal with Lq != Lk
     rc = lib.dlt_flash_fwd(one, st4, one, st4, one, st4, one, st4, one, st3, fshape, None)
     assert rc == 1 and b"causal" in lib.dlt_last_error()

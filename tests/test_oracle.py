@@ -221,3 +221,47 @@ def test_composed_rope_swa_grads_are_autograd_of_composition():
     assert torch.allclose(o, oa.detach(), atol=1e-6)
     assert torch.allclose(dq, qa.grad, atol=1e-5) and torch.allclose(dk, ka.grad, atol=1e-5)
     assert torch.allclose(dv, va.grad, atol=1e-5)
+
+
+# ---- layout adapters (src/tiled_swa.py:753-755) -------------------------------------------------
+@pytest.mark.parametrize("th,tw,bh,bw", [(2, 3, 4, 4), (3, 2, 2, 5), (4, 5, 1, 1), (1, 4, 3, 1), (5, 1, 1, 7)])
+def test_image_layout_three_formulations_agree(th, tw, bh, bw):
+    """reshape/permute (the reference's text), the closed-form index and plain loops give one map."""
+    B, H, D = 2, 3, 4
+    N = th * tw * bh * bw
+    x = torch.arange(B * H * N * D, dtype=torch.float32).reshape(B, H, N, D)
+    img = orc.tokens_to_image(x, th, tw, bh, bw)
+    assert img.shape == (B, th * bh, tw * bw, H, D)
+    assert torch.equal(orc.image_to_tokens(img, th, tw, bh, bw), x)          # inverse
+    index = orc.image_token_index(th, tw, bh, bw)
+    assert sorted(index.reshape(-1).tolist()) == list(range(N))               # a permutation
+    for y in range(th * bh):                                                  # loops: tile, then pixel inside the tile
+        for xx in range(tw * bw):
+            tile = (y // bh) * tw + xx // bw
+            n = tile * bh * bw + (y % bh) * bw + xx % bw
+            assert index[y, xx] == n
+            assert torch.equal(img[:, y, xx], x[:, :, n])
+    sy, sx = 1000, 7
+    off = orc.image_token_offsets(th, tw, bh, bw, sy, sx)
+    for n in (0, N // 2, N - 1):
+        y, xx = np.argwhere(index == n)[0]
+        assert off[n] == y * sy + xx * sx
+
+
+def test_image_layout_attention_commutes_with_the_adapter():
+    """Attention on tokens and on the image are the same numbers in two layouts; the tiles of the image
+    are bh x bw pixel blocks whose neighbour sets are those of the tile grid."""
+    th, tw, bh, bw, H, d = 3, 4, 2, 2, 2, 8
+    q, k, v, _ = orc.make_qkv(5, 1, H, th * tw * bh * bw, th * tw * bh * bw, d, d)
+    o = orc.tiled_swa_ref(q, k, v, bh * bw, th, tw, 1, 1, 0.3)
+    o_img = orc.tokens_to_image(o, th, tw, bh, bw)
+    # pixel (y, x) attends pixel (y', x') iff their tiles are neighbours: brute force on the image
+    qi, ki, vi = (orc.tokens_to_image(t, th, tw, bh, bw) for t in (q, k, v))
+    for (y, x) in [(0, 0), (3, 5), (5, 7), (2, 2)]:
+        ys = [yy for yy in range(th * bh) if abs(yy // bh - y // bh) <= 1]
+        xs = [xx for xx in range(tw * bw) if abs(xx // bw - x // bw) <= 1]
+        for h in range(H):
+            keys = torch.stack([ki[0, yy, xx, h] for yy in ys for xx in xs])
+            vals = torch.stack([vi[0, yy, xx, h] for yy in ys for xx in xs])
+            p = torch.softmax(keys @ qi[0, y, x, h] * 0.3, dim=0)
+            assert torch.allclose(p @ vals, o_img[0, y, x, h], atol=1e-5)
