@@ -5,7 +5,9 @@
 
 One "step" is one forward + backward pass of the fused RoPE-2D + tiled 2D sliding-window
 attention over one synthetic batch of benchmark config 3 (bf16, B=2, H=8, 64x64 token grid,
-d=64, 13x13 window), inputs resident in HBM.  `value` is the effective TFLOP/s of that
+d=64, 13x13 window), inputs resident in HBM: the forward kernel rotates q and k as it loads its
+tiles and keeps the rotated tensors, the backward kernels read those and rotate dq / dk back as they
+store them (dlt_swa_fwd_rot / dlt_swa_bwd_rot).  `value` is the effective TFLOP/s of that
 step (in-window FLOPs only: fwd 2*pairs*(dk+dv), bwd 2*pairs*(3dk+2dv)).  The JSON line also
 carries the roofline of the dominant kernel (per-kernel HIP-event durations taken inside the
 timed steps), the standalone RoPE-2D bandwidth (config 2), configs 4 / 5 as extras, and a CPU
@@ -117,11 +119,16 @@ def try_graph(wl, steps, warmup):
 
 # ------------------------------------------------------------------------------------------ SWA
 class SwaWorkload:
-    def __init__(self, name, B, H, th, tw, W, d, fused_rope, nsets, seed=0, dtype=torch.bfloat16, b_size=1, scale=None):
+    def __init__(self, name, B, H, th, tw, W, d, fused_rope, nsets, seed=0, dtype=torch.bfloat16, b_size=1, scale=None,
+                 keep_rotated=True):
         from dl_templates_amd import _lib, tiled_swa
         from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
         from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as Rope
         self.name, self.B, self.H, self.th, self.tw, self.W, self.d = name, B, H, th, tw, W, d
+        # fused rotation: the forward pass keeps the rotated q, k for the backward pass (dlt_swa_fwd_rot /
+        # dlt_swa_bwd_rot, what TiledSwaRope does by default) or every tile load of the backward kernels
+        # rotates again (dlt_swa_fwd / dlt_swa_bwd with the rotary operands)
+        self.keep_rotated = bool(fused_rope and keep_rotated)
         dev = torch.device("cuda:0")
         N = th * tw * b_size
         self.sets = []
@@ -131,7 +138,8 @@ class SwaWorkload:
             lse = torch.empty((B, H, N), dtype=torch.float32, device=dev)
             delta = torch.empty_like(lse)
             dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-            self.sets.append((q, k, v, do, o, lse, delta, dq, dk, dv))
+            rot = (torch.empty_like(q), torch.empty_like(k)) if self.keep_rotated else (None, None)
+            self.sets.append((q, k, v, do, o, lse, delta, dq, dk, dv) + rot)
         self.shape = _lib.SwaShape(B, H, b_size, th, tw, W, W, d, d, scale if scale is not None else 1.0 / math.sqrt(d),
                                    _lib.dtype_code(self.sets[0][0]))
         self.rope = None
@@ -146,6 +154,8 @@ class SwaWorkload:
         self.lib = _lib.load()
         self._lib = _lib
         self.stream = _lib.stream_of(self.sets[0][0])
+        self._fwd = self.lib.dlt_swa_fwd_rot if self.keep_rotated else self.lib.dlt_swa_fwd
+        self._bwd = self.lib.dlt_swa_bwd_rot if self.keep_rotated else self.lib.dlt_swa_bwd
         self.calls = [self._build_calls(s) for s in self.sets]
         self.i = 0
         self.pairs = swa_pairs(B, H, b_size, th, tw, W, W)
@@ -154,10 +164,14 @@ class SwaWorkload:
 
     def _build_calls(self, s):
         L = self._lib
-        q, k, v, do, o, lse, delta, dq, dk, dv = s
+        q, k, v, do, o, lse, delta, dq, dk, dv, q_rot, k_rot = s
         fwd = (L.ptr(q), L.strides(q), L.ptr(k), L.strides(k), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
-               L.ptr(lse), L.strides(lse), self.shape, self.rope, self.stream)
-        bwd = (L.ptr(q), L.strides(q), L.ptr(k), L.strides(k), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
+               L.ptr(lse), L.strides(lse))
+        if self.keep_rotated:
+            fwd += (L.ptr(q_rot), L.strides(q_rot), L.ptr(k_rot), L.strides(k_rot))
+        fwd += (self.shape, self.rope, self.stream)
+        qb, kb = (q_rot, k_rot) if self.keep_rotated else (q, k)
+        bwd = (L.ptr(qb), L.strides(qb), L.ptr(kb), L.strides(kb), L.ptr(v), L.strides(v), L.ptr(o), L.strides(o),
                L.ptr(do), L.strides(do), L.ptr(lse), L.ptr(delta), L.strides(lse), L.ptr(dq), L.strides(dq),
                L.ptr(dk), L.strides(dk), L.ptr(dv), L.strides(dv), self.shape, self.rope, self.stream)
         return fwd, bwd
@@ -165,15 +179,15 @@ class SwaWorkload:
     def step(self):
         fwd, bwd = self.calls[self.i % len(self.calls)]
         self.i += 1
-        rc = self.lib.dlt_swa_fwd(*fwd)
-        rc = rc or self.lib.dlt_swa_bwd(*bwd)
+        rc = self._fwd(*fwd)
+        rc = rc or self._bwd(*bwd)
         if rc:
             self._lib.check(rc)
 
     def fwd_only(self):
         fwd, _ = self.calls[self.i % len(self.calls)]
         self.i += 1
-        rc = self.lib.dlt_swa_fwd(*fwd)
+        rc = self._fwd(*fwd)
         if rc:
             self._lib.check(rc)
 
@@ -382,7 +396,8 @@ def main():
     ms_eager, wall_eager = Timer.run(wl.step, K, W)
     kb = kernel_breakdown(wl.step, K)
     ms_graph = try_graph(wl, K, W)
-    ms_step = ms_graph if ms_graph is not None else ms_eager
+    # the same K steps were run twice, as eager launches and replayed from a HIP graph: the faster one counts
+    ms_step = min(ms_graph, ms_eager) if ms_graph is not None else ms_eager
     flops_step = wl.flops_fwd + wl.flops_bwd
     value = flops_step / (ms_step * 1e-3) / 1e12
 
@@ -400,7 +415,7 @@ def main():
             kernels[k_]["frac_mfma_peak"] = kernels[k_]["eff_tflops"] / PEAK_BF16_TFLOPS
 
     extra = {"ms_per_step_eager_events": ms_eager, "ms_per_step_eager_wall": wall_eager, "ms_per_step_graph": ms_graph,
-             "step_source": "hip graph replay" if ms_graph is not None else "eager launches",
+             "step_source": "hip graph replay" if ms_graph is not None and ms_graph <= ms_eager else "eager launches",
              "frac_mfma_peak_effective": value / PEAK_BF16_TFLOPS, "kernels": kernels,
              "hbm_floor_ms": 101e6 / (PEAK_HBM_GBPS * 1e9) * 1e3}
 
@@ -409,6 +424,14 @@ def main():
     extra["copy_bandwidth"] = copy_bandwidth()
 
     if not args.quick:
+        # the same step when nothing but the caller's q, k is kept: every K / Q tile load of the backward
+        # kernels rotates again (dlt_swa_fwd / dlt_swa_bwd with the rotary operands)
+        wl2 = SwaWorkload("C3", 2, 8, 64, 64, 6, 64, fused_rope=True, nsets=4, keep_rotated=False)
+        ms2, _ = Timer.run(wl2.step, K, W)
+        kb2 = kernel_breakdown(wl2.step, K)
+        extra["C3_rotation_in_every_tile_load"] = {"ms_per_step_eager_events": ms2, "eff_tflops": flops_step / (ms2 * 1e-3) / 1e12,
+                                                   "kernels_ms": {k_: v_["avg_ms"] for k_, v_ in kb2.items()}}
+        del wl2
         for name, (B, H, th, tw, Wn, d) in {"C4_128x128": (1, 16, 128, 128, 10, 128), "C4_96x160": (1, 16, 96, 160, 10, 128)}.items():
             w4 = SwaWorkload(name, B, H, th, tw, Wn, d, fused_rope=False, nsets=1)
             ms4, _ = Timer.run(w4.step, max(K // 5, 3), 2)
@@ -468,7 +491,7 @@ def main():
         "warmup": W, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "C3: fused RoPE-2D + tiled 2D SWA fwd+bwd, B=2 H=8 64x64 grid b_size=1 d=64 13x13 window, "
-                               "bf16, 5% no-PE tokens, 4 input sets cycled",
+                               "bf16, 5% no-PE tokens, 4 input sets cycled; rotated q, k kept by the forward pass for the backward pass",
                    "peak_bf16_tflops": PEAK_BF16_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS},
         "roofline": roofline, "cpu_baseline": cpu,
         "rope2d_gbps": rope["cold"]["gbps"], "rope2d_frac_hbm": rope["cold"]["frac_of_hbm_peak"],

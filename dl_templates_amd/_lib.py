@@ -26,7 +26,7 @@ EXPORTS = (
     "dlt_last_error", "dlt_version", "dlt_rope2d", "dlt_rope2d_pair", "dlt_rope_pe_mask",
     "dlt_swa_fwd", "dlt_swa_bwd", "dlt_swa_neighbors", "dlt_flash_fwd", "dlt_flash_bwd",
     "dlt_timing_enable", "dlt_timing_collect", "dlt_debug_copy",
-    "dlt_swa_fwd_image", "dlt_swa_bwd_image", "dlt_swa_image_offsets",
+    "dlt_swa_fwd_image", "dlt_swa_bwd_image", "dlt_swa_image_offsets", "dlt_swa_fwd_rot", "dlt_swa_bwd_rot",
 )
 KERNEL_NAMES = ("rope2d", "attn_fwd", "attn_delta", "attn_bwd_kv", "attn_bwd_q")
 
@@ -106,6 +106,10 @@ def _declare(lib) -> None:
     lib.dlt_swa_fwd.argtypes = fwd + [POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
     lib.dlt_swa_bwd.restype = c_int
     lib.dlt_swa_bwd.argtypes = bwd + [POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
+    lib.dlt_swa_fwd_rot.restype = c_int
+    lib.dlt_swa_fwd_rot.argtypes = fwd + [c_void_p, P64, c_void_p, P64, POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
+    lib.dlt_swa_bwd_rot.restype = c_int
+    lib.dlt_swa_bwd_rot.argtypes = bwd + [POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
     lib.dlt_swa_fwd_image.restype = c_int
     lib.dlt_swa_fwd_image.argtypes = fwd + [POINTER(SwaShape), POINTER(SwaTile), POINTER(RopeDesc), c_void_p]
     lib.dlt_swa_bwd_image.restype = c_int

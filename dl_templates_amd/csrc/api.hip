@@ -133,6 +133,7 @@ int swa_problem(const char* who, const dlt_swa_shape_t* s, const dlt_rope_t* rop
     if (rc != DLT_OK) return rc;
   }
   p.rope = dlt_make_rope_dev(rope, 0);
+  p.rope_prerot = 0;
   p.tm = dlt_tokmap_none();
   return DLT_OK;
 }
@@ -148,6 +149,7 @@ int flash_problem(const char* who, const dlt_flash_shape_t* s, AttnProblem& p) {
   p.g.XLq = s->Lq; p.g.XLk = s->Lk;
   p.B = s->B; p.H = s->H; p.dk = s->dk; p.dv = s->dv; p.sm_scale = s->sm_scale; p.dtype = s->dtype;
   p.rope = dlt_make_rope_dev(nullptr, 0);
+  p.rope_prerot = 0;
   p.tm = dlt_tokmap_none();
   return DLT_OK;
 }
@@ -380,5 +382,49 @@ extern "C" int dlt_swa_bwd_image(const void* q, const int64_t q_strides[5], cons
     if (rc != DLT_OK) return rc;
   }
   image_finish(p, tile, mine, 8);
+  return dlt_attn_backward(p, t, (hipStream_t)stream);
+}
+
+// ---- fused rotation with the rotated q, k kept for the backward pass -------------------------------
+extern "C" int dlt_swa_fwd_rot(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                               const void* v, const int64_t v_strides[4], void* o, const int64_t o_strides[4],
+                               float* lse2, const int64_t lse_strides[3],
+                               void* q_rot, const int64_t q_rot_strides[4], void* k_rot, const int64_t k_rot_strides[4],
+                               const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream) {
+  const char* who = "swa_fwd_rot";
+  DLT_REQUIRE(rope != nullptr, "%s: rope is NULL", who);
+  AttnProblem p;
+  int rc = swa_problem(who, shape, rope, p);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  rc = fill_fwd(who, t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, lse2, lse_strides);
+  if (rc != DLT_OK) return rc;
+  DLT_REQUIRE(q_rot != nullptr && k_rot != nullptr && q_rot_strides != nullptr && k_rot_strides != nullptr,
+              "%s: q_rot / k_rot is NULL", who);
+  // other workgroups still read q and k while a workgroup stores its rotated tokens
+  DLT_REQUIRE(q_rot != q && k_rot != k && q_rot != k && k_rot != q && q_rot != k_rot,
+              "%s: q_rot and k_rot must be distinct buffers that do not alias q or k", who);
+  t.q_rot = q_rot; t.k_rot = k_rot;
+  cp4(t.qrs, q_rot_strides); cp4(t.krs, k_rot_strides);
+  return dlt_attn_forward(p, t, (hipStream_t)stream);
+}
+
+extern "C" int dlt_swa_bwd_rot(const void* q_rot, const int64_t q_rot_strides[4], const void* k_rot,
+                               const int64_t k_rot_strides[4], const void* v, const int64_t v_strides[4], const void* o,
+                               const int64_t o_strides[4], const void* d_o, const int64_t do_strides[4],
+                               const float* lse2, float* delta, const int64_t lse_strides[3],
+                               void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                               void* dv, const int64_t dv_strides[4],
+                               const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream) {
+  const char* who = "swa_bwd_rot";
+  DLT_REQUIRE(rope != nullptr, "%s: rope is NULL", who);
+  AttnProblem p;
+  int rc = swa_problem(who, shape, rope, p);
+  if (rc != DLT_OK) return rc;
+  p.rope_prerot = 1;
+  AttnTensors t;
+  rc = fill_bwd(who, t, q_rot, q_rot_strides, k_rot, k_rot_strides, v, v_strides, o, o_strides, d_o, do_strides, lse2, delta,
+                lse_strides, dq, dq_strides, dk, dk_strides, dv, dv_strides);
+  if (rc != DLT_OK) return rc;
   return dlt_attn_backward(p, t, (hipStream_t)stream);
 }

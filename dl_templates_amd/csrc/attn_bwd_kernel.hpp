@@ -130,6 +130,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
   const float* lseb = a.lse + b * a.ls[0] + h * a.ls[1];
   const float* delb = a.delta + b * a.ls[0] + h * a.ls[1];
   RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
+  if (a.p.rope_prerot) fwd_rope.enabled = 0;  // q and k arrive rotated
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
 
@@ -274,6 +275,7 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
   const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
   const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
   RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
+  if (a.p.rope_prerot) fwd_rope.enabled = 0;  // q and k arrive rotated
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
 

@@ -143,7 +143,7 @@ void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int
   plan.nblk_r = (p.g.TR + 3) / 4;
   plan.nblk_c = (p.g.TC + 15) / 16;
   const int ncgmax = c.wclass == 0 ? 4 : 6;
-  const bool wide = c.rope_mode == 0;  // must match WIDE in the kernels
+  const bool wide = c.rope_mode == 0 || c.rope_mode == 3;  // must match WIDE in the kernels
   plan.lds_bytes = cr * hcw * (swa1_pitch(c.D, ncgmax, 0, wide, kv) + swa1_pitch(c.D, ncgmax, 1, wide, kv)) + extra_bytes;
   const int own_tile = 64 * (c.D * 2 + 16);  // output tile of the epilogue
   if (plan.lds_bytes < own_tile) plan.lds_bytes = own_tile;
@@ -155,7 +155,9 @@ bool swa1_strides_fit(const AttnTensors& t) {
   return t.qs[2] < lim && t.ks[2] < lim && t.vs[2] < lim && (t.d_o == nullptr || t.dos[2] < lim);
 }
 
-int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c, hipStream_t stream) {
+int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c_in, hipStream_t stream) {
+  Swa1Class c = c_in;
+  if (p.rope_prerot && c.rope_mode != 0) c.rope_mode = 3;  // rotated q, k: plain tile loads, gradients rotated back on store
   const int es = dlt_elem_size(p.dtype);
   // delta = rowsum(o * dO): folded into the dQ kernel when o can be read in 16-byte pieces like the
   // other operands, else the pre-pass kernel shared with the generic path
@@ -212,6 +214,9 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
   for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.q_rot = c.rope_mode != 0 ? t.q_rot : nullptr;
+  a.k_rot = c.rope_mode != 0 ? t.k_rot : nullptr;
+  for (int i = 0; i < 4; i++) { a.qrs[i] = t.qrs[i]; a.krs[i] = t.krs[i]; }
   a.q_vec = tvec_ok(t.q, t.qs, p.dk, es);
   a.o_vec = tvec_ok(t.out_o, t.os, p.dv, es);
   a.rope_pbit = c.pbit;
@@ -337,9 +342,27 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
     const bool streamed[2] = {tvec_ok(t.k, t.ks, p.dk, es), tvec_ok(t.v, t.vs, p.dv, es)};
     Swa1Class c;
     if (swa1_eligible(p, streamed, 2, c) && swa1_strides_fit(t)) {
-      rc = swa1_forward(p, t, c, stream);
-      if (rc != -1) return rc;
+      // rotated side outputs come from the fused kernels only (16-byte rows); otherwise see below
+      const bool side_ok = t.q_rot == nullptr || (c.rope_mode != 0 && tvec_ok(t.q_rot, t.qrs, p.dk, es) &&
+                                                  tvec_ok(t.k_rot, t.krs, p.dk, es) && tvec_ok(t.q, t.qs, p.dk, es));
+      if (side_ok) {
+        rc = swa1_forward(p, t, c, stream);
+        if (rc != -1) return rc;
+      }
     }
+  }
+  if (t.q_rot != nullptr) {
+    // rotate q and k out of place, then run the plain operator on the rotated tensors (any kernel family)
+    rc = dlt_rope_rotate_copy(t.q, t.qs, t.q_rot, t.qrs, p.B, p.H, (int64_t)p.g.TR * p.g.XLq, p.dk, p.rope, p.dtype, stream);
+    if (rc == DLT_OK)
+      rc = dlt_rope_rotate_copy(t.k, t.ks, t.k_rot, t.krs, p.B, p.H, (int64_t)p.g.TR * p.g.XLk, p.dk, p.rope, p.dtype, stream);
+    if (rc != DLT_OK) return rc;
+    AttnProblem p2 = p;
+    p2.rope = dlt_make_rope_dev(nullptr, 0);
+    AttnTensors t2 = t;
+    t2.q = t.q_rot; t2.k = t.k_rot; t2.q_rot = t2.k_rot = nullptr;
+    for (int i = 0; i < 5; i++) { t2.qs[i] = t.qrs[i]; t2.ks[i] = t.krs[i]; }
+    return dlt_attn_forward(p2, t2, stream);
   }
   if (flash_eligible(p, t, false)) return flash_forward(p, t, dc, stream);
   const int np = p.g.mode == DLT_GEOM_SWA ? 1 : 2;

@@ -42,16 +42,21 @@ struct RopeDev {
 
 int dlt_validate_rope(const dlt_rope_t* rope, int64_t n_dim);
 RopeDev dlt_make_rope_dev(const dlt_rope_t* rope, int inverse);
+// dst = rotate(src) for [B, H, N, C] tensors with any strides (every element is copied)
+int dlt_rope_rotate_copy(const void* src, const int64_t* ss, void* dst, const int64_t* ds, int B, int H, int64_t N, int C,
+                         const RopeDev& rope, int dtype, hipStream_t stream);
 
 // ---- attention core (attn_fwd.hip / attn_bwd.hip) -------------------------------------
 struct AttnTensors {
   const void *q, *k, *v, *o, *d_o;
   void *out_o, *dq, *dk, *dv;
+  void *q_rot, *k_rot;  // forward: optional outputs, the rotated q and k (NULL: not wanted)
   float* lse;        // written by forward, read by backward
   float* delta;      // scratch written by the backward pre-pass
   // element strides [B, H, N, D]; entry 4 is only used with an image token map (AttnProblem::tm):
   // then [2] is the stride of a pixel column and [4] the stride of a pixel row
   int64_t qs[5], ks[5], vs[5], os[5], dos[5], dqs[5], dks[5], dvs[5], ls[3];
+  int64_t qrs[5], krs[5];
 };
 
 struct AttnProblem {
@@ -60,6 +65,7 @@ struct AttnProblem {
   float sm_scale;
   int32_t dtype;
   RopeDev rope;
+  int32_t rope_prerot;  // backward: q and k arrive rotated; only dq and dk are rotated (back) on store
   DltTokMap tm;  // token -> element offset map of q, k, v, o and the gradients (lse2 / delta stay [B, H, N])
 };
 

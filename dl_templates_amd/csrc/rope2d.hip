@@ -144,6 +144,50 @@ __global__ __launch_bounds__(256) void rope2d_generic_kernel(RopeKArgs a) {
   }
 }
 
+// Out-of-place rotation of a [B, H, N, C] tensor with any strides: dst = rotate(src), every element
+// copied (pass-through dims and unrotated tokens included).  One thread per element; the slow,
+// layout-agnostic companion of the in-place kernels, used when a caller wants the rotated tensor
+// next to the original and the attention kernels cannot produce it themselves.
+struct RopeCopyArgs {
+  const void* src;
+  void* dst;
+  int64_t ss[4], ds[4];
+  int32_t B, H, N, C;
+  RopeDev r;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope2d_copy_kernel(RopeCopyArgs a) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t per_bh = (int64_t)a.N * a.C;
+  const int64_t bh = gid / per_bh;
+  if (bh >= (int64_t)a.B * a.H) return;
+  const int64_t rem = gid - bh * per_bh;
+  const int n = (int)(rem / a.C), d = (int)(rem - (int64_t)n * a.C);
+  const int b = (int)(bh / a.H), h = (int)(bh - (int64_t)b * a.H);
+  const T* ps = reinterpret_cast<const T*>(a.src) + b * a.ss[0] + h * a.ss[1] + n * a.ss[2];
+  T* pd = reinterpret_cast<T*>(a.dst) + b * a.ds[0] + h * a.ds[1] + n * a.ds[2];
+  const T self = ps[d * a.ss[3]];
+  T out = self;
+  if (d < 4 * a.r.R) {
+    const int region = d / a.r.R, i = d - region * a.r.R, ax = region >> 1;
+    const int32_t id = a.r.idx[n];
+    int p = ax == 0 ? dlt_rope_row(id) : dlt_rope_col(id);
+    if (p >= 0) {
+      p = dlt_imin(p, (ax == 0 ? a.r.row_len : a.r.col_len) - 1);
+      const float* tab = (ax == 0 ? a.r.row_cs + (int64_t)p * a.r.rs0 : a.r.col_cs + (int64_t)p * a.r.cs0) + 2 * i;
+      const float c = tab[0];
+      const float s = a.r.inverse ? -tab[1] : tab[1];
+      const bool is_x0 = (region & 1) == 0;
+      const float other = to_f(ps[(is_x0 ? d + a.r.R : d - a.r.R) * a.ss[3]]);
+      float y0, y1;
+      rotate(is_x0 ? to_f(self) : other, is_x0 ? other : to_f(self), c, s, y0, y1);
+      out = from_f<T>(is_x0 ? y0 : y1);
+    }
+  }
+  pd[d * a.ds[3]] = out;
+}
+
 __global__ void rope_pe_mask_kernel(const int32_t* idx, int64_t n_tokens, uint8_t* bits) {
   const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= n_tokens) return;
@@ -210,6 +254,28 @@ int rope_impl(void* const x[2], const int64_t* const st[2], const int64_t nb[2],
 }
 
 }  // namespace
+
+int dlt_rope_rotate_copy(const void* src, const int64_t* ss, void* dst, const int64_t* ds, int B, int H, int64_t N, int C,
+                         const RopeDev& rope, int dtype, hipStream_t stream) {
+  RopeCopyArgs a;
+  a.src = src; a.dst = dst;
+  for (int i = 0; i < 4; i++) { a.ss[i] = ss[i]; a.ds[i] = ds[i]; }
+  a.B = B; a.H = H; a.N = (int32_t)N; a.C = C;
+  a.r = rope;
+  const int64_t total = (int64_t)B * H * N * C;
+  if (total == 0) return DLT_OK;
+  const int64_t gx = (total + 255) / 256;
+  if (gx > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "rope rotate-copy: tensor too large");
+  dlt_timing_before(DLT_K_ROPE, stream);
+  switch (dtype) {
+    case DLT_BF16: hipLaunchKernelGGL(rope2d_copy_kernel<bf16_t>, dim3((unsigned)gx), dim3(256), 0, stream, a); break;
+    case DLT_FP16: hipLaunchKernelGGL(rope2d_copy_kernel<f16_t>, dim3((unsigned)gx), dim3(256), 0, stream, a); break;
+    default: hipLaunchKernelGGL(rope2d_copy_kernel<float>, dim3((unsigned)gx), dim3(256), 0, stream, a); break;
+  }
+  dlt_timing_after(stream);
+  DLT_CHECK_LAUNCH("rope rotate-copy launch");
+  return DLT_OK;
+}
 
 int dlt_validate_rope(const dlt_rope_t* rope, int64_t n_dim) {
   DLT_REQUIRE(rope != nullptr, "rope: descriptor is NULL");

@@ -145,7 +145,9 @@ template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr bool WIDE = ROPE == 0;
+  // ROPE 3: q and k arrive rotated (saved by the forward pass); only the gradients are rotated back on store
+  constexpr int LROT = ROPE == 3 ? 0 : ROPE;  // rotation applied to the tile loads
+  constexpr bool WIDE = LROT == 0;
   constexpr int PA = swa1_pitch(D, NCGMAX, 0, WIDE, true), PB = swa1_pitch(D, NCGMAX, 1, WIDE, true);  // Q rows, dO rows
   constexpr int KC = D / 32, DB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
@@ -176,12 +178,12 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
-  constexpr bool use_rope = ROPE != 0;
-  constexpr bool BAL = ROPE == 2;
+  constexpr bool use_rope = LROT != 0, store_rope = ROPE != 0;
+  constexpr bool BAL = LROT == 2;
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
+  constexpr bool TAIL = LROT == 0 && swa1_use_tail(D, HCW, CR);
   constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
   swa1_plan_init<D, HCW, CR, BAL, TAIL, WIDE, PA, PB>(sp, G, tid, a.rope_pbit);
@@ -209,8 +211,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   for (int d = 0; d < DB; d++) { dk_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; dv_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
   const float scale = a.scale_log2;
 
-  if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
-  swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
+  if (LROT == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
+  swa1_commit<CT, NI, BAL, LROT, TAIL, 0, PA>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
   swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
   swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
@@ -275,9 +277,9 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
     swa1_issue<NI, BAL, TAIL, 0>(srq, sp, on_k, qb, sn2q, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
     swa1_issue<NI, BAL, TAIL, 1>(srd, sp, on_v, dob, sn2d, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
-    if (ROPE == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
+    if (LROT == 2) swa1_tab_issue(tr_srq, srq, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, LROT, TAIL, 0, PA>(srq, sp, sQ, a.rope_pbit, fwd_rope, on_k, &tr_srq, (sp.t_off >> 1) < a.p.dk);
     swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srd, sp, sDO, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     swa1_commit_scalar<HCW, CR>(r_lse, sLse, tid);
     swa1_commit_scalar<HCW, CR>(r_del, sDel, tid);
@@ -290,11 +292,11 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : 
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
   if (a.dk_vec != 0 && a.dv_vec != 0) {  // the loop ended with a workgroup barrier: the chunk buffers are free
     char* sW = smem + wave * 16 * (D * 2 + 16);
-    swa1_store_own<TIO, CT, D>(sW, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.p.dk, G, wave, lane, inv_rope, use_rope);
+    swa1_store_own<TIO, CT, D>(sW, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.p.dk, G, wave, lane, inv_rope, store_rope);
     swa1_store_own<TIO, CT, D>(sW, dv_acc, 1.0f, dvb, a.dvs[2], a.p.dv, G, wave, lane, no_rope, false);
     return;
   }
-  swa1_write_grad<TIO, D>(smem, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.dks[3], a.p.dk, a.dk_vec != 0, L, use_rope ? inv_rope : no_rope, wave, n, g, tid);
+  swa1_write_grad<TIO, D>(smem, dk_acc, a.p.sm_scale, dkb, a.dks[2], a.dks[3], a.p.dk, a.dk_vec != 0, L, store_rope ? inv_rope : no_rope, wave, n, g, tid);
   swa1_write_grad<TIO, D>(smem, dv_acc, 1.0f, dvb, a.dvs[2], a.dvs[3], a.p.dv, a.dv_vec != 0, L, no_rope, wave, n, g, tid);
 }
 
@@ -303,7 +305,9 @@ template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
 __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_q_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr bool WIDE = ROPE == 0;
+  // ROPE 3: q and k arrive rotated (saved by the forward pass); only the gradients are rotated back on store
+  constexpr int LROT = ROPE == 3 ? 0 : ROPE;  // rotation applied to the tile loads
+  constexpr bool WIDE = LROT == 0;
   constexpr int PA = swa1_pitch(D, NCGMAX, 0, WIDE), PB = swa1_pitch(D, NCGMAX, 1, WIDE);  // K rows, V rows
   constexpr int KC = D / 32, DB = D / 16;
   constexpr int HCW = swa1_hcw(NCGMAX);
@@ -330,12 +334,12 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   RopeDev fwd_rope = a.p.rope;  fwd_rope.inverse = 0;
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
-  constexpr bool use_rope = ROPE != 0;
-  constexpr bool BAL = ROPE == 2;
+  constexpr bool use_rope = LROT != 0, store_rope = ROPE != 0;
+  constexpr bool BAL = LROT == 2;
   const int32_t* rope_idx = use_rope ? a.p.rope.idx : nullptr;
   auto own_token = [&](int row) { return L.own_token(row); };
 
-  constexpr bool TAIL = ROPE == 0 && swa1_use_tail(D, HCW, CR);
+  constexpr bool TAIL = LROT == 0 && swa1_use_tail(D, HCW, CR);
   constexpr int NI = swa1_items_t(D, HCW, CR, TAIL);
   StagePlan<NI> sp;
   swa1_plan_init<D, HCW, CR, BAL, TAIL, WIDE, PA, PB>(sp, G, tid, a.rope_pbit);
@@ -386,8 +390,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   for (int d = 0; d < DB; d++) dq_acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const float scale = a.scale_log2;
 
-  if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
-  swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+  if (LROT == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
+  swa1_commit<CT, NI, BAL, LROT, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
   swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   __syncthreads();
   pin_loaded(qf);
@@ -442,9 +446,9 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
     swa1_issue<NI, BAL, TAIL, 0>(srk, sp, on_k, kb_, sn2k, G, CR * ch + CR, rope_idx, (sp.t_off >> 1) < a.p.dk);
     swa1_issue<NI, BAL, TAIL, 1>(srv, sp, on_v, vb_, sn2v, G, CR * ch + CR, nullptr, (sp.t_off >> 1) < a.p.dv);
     consume(ch);
-    if (ROPE == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
+    if (LROT == 2) swa1_tab_issue(tr_srk, srk, sp, fwd_rope);
     __syncthreads();
-    swa1_commit<CT, NI, BAL, ROPE, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
+    swa1_commit<CT, NI, BAL, LROT, TAIL, 0, PA>(srk, sp, sK, a.rope_pbit, fwd_rope, on_k, &tr_srk, (sp.t_off >> 1) < a.p.dk);
     swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srv, sp, sV, 1, no_rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
     __syncthreads();
   }
@@ -454,8 +458,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 4 : 2) : 
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
   if (a.dq_vec != 0) {
     swa1_store_own<TIO, CT, D>(smem + wave * 16 * (D * 2 + 16), dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.p.dk, G, wave, lane,
-                               inv_rope, use_rope);
+                               inv_rope, store_rope);
     return;
   }
-  swa1_write_grad<TIO, D>(smem, dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.dqs[3], a.p.dk, a.dq_vec != 0, L, use_rope ? inv_rope : no_rope, wave, n, g, tid);
+  swa1_write_grad<TIO, D>(smem, dq_acc, a.p.sm_scale, dqb, a.dqs[2], a.dqs[3], a.p.dk, a.dq_vec != 0, L, store_rope ? inv_rope : no_rope, wave, n, g, tid);
 }

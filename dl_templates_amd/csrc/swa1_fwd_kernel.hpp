@@ -25,6 +25,10 @@ struct Swa1FwdArgs {
   void* o;
   float* lse;
   int64_t qs[4], ks[4], vs[4], os[4], ls[3];
+  // optional side outputs of the fused rotation: the rotated q and k (NULL: not stored); rows of
+  // element stride 1, 16-byte aligned
+  void *q_rot, *k_rot;
+  int64_t qrs[4], krs[4];
   int32_t q_vec, o_vec;
   int32_t rope_pbit;  // chunk distance between rotary partners (R / 8), 1 without rotation
   int32_t rope_mode;  // 0 none, 1 rotation with the plain staging map, 2 balanced staging map
@@ -103,6 +107,10 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   // own queries straight into B-operand fragments (rotated on the way when fused)
   u32x4 qf[KC];
   swa1_load_own<TIO, CT, D>(qf, qb, a.qs[2], a.p.dk, tq_own, g, a.p.rope, use_rope);
+  // side outputs of the fused rotation (optional): this workgroup's own queries and keys, rotated
+  const bool save_rot = use_rope && a.k_rot != nullptr;
+  u32x4 kf_own[KC];
+  if (save_rot) swa1_load_own<TIO, CT, D>(kf_own, kb_, a.ks[2], a.p.dk, tq_own, g, a.p.rope, true);
 
   // ---- window of this lane's query in halo coordinates -> additive biases
   const int qr_l = n >> 2, qc_l = n & 3;
@@ -138,6 +146,18 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   swa1_commit<CT, NI, BAL, 0, TAIL, 1, PB>(srv, sp, sV, 1, a.p.rope, false, nullptr, (sp.t_off >> 1) < a.p.dv);
   __syncthreads();
   pin_loaded(qf);
+  if (save_rot && tq_own >= 0) {
+    TIO* qr = reinterpret_cast<TIO*>(a.q_rot) + b * a.qrs[0] + h * a.qrs[1] + tq_own * a.qrs[2];
+    TIO* kr = reinterpret_cast<TIO*>(a.k_rot) + b * a.krs[0] + h * a.krs[1] + tq_own * a.krs[2];
+#pragma unroll
+    for (int c = 0; c < KC; c++) {
+      const int ch = 4 * c + g;
+      if (8 * ch < a.p.dk) {
+        *reinterpret_cast<u32x4*>(qr + 8 * ch) = qf[c];
+        *reinterpret_cast<u32x4*>(kr + 8 * ch) = kf_own[c];
+      }
+    }
+  }
 
   // products and softmax update of the chunk resident in LDS
   auto consume = [&](const int ch) {

@@ -66,7 +66,8 @@ int swa1_launch_bwd_t(const Swa1BwdArgs& a, int grid, int lds_kv, int lds_q, hip
   switch (a.rope_mode) {
     case 0: return swa1_launch_bwd_r<TIO, NCGMAX, 0>(a, grid, lds_kv, lds_q, stream);
     case 1: return swa1_launch_bwd_r<TIO, NCGMAX, 1>(a, grid, lds_kv, lds_q, stream);
-    default: return swa1_launch_bwd_r<TIO, NCGMAX, 2>(a, grid, lds_kv, lds_q, stream);
+    case 2: return swa1_launch_bwd_r<TIO, NCGMAX, 2>(a, grid, lds_kv, lds_q, stream);
+    default: return swa1_launch_bwd_r<TIO, NCGMAX, 3>(a, grid, lds_kv, lds_q, stream);  // rotated inputs, gradients rotated back on store
   }
 }
 }  // namespace

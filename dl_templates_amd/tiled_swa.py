@@ -9,8 +9,8 @@ device, :608-609), the saved log-sum-exp is fp32, and tiles smaller than 16 toke
 backward (the reference raises, :660-661).
 
 ``TiledSwaRope`` is the fused RoPE-2D + attention op: it equals ``RotaryPE2D`` applied to
-q and k followed by ``TiledSwa`` (the composition of README.md:11) without writing the
-rotated q / k to HBM; its backward returns gradients for the un-rotated q and k.
+q and k followed by ``TiledSwa`` (the composition of README.md:11) with the caller's q and k
+left untouched; its backward returns gradients for the un-rotated q and k.
 
 ``TiledSwaImage`` takes q, k, v as images ``[B, IH, IW, heads, D]`` (the layout the reference's
 demo converts from with reshape / permute / reshape, src/tiled_swa.py:753-755) and returns o in
@@ -95,8 +95,50 @@ class TiledSwa(torch.autograd.Function):
         return dq, dk, dv, None, None, None, None, None, None,
 
 
+def _forward_rot(q, k, v, shape, rope):
+    """Forward of the fused op that also returns the rotated q and k (kept for the backward pass)."""
+    _lib.require_cuda(q, k, v)
+    B, H, N, _ = q.shape
+    o = torch.empty((B, H, N, v.shape[-1]), dtype=q.dtype, device=q.device)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+    q_rot = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    k_rot = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    desc, keep = _lib.rope_desc(*rope)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().dlt_swa_fwd_rot(
+            _lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v), _lib.strides(v),
+            _lib.ptr(o), _lib.strides(o), _lib.ptr(lse), _lib.strides(lse),
+            _lib.ptr(q_rot), _lib.strides(q_rot), _lib.ptr(k_rot), _lib.strides(k_rot), shape, desc, _lib.stream_of(q)))
+    del keep
+    return o, lse, q_rot, k_rot
+
+
+def _backward_rot(q_rot, k_rot, v, o, lse, do, shape, rope):
+    _lib.require_cuda(q_rot, k_rot, v, o, lse, do)
+    dq, dk, dv = torch.empty_like(q_rot), torch.empty_like(k_rot), torch.empty_like(v)
+    delta = torch.empty_like(lse)
+    desc, keep = _lib.rope_desc(*rope)
+    with torch.cuda.device(v.device):
+        _lib.check(_lib.load().dlt_swa_bwd_rot(
+            _lib.ptr(q_rot), _lib.strides(q_rot), _lib.ptr(k_rot), _lib.strides(k_rot), _lib.ptr(v), _lib.strides(v),
+            _lib.ptr(o), _lib.strides(o), _lib.ptr(do), _lib.strides(do),
+            _lib.ptr(lse), _lib.ptr(delta), _lib.strides(lse),
+            _lib.ptr(dq), _lib.strides(dq), _lib.ptr(dk), _lib.strides(dk), _lib.ptr(dv), _lib.strides(dv),
+            shape, desc, _lib.stream_of(v)))
+    del keep
+    return dq, dk, dv
+
+
 class TiledSwaRope(torch.autograd.Function):
-    """o = TiledSwa(rope(q), rope(k), v) with the rotation fused into the q / k tile loads."""
+    """o = TiledSwa(rope(q), rope(k), v) with the rotation fused into the q / k tile loads.
+
+    ``save_rotated`` (class attribute, default True): the forward pass also stores the rotated q and k
+    (what ``RotaryPE2D`` leaves in place in the reference's composition) and the backward pass reads
+    those, rotating only dq and dk back as they are stored.  False keeps nothing but the caller's q and k
+    and rotates every staged tile again in the backward kernels: two tensors less memory, slower.
+    """
+
+    save_rotated = True
 
     @staticmethod
     def forward(ctx, q, k, v, idx, row_cs_buffer, col_cs_buffer, b_size, t_height, t_width, row_size, col_size,
@@ -104,8 +146,14 @@ class TiledSwaRope(torch.autograd.Function):
         shape = _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)
         assert row_cs_buffer.shape[1] == col_cs_buffer.shape[1]
         assert idx.shape[0] == q.shape[2]
-        o, m = _forward(q, k, v, shape, (idx, row_cs_buffer, col_cs_buffer))
-        ctx.save_for_backward(q, k, v, m, o, idx, row_cs_buffer, col_cs_buffer)
+        rope = (idx, row_cs_buffer, col_cs_buffer)
+        ctx.rotated = bool(TiledSwaRope.save_rotated)
+        if ctx.rotated:
+            o, m, q_rot, k_rot = _forward_rot(q, k, v, shape, rope)
+            ctx.save_for_backward(q_rot, k_rot, v, m, o, idx, row_cs_buffer, col_cs_buffer)
+        else:
+            o, m = _forward(q, k, v, shape, rope)
+            ctx.save_for_backward(q, k, v, m, o, idx, row_cs_buffer, col_cs_buffer)
         ctx.scalars = (b_size, t_height, t_width, row_size, col_size, sm_scale)
         return o
 
@@ -113,7 +161,11 @@ class TiledSwaRope(torch.autograd.Function):
     def backward(ctx, do):
         q, k, v, m, o, idx, row_cs_buffer, col_cs_buffer = ctx.saved_tensors
         shape = _shape(q, k, v, *ctx.scalars)
-        dq, dk, dv = _backward(q, k, v, o, m, do, shape, (idx, row_cs_buffer, col_cs_buffer))
+        rope = (idx, row_cs_buffer, col_cs_buffer)
+        if ctx.rotated:
+            dq, dk, dv = _backward_rot(q, k, v, o, m, do, shape, rope)
+        else:
+            dq, dk, dv = _backward(q, k, v, o, m, do, shape, rope)
         return (dq, dk, dv) + (None,) * 9
 
 

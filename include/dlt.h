@@ -109,6 +109,32 @@ int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void* k, const 
                 void* dv, const int64_t dv_strides[4],
                 const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream);
 
+/* The fused call with the rotated tensors kept: forward as dlt_swa_fwd with `rope`, which in addition
+ * stores the rotated q and k into q_rot / k_rot (shapes and element type of q / k, own strides; must
+ * not alias q, k or each other).  These are the tensors RotaryPE2D leaves behind in the reference's
+ * composition (it rotates q and k in place and autograd saves the rotated tensors,
+ * src/fused_rope2d.py:143-147).  On token grids the attention kernel itself writes them (each
+ * workgroup its own tokens); otherwise q and k are rotated out of place first and the plain operator
+ * runs on the result. */
+int dlt_swa_fwd_rot(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                    const void* v, const int64_t v_strides[4], void* o, const int64_t o_strides[4],
+                    float* lse2, const int64_t lse_strides[3],
+                    void* q_rot, const int64_t q_rot_strides[4], void* k_rot, const int64_t k_rot_strides[4],
+                    const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream);
+
+/* Backward of the fused call from the saved rotated tensors: q_rot / k_rot are read as they are (no
+ * rotation in the tile loads: every halo token would be rotated again by each workgroup that stages
+ * it); dq and dk get the transposed rotation as they are stored (rope2d_bwd_kernel,
+ * src/fused_rope2d.py:74-122, folded into the epilogue), so they are gradients with respect to the
+ * UN-rotated q and k, exactly as dlt_swa_bwd with `rope` returns them. */
+int dlt_swa_bwd_rot(const void* q_rot, const int64_t q_rot_strides[4], const void* k_rot, const int64_t k_rot_strides[4],
+                    const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],
+                    const void* d_o, const int64_t do_strides[4],
+                    const float* lse2, float* delta, const int64_t lse_strides[3],
+                    void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                    void* dv, const int64_t dv_strides[4],
+                    const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream);
+
 /* Debug export: mask[i * T + j] = 1 iff query tile i attends kv tile j (T = t_height *
  * t_width, row-major tiles), produced on the device by the SAME window routine the
  * attention kernels call (src/tiled_swa.py:76-79, :97-100, :212-214, :701-713). */

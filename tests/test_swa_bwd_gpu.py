@@ -106,9 +106,14 @@ def test_strided_grad_and_inputs():
 
 # (head dim, rotary dims): token-grid kernels with the balanced staging map (64/8, 128/16), with the
 # plain map (64/16: the rotation covers the whole head dim; 128/8: a quarter), generic kernels (4, 3)
+@pytest.mark.parametrize("save_rotated", [True, False])
 @pytest.mark.parametrize("d,R", [(64, 8), (64, 16), (128, 16), (128, 8), (64, 4), (64, 3)])
-def test_fused_rope_backward(d, R):
+def test_fused_rope_backward(d, R, save_rotated, monkeypatch):
+    """save_rotated: the forward pass keeps the rotated q, k and the backward pass reads them, rotating
+    only dq / dk back on store (dlt_swa_fwd_rot / dlt_swa_bwd_rot); otherwise every tile load of the
+    backward kernels rotates again (dlt_swa_fwd / dlt_swa_bwd with rope)."""
     sw = _swa()
+    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save_rotated)
     B, H, th, tw = 1, 2, 16, 16
     N = th * tw
     q, k, v, do = orc.make_qkv(9, B, H, N, N, d, d, torch.bfloat16)
@@ -132,3 +137,58 @@ def test_fused_rope_backward(d, R):
         o2.backward(do.cuda())
         assert torch.equal(o2, o)
         assert torch.equal(q2.grad, qg.grad) and torch.equal(k2.grad, kg.grad) and torch.equal(v2.grad, vg.grad)
+
+
+def test_rotated_side_outputs_and_backward_from_them():
+    """dlt_swa_fwd_rot stores exactly what the standalone rotation produces, leaves q / k alone, accepts
+    strided side outputs, and dlt_swa_bwd_rot from those tensors equals dlt_swa_bwd from the originals."""
+    from dl_templates_amd import fused_rope2d as fr
+    sw = _swa()
+    for (B, H, th, tw, S, d, R, W) in [(2, 2, 12, 20, 1, 64, 8, 3),      # token grid: the attention kernel writes q_rot / k_rot
+                                       (1, 2, 9, 7, 1, 128, 16, 2),      # odd grid, partial workgroups
+                                       (1, 2, 4, 5, 16, 64, 8, 1),       # 16-token tiles: rotate-copy, then tile mode
+                                       (1, 1, 6, 6, 4, 64, 6, 1)]:       # 4-token tiles, R not a multiple of 8
+        N = th * tw * S
+        q, k, v, do = orc.make_qkv(21 + S, B, H, N, N, d, d, torch.bfloat16)
+        idx = torch.cat([orc.make_rope_idx(3, th, tw, 0.1)] * S).reshape(S, -1).t().reshape(-1).contiguous()
+        rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+        rope = (idx.cuda(), rcs.cuda(), ccs.cuda())
+        o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, S, th, tw, W, W, 0.125)
+        qg, kg, vg, dog = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+        shape = sw._shape(qg, kg, vg, S, th, tw, W, W, 0.125)
+        o, lse, q_rot, k_rot = sw._forward_rot(qg, kg, vg, shape, rope)
+        assert torch.equal(qg.cpu(), q) and torch.equal(kg.cpu(), k)
+        q2, k2 = fr.rope2d_qk_(q.cuda().clone(), k.cuda().clone(), *rope)
+        assert torch.equal(q_rot, q2) and torch.equal(k_rot, k2)
+        assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
+        dq, dk, dv = sw._backward_rot(q_rot, k_rot, vg, o, lse, dog, shape, rope)
+        errs = (_rel(dq, dq_w), _rel(dk, dk_w), _rel(dv, dv_w))
+        assert max(errs) <= GRAD_TOL, errs
+        o1, lse1 = sw._forward(qg, kg, vg, shape, rope)
+        dq1, dk1, dv1 = sw._backward(qg, kg, vg, o1, lse1, dog, shape, rope)
+        assert (o1.float() - o.float()).abs().max().item() <= 1e-2
+        for a, b_ in ((dq, dq1), (dk, dk1), (dv, dv1)):
+            assert (a.float() - b_.float()).abs().max().item() <= 2e-2 * max(1.0, b_.float().abs().max().item())
+
+
+def test_rotated_side_outputs_reject_aliasing():
+    from dl_templates_amd import _lib
+    sw = _swa()
+    B, H, th, tw, d = 1, 1, 8, 8, 64
+    q = torch.zeros((B, H, th * tw, d), dtype=torch.bfloat16, device="cuda")
+    k, v, o, qr = (torch.zeros_like(q) for _ in range(4))
+    lse = torch.zeros((B, H, th * tw), dtype=torch.float32, device="cuda")
+    idx = orc.encode_idx(th, tw).cuda()
+    tabs = orc.rope_tables(8, 8).cuda()
+    desc, keep = _lib.rope_desc(idx, tabs, tabs)
+    shape = sw._shape(q, k, v, 1, th, tw, 1, 1, 1.0)
+    lib = _lib.load()
+    args = lambda qrot, krot: (_lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v), _lib.strides(v),
+                               _lib.ptr(o), _lib.strides(o), _lib.ptr(lse), _lib.strides(lse), _lib.ptr(qrot),
+                               _lib.strides(qrot), _lib.ptr(krot), _lib.strides(krot), shape, desc, _lib.stream_of(q))
+    assert lib.dlt_swa_fwd_rot(*args(q, qr)) == 1 and b"alias" in lib.dlt_last_error()
+    assert lib.dlt_swa_fwd_rot(*args(qr, qr)) == 1 and b"alias" in lib.dlt_last_error()
+    a = list(args(qr, o))
+    a[-2] = None
+    assert lib.dlt_swa_fwd_rot(*a) == 1 and b"rope is NULL" in lib.dlt_last_error()
+    del keep
