@@ -144,12 +144,14 @@ def test_rotated_side_outputs_and_backward_from_them():
     strided side outputs, and dlt_swa_bwd_rot from those tensors equals dlt_swa_bwd from the originals."""
     from dl_templates_amd import fused_rope2d as fr
     sw = _swa()
-    for (B, H, th, tw, S, d, R, W) in [(2, 2, 12, 20, 1, 64, 8, 3),      # token grid: the attention kernel writes q_rot / k_rot
-                                       (1, 2, 9, 7, 1, 128, 16, 2),      # odd grid, partial workgroups
-                                       (1, 2, 4, 5, 16, 64, 8, 1),       # 16-token tiles: rotate-copy, then tile mode
-                                       (1, 1, 6, 6, 4, 64, 6, 1)]:       # 4-token tiles, R not a multiple of 8
+    bf16, f16, f32 = torch.bfloat16, torch.float16, torch.float32
+    for (B, H, th, tw, S, d, R, W, dt) in [(2, 2, 12, 20, 1, 64, 8, 3, bf16),    # token grid: the attention kernel writes q_rot / k_rot
+                                           (1, 2, 9, 7, 1, 128, 16, 2, f16),     # odd grid, partial workgroups
+                                           (1, 2, 4, 5, 16, 64, 8, 1, bf16),     # 16-token tiles: rotate-copy, then tile mode
+                                           (1, 1, 6, 6, 4, 64, 6, 1, bf16),      # 4-token tiles, R not a multiple of 8
+                                           (1, 2, 8, 8, 1, 32, 8, 2, f32)]:      # fp32 tensors: rotate-copy, generic kernels
         N = th * tw * S
-        q, k, v, do = orc.make_qkv(21 + S, B, H, N, N, d, d, torch.bfloat16)
+        q, k, v, do = orc.make_qkv(21 + S, B, H, N, N, d, d, dt)
         idx = torch.cat([orc.make_rope_idx(3, th, tw, 0.1)] * S).reshape(S, -1).t().reshape(-1).contiguous()
         rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
         rope = (idx.cuda(), rcs.cuda(), ccs.cuda())
