@@ -120,3 +120,32 @@ def test_image_entry_rejects_bad_arguments():
                                _lib.ptr(q), _lib.strides(q), _lib.ptr(lse), _lib.strides(lse), shape, tile, None,
                                _lib.stream_of(q))
     assert rc == 1 and b"negative stride" in lib.dlt_last_error()
+
+
+def test_image_layout_with_fused_rotation():
+    """The rotary operands stay indexed by the tile-major token number when the tensors are images."""
+    from dl_templates_amd import _lib
+    sw = _swa()
+    B, H, th, tw, bh, bw, d, R = 1, 2, 5, 6, 2, 2, 64, 8
+    S, N = bh * bw, th * tw * bh * bw
+    q, k, v, do = orc.make_qkv(41, B, H, N, N, d, d, torch.bfloat16)
+    idx = torch.cat([orc.make_rope_idx(4, th, tw, 0.1)] * S).reshape(S, -1).t().reshape(-1).contiguous()
+    rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+    o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, S, th, tw, 1, 1, 0.125)
+    to_img = lambda t: orc.tokens_to_image(t, th, tw, bh, bw).contiguous()
+    qi, ki, vi, doi = (to_img(t).cuda() for t in (q, k, v, do))
+    shape, tile = sw._image_shape(qi, ki, vi, bh, bw, 1, 1, 0.125)
+    desc, keep = _lib.rope_desc(idx.cuda(), rcs.cuda(), ccs.cuda())
+    o = torch.empty_like(vi)
+    lse = torch.empty((B, H, N), dtype=torch.float32, device="cuda")
+    lib, P, S_ = _lib.load(), _lib.ptr, _lib.strides
+    _lib.check(lib.dlt_swa_fwd_image(P(qi), S_(qi), P(ki), S_(ki), P(vi), S_(vi), P(o), S_(o), P(lse), S_(lse), shape, tile,
+                                     desc, _lib.stream_of(qi)))
+    assert (o.float().cpu() - to_img(o_w)).abs().max().item() <= FWD_TOL
+    dq, dk, dv, delta = torch.empty_like(qi), torch.empty_like(ki), torch.empty_like(vi), torch.empty_like(lse)
+    _lib.check(lib.dlt_swa_bwd_image(P(qi), S_(qi), P(ki), S_(ki), P(vi), S_(vi), P(o), S_(o), P(doi), S_(doi),
+                                     P(lse), P(delta), S_(lse), P(dq), S_(dq), P(dk), S_(dk), P(dv), S_(dv), shape, tile,
+                                     desc, _lib.stream_of(qi)))
+    errs = (_rel(dq, to_img(dq_w)), _rel(dk, to_img(dk_w)), _rel(dv, to_img(dv_w)))
+    assert max(errs) <= GRAD_TOL, errs
+    del keep
