@@ -316,7 +316,8 @@ def calibration_copy():
 
 def copy_bandwidth():
     """What the memory system sustains for a plain copy (read + write bytes per second): 64 MiB
-    (resident in the 256 MB infinity cache after the first pass) and 1 GiB (HBM)."""
+    (resident in the 256 MB infinity cache after the first pass), 1 GiB (HBM), and 24 MiB copies from
+    cold buffers (a launch of the size of the RoPE benchmark)."""
     from dl_templates_amd import _lib
     lib = _lib.load()
     out = {}
@@ -328,6 +329,20 @@ def copy_bandwidth():
         ms, _ = Timer.run(fn, reps, 2)
         out[name] = {"ms": ms, "gbps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9}
         del a, b
+    # a copy with the real traffic of one RoPE C2 launch (about 48 MiB), cold: 13 buffer pairs cycled (624 MiB)
+    nbytes, npairs = 24 << 20, 13
+    bufs = [(torch.empty(nbytes, dtype=torch.uint8, device="cuda:0"), torch.empty(nbytes, dtype=torch.uint8, device="cuda:0"))
+            for _ in range(npairs)]
+    st = _lib.stream_of(bufs[0][0])
+    state = {"i": 0}
+
+    def cold():
+        a, b = bufs[state["i"] % npairs]
+        state["i"] += 1
+        _lib.check(lib.dlt_debug_copy(_lib.ptr(b), _lib.ptr(a), nbytes, st))
+
+    ms, _ = Timer.run(cold, 5 * npairs, npairs)
+    out["24MiB_cold"] = {"ms": ms, "gbps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9}
     return out
 
 
