@@ -89,8 +89,12 @@ def test_c4_band_against_cpu_oracle():
     assert rel(vg.grad.float().cpu()[:, :, inner2], dv_w[:, :, inner2_b]) <= 5e-2
 
 
-def test_c3_full_batch_fused_rope_equals_composition():
+@pytest.mark.parametrize("save_rotated", [True, False])
+def test_c3_full_batch_fused_rope_equals_composition(save_rotated, monkeypatch):
+    """Both fused variants (rotated q, k kept for the backward pass / rotated again in every tile load) at the
+    full size of config 3, bit-equal to the composition of the standalone rotation and the plain operator."""
     sw, _, fr = _mods()
+    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save_rotated)
     B, H, th, tw, d, W = 2, 8, 64, 64, 64, 6
     N = th * tw
     q, k, v, do = (t.cuda() for t in orc.make_qkv(3, B, H, N, N, d, d, torch.bfloat16))
