@@ -261,7 +261,7 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
   a.tile = p.g.mode == DLT_GEOM_SWA;
   a.g = p.g;
   a.o_vec = tvec_ok(t.out_o, t.os, p.dv, 2);
-  const int chunk = FLASH_CK * (dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD), tile = own * (dc.DV * 2 + 16);
+  const int chunk = flash_ck_fwd(dc.DK, dc.DV) * (dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD), tile = own * (dc.DV * 2 + 16);
   a.lds_bytes = chunk > tile ? chunk : tile;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   const int64_t grid = (int64_t)p.B * p.H * p.g.TR * a.nblk;
@@ -312,11 +312,12 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   a.dq_vec = tvec_ok(t.dq, t.dqs, p.dk, 2);
   a.dk_vec = tvec_ok(t.dk, t.dks, p.dk, 2);
   a.dv_vec = tvec_ok(t.dv, t.dvs, p.dv, 2);
-  const int chunk = FLASH_CK * (dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD);
+  const int row = dc.DK * 2 + FLASH_PAD + dc.DV * 2 + FLASH_PAD;   // one streamed token in both LDS regions
+  const int chunk_q = flash_ck_q(dc.DK, dc.DV) * row, ck_kv = flash_ck_kv(dc.DK, dc.DV);
   const int tile_q = own * (dc.DK * 2 + 16);
   const int tile_k = own_kv * (dc.DK * 2 + 16), tile_v = own_kv * (dc.DV * 2 + 16);
-  a.lds_q = chunk > tile_q ? chunk : tile_q;
-  a.lds_kv = chunk + 2 * FLASH_CK * 4;
+  a.lds_q = chunk_q > tile_q ? chunk_q : tile_q;
+  a.lds_kv = ck_kv * row + 2 * ck_kv * 4;
   if (tile_k > a.lds_kv) a.lds_kv = tile_k;
   if (tile_v > a.lds_kv) a.lds_kv = tile_v;
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;

@@ -8,7 +8,7 @@
 namespace {
 template <typename TIO, int MODE>
 int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
-  auto kern = flash_fwd_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, FLASH_CK, MODE>;
+  auto kern = flash_fwd_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, flash_ck_fwd(DLT_DK, DLT_DV), MODE>;
   if (a.lds_bytes > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, a.lds_bytes);
     if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", a.lds_bytes, hipGetErrorString(e));
@@ -39,7 +39,7 @@ template <typename TIO, int MODE>
 int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
   // dQ first: with fuse_delta it produces the delta vector the dK/dV kernel consumes
   {
-    auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, flash_np_q(DLT_DK, DLT_DV), FLASH_CK, MODE>;
+    auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, flash_np_q(DLT_DK, DLT_DV), flash_ck_q(DLT_DK, DLT_DV), MODE>;
     int rc = flash_set_lds(kern, a.lds_q);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_Q, stream);
@@ -48,7 +48,7 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
     DLT_CHECK_LAUNCH("flash dQ launch");
   }
   {
-    auto kern = flash_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, flash_np_kv(DLT_DK, DLT_DV), FLASH_CK, MODE>;
+    auto kern = flash_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, flash_np_kv(DLT_DK, DLT_DV), flash_ck_kv(DLT_DK, DLT_DV), MODE>;
     int rc = flash_set_lds(kern, a.lds_kv);
     if (rc != DLT_OK) return rc;
     dlt_timing_before(DLT_K_BWD_KV, stream);

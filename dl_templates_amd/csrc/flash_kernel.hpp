@@ -40,11 +40,23 @@ DLT_DEV int flash_stage_tid(int tid) {
 #ifndef FLASH_NP_DEF
 #define FLASH_NP_DEF 2
 #endif
-#ifndef FLASH_CK_DEF
-#define FLASH_CK_DEF 64
-#endif
 constexpr int FLASH_NP = FLASH_NP_DEF;  // 16-query blocks per wave (forward and dQ)
-constexpr int FLASH_CK = FLASH_CK_DEF;  // streamed tokens per LDS chunk
+// Streamed tokens per LDS chunk, per kernel and head-dim class.  128 halves the barriers per key but
+// doubles the staging registers and the score registers of a chunk: it pays where the register
+// allocation still fits the occupancy target below (measured per class: forward at 64/128 -4 %, dQ at
+// 32/32 -8 % in tile mode, dK/dV at 128/128 -8 % in tile mode; elsewhere it spills or changes nothing).
+#ifndef FLASH_CK_FWD
+#define FLASH_CK_FWD(dk, dv) ((dk) == 64 && (dv) == 128 ? 128 : 64)
+#endif
+#ifndef FLASH_CK_Q
+#define FLASH_CK_Q(dk, dv) ((dk) + (dv) <= 64 ? 128 : 64)
+#endif
+#ifndef FLASH_CK_KV
+#define FLASH_CK_KV(dk, dv) ((dk) + (dv) > 192 ? 128 : 64)
+#endif
+constexpr int flash_ck_fwd(int dk, int dv) { return FLASH_CK_FWD(dk, dv); }
+constexpr int flash_ck_q(int dk, int dv) { return FLASH_CK_Q(dk, dv); }
+constexpr int flash_ck_kv(int dk, int dv) { return FLASH_CK_KV(dk, dv); }
 // key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
 constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 128 ? 1 : 2; }
 // query blocks per wave in the dQ kernel: one at 128/128 (accumulators, q and dO fragments of two blocks do not fit 256 registers)
