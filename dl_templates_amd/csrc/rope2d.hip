@@ -188,6 +188,43 @@ __global__ __launch_bounds__(256) void rope2d_copy_kernel(RopeCopyArgs a) {
   pd[d * a.ds[3]] = out;
 }
 
+// The same for rows of element stride 1 whose 8-element chunks are 16-byte (32-byte for fp32) aligned and
+// R % 8 == 0: one thread per chunk, the partner chunk is read a second time (from L1).
+template <typename T>
+__global__ __launch_bounds__(256) void rope2d_copy_vec_kernel(RopeCopyArgs a) {
+  const int nch = a.C >> 3;
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t per_bh = (int64_t)a.N * nch;
+  const int64_t bh = gid / per_bh;
+  if (bh >= (int64_t)a.B * a.H) return;
+  const int64_t rem = gid - bh * per_bh;
+  const int n = (int)(rem / nch), c = (int)(rem - (int64_t)n * nch);
+  const int b = (int)(bh / a.H), h = (int)(bh - (int64_t)b * a.H);
+  const T* ps = reinterpret_cast<const T*>(a.src) + b * a.ss[0] + h * a.ss[1] + n * a.ss[2];
+  T* pd = reinterpret_cast<T*>(a.dst) + b * a.ds[0] + h * a.ds[1] + n * a.ds[2];
+  Vec8<T> self = *reinterpret_cast<const Vec8<T>*>(ps + 8 * c);
+  const int r8 = a.r.R >> 3;
+  if (c < 4 * r8) {
+    const int region = c / r8, ci = c - region * r8, ax = region >> 1;
+    const bool is_x0 = (region & 1) == 0;
+    const Vec8<T> other = *reinterpret_cast<const Vec8<T>*>(ps + 8 * (is_x0 ? c + r8 : c - r8));
+    const int32_t id = a.r.idx[n];
+    int p = ax == 0 ? dlt_rope_row(id) : dlt_rope_col(id);
+    if (p >= 0) {
+      p = dlt_imin(p, (ax == 0 ? a.r.row_len : a.r.col_len) - 1);
+      const float* tab = (ax == 0 ? a.r.row_cs + (int64_t)p * a.r.rs0 : a.r.col_cs + (int64_t)p * a.r.cs0) + 16 * ci;
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        const float cs = tab[2 * j], sn = a.r.inverse ? -tab[2 * j + 1] : tab[2 * j + 1];
+        float y0, y1;
+        rotate(is_x0 ? to_f(self.v[j]) : to_f(other.v[j]), is_x0 ? to_f(other.v[j]) : to_f(self.v[j]), cs, sn, y0, y1);
+        self.v[j] = from_f<T>(is_x0 ? y0 : y1);
+      }
+    }
+  }
+  *reinterpret_cast<Vec8<T>*>(pd + 8 * c) = self;
+}
+
 __global__ void rope_pe_mask_kernel(const int32_t* idx, int64_t n_tokens, uint8_t* bits) {
   const int64_t n = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (n >= n_tokens) return;
@@ -262,15 +299,27 @@ int dlt_rope_rotate_copy(const void* src, const int64_t* ss, void* dst, const in
   for (int i = 0; i < 4; i++) { a.ss[i] = ss[i]; a.ds[i] = ds[i]; }
   a.B = B; a.H = H; a.N = (int32_t)N; a.C = C;
   a.r = rope;
-  const int64_t total = (int64_t)B * H * N * C;
+  const int es = dlt_elem_size(dtype), vb = 8 * es;
+  bool vec = C % 8 == 0 && rope.R % 8 == 0 && ss[3] == 1 && ds[3] == 1 && (uintptr_t)src % vb == 0 && (uintptr_t)dst % vb == 0;
+  for (int i = 0; i < 3; i++) vec = vec && (ss[i] * es) % vb == 0 && (ds[i] * es) % vb == 0;
+  const int64_t total = (int64_t)B * H * N * (vec ? C / 8 : C);
   if (total == 0) return DLT_OK;
   const int64_t gx = (total + 255) / 256;
   if (gx > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "rope rotate-copy: tensor too large");
   dlt_timing_before(DLT_K_ROPE, stream);
-  switch (dtype) {
-    case DLT_BF16: hipLaunchKernelGGL(rope2d_copy_kernel<bf16_t>, dim3((unsigned)gx), dim3(256), 0, stream, a); break;
-    case DLT_FP16: hipLaunchKernelGGL(rope2d_copy_kernel<f16_t>, dim3((unsigned)gx), dim3(256), 0, stream, a); break;
-    default: hipLaunchKernelGGL(rope2d_copy_kernel<float>, dim3((unsigned)gx), dim3(256), 0, stream, a); break;
+  const dim3 grid((unsigned)gx), block(256);
+  if (vec) {
+    switch (dtype) {
+      case DLT_BF16: hipLaunchKernelGGL(rope2d_copy_vec_kernel<bf16_t>, grid, block, 0, stream, a); break;
+      case DLT_FP16: hipLaunchKernelGGL(rope2d_copy_vec_kernel<f16_t>, grid, block, 0, stream, a); break;
+      default: hipLaunchKernelGGL(rope2d_copy_vec_kernel<float>, grid, block, 0, stream, a); break;
+    }
+  } else {
+    switch (dtype) {
+      case DLT_BF16: hipLaunchKernelGGL(rope2d_copy_kernel<bf16_t>, grid, block, 0, stream, a); break;
+      case DLT_FP16: hipLaunchKernelGGL(rope2d_copy_kernel<f16_t>, grid, block, 0, stream, a); break;
+      default: hipLaunchKernelGGL(rope2d_copy_kernel<float>, grid, block, 0, stream, a); break;
+    }
   }
   dlt_timing_after(stream);
   DLT_CHECK_LAUNCH("rope rotate-copy launch");
