@@ -404,6 +404,22 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
     Swa1Class c;
     if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(t)) return swa1_backward(p, t, c, stream);
   }
+  if (p.rope_prerot && p.rope.enabled && p.rope.R > 0 && !p.tm.img) {
+    // rotated q, k and no token-grid kernel: the plain operator (any kernel family) yields the gradients of the
+    // rotated tensors; the standalone rotation turns them back in place
+    AttnProblem p2 = p;
+    p2.rope = dlt_make_rope_dev(nullptr, 0);
+    p2.rope_prerot = 0;
+    rc = dlt_attn_backward(p2, t, stream);
+    if (rc != DLT_OK) return rc;
+    dlt_rope_t r;
+    r.idx = p.rope.idx; r.row_cs = p.rope.row_cs; r.col_cs = p.rope.col_cs;
+    r.row_cs_stride0 = p.rope.rs0; r.col_cs_stride0 = p.rope.cs0;
+    r.n_rdim = p.rope.R; r.row_len = p.rope.row_len; r.col_len = p.rope.col_len;
+    rc = dlt_rope_inplace_4d(t.dq, t.dqs, p.B, p.H, (int64_t)p.g.TR * p.g.XLq, p.dk, &r, 1, p.dtype, stream);
+    if (rc != DLT_OK) return rc;
+    return dlt_rope_inplace_4d(t.dk, t.dks, p.B, p.H, (int64_t)p.g.TR * p.g.XLk, p.dk, &r, 1, p.dtype, stream);
+  }
   if (flash_eligible(p, t, true)) return flash_backward(p, t, dc, stream);
   const int np = 1;
   const int own = 64 * np;

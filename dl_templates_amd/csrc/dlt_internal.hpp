@@ -42,6 +42,9 @@ struct RopeDev {
 
 int dlt_validate_rope(const dlt_rope_t* rope, int64_t n_dim);
 RopeDev dlt_make_rope_dev(const dlt_rope_t* rope, int inverse);
+// in-place rotation of a [B, H, N, C] tensor with any strides (the standalone kernels)
+int dlt_rope_inplace_4d(void* x, const int64_t* st, int B, int H, int64_t N, int C, const dlt_rope_t* rope, int inverse,
+                        int dtype, hipStream_t stream);
 // dst = rotate(src) for [B, H, N, C] tensors with any strides (every element is copied)
 int dlt_rope_rotate_copy(const void* src, const int64_t* ss, void* dst, const int64_t* ds, int B, int H, int64_t N, int C,
                          const RopeDev& rope, int dtype, hipStream_t stream);

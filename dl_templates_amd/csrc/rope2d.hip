@@ -326,6 +326,23 @@ int dlt_rope_rotate_copy(const void* src, const int64_t* ss, void* dst, const in
   return DLT_OK;
 }
 
+// In-place rotation of a [B, H, N, C] tensor with any strides through the standalone kernels: one launch
+// when (B, H) collapses into one batch stride, else one per b.
+int dlt_rope_inplace_4d(void* x, const int64_t* st, int B, int H, int64_t N, int C, const dlt_rope_t* rope, int inverse,
+                        int dtype, hipStream_t stream) {
+  const bool flat = B == 1 || st[0] == (int64_t)H * st[1];
+  const int64_t s3[3] = {st[1], st[2], st[3]};
+  const int es = dlt_elem_size(dtype);
+  for (int b = 0; b < (flat ? 1 : B); b++) {
+    void* const xs[2] = {static_cast<char*>(x) + (int64_t)b * st[0] * es, nullptr};
+    const int64_t* const sts[2] = {s3, nullptr};
+    const int64_t nb[2] = {flat ? (int64_t)B * H : H, 0};
+    int rc = rope_impl(xs, sts, nb, 1, N, C, rope, inverse, dtype, stream);
+    if (rc != DLT_OK) return rc;
+  }
+  return DLT_OK;
+}
+
 int dlt_validate_rope(const dlt_rope_t* rope, int64_t n_dim) {
   DLT_REQUIRE(rope != nullptr, "rope: descriptor is NULL");
   DLT_REQUIRE(rope->n_rdim >= 0, "rope: n_rdim %d < 0", rope->n_rdim);
