@@ -236,9 +236,23 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
     for (int kb = 0; kb < NKB; kb++) {
       if (on[kb]) {
         const int key0 = 4 * wave + 4 * (CR == 8 ? kb : 2 * kb);
+        if (D > 64) {
+          // two waves per SIMD: V^T fragments are requested four at a time ahead of their products, so that
+          // one LDS latency is paid per group instead of one per product
 #pragma unroll
-        for (int d = 0; d < VB; d++)
-          acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PB, HCW, key0, 16 * d, n, g, MB_STEP), pb[kb], acc[d]);
+          for (int d0 = 0; d0 < VB; d0 += 4) {
+            u32x4 vfr[4];
+#pragma unroll
+            for (int d = 0; d < 4; d++) vfr[d] = swa1_read_tokens_as_k(sV, PB, HCW, key0, 16 * (d0 + d), n, g, MB_STEP);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int d = 0; d < 4; d++) acc[d0 + d] = Mma<CT>::mfma(vfr[d], pb[kb], acc[d0 + d]);
+          }
+        } else {
+#pragma unroll
+          for (int d = 0; d < VB; d++)
+            acc[d] = Mma<CT>::mfma(swa1_read_tokens_as_k(sV, PB, HCW, key0, 16 * d, n, g, MB_STEP), pb[kb], acc[d]);
+        }
         if (ONES) acc_l = Mma<CT>::mfma(ones, pb[kb], acc_l);
       }
     }
