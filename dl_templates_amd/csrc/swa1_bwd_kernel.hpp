@@ -142,7 +142,11 @@ DLT_DEV void swa1_write_grad(char* sT, f32x4 (&acc)[D / 16], float mul, TIO* bas
 
 // =============================================================================================
 template <typename TIO, int D, int NCGMAX, int CR, int ROPE>
-__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
+// Occupancy target of the variants with rotation: one below what the kernel reaches (its register count
+// still admits three workgroups per CU).  With a target of three the compiler, a few registers over its
+// budget, reschedules the whole kernel for minimum register pressure and the product loop loses its
+// read-ahead (LDS reads issued one or two ahead of their MFMA instead of a dozen).
+__global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 && NCGMAX <= 4 && ROPE == 0 ? 3 : 2) : (CR == 4 ? 2 : 1))) void swa1_bwd_kv_kernel(const Swa1BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
   // ROPE 3: q and k arrive rotated (saved by the forward pass); only the gradients are rotated back on store
