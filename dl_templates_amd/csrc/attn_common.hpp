@@ -201,7 +201,9 @@ DLT_DEV RopeChunk rope_chunk_setup(const RopeDev& r, int c, bool vec) {
   if (!r.enabled || r.R == 0 || 8 * c >= 4 * r.R) return rc;
   if (vec && (r.R & 7) == 0) {
     const int r8 = r.R >> 3;
-    const int region = c / r8, ci = c - region * r8;
+    // r8 is wave-uniform; the usual sizes are powers of two, where a shift replaces the per-lane division
+    const int region = (r8 & (r8 - 1)) == 0 ? c >> __builtin_ctz(r8) : c / r8;
+    const int ci = c - region * r8;
     rc.mode = 1;
     rc.axis = region >> 1;
     rc.is_x0 = (region & 1) == 0;
