@@ -186,6 +186,17 @@ DLT_DEV float rope_mix(float self, float partner, float c, float s, bool is_x0) 
   return is_x0 ? a - b : b + a;
 }
 
+// The same value with the sign of the sine decided once per chunk instead of once per element:
+// a - b == a + (-b) and b + a == a + b bit for bit, and (-s) * x == -(s * x), so
+// rope_mix(self, partner, c, s, is_x0) == rope_mix_signed(self, partner, c, is_x0 ? -s : s).
+DLT_DEV unsigned rope_sign_mask(bool is_x0, bool inverse) { return is_x0 != inverse ? 0x80000000u : 0u; }
+DLT_DEV float rope_mix_signed(float self, float partner, float c, float s_raw, unsigned sign_mask) {
+#pragma clang fp contract(off)
+  const float s = __uint_as_float(__float_as_uint(s_raw) ^ sign_mask);
+  const float a = self * c, b = partner * s;
+  return a + b;
+}
+
 // Per-thread rotary context for a fixed 8-dim chunk index `c` (dims 8c .. 8c+7).
 struct RopeChunk {
   int mode;      // 0: chunk not rotated, 1: whole-chunk fast path (R % 8 == 0), 2: per-element path
@@ -231,11 +242,9 @@ DLT_DEV void rope_apply8(const RopeDev& r, const RopeChunk& rc, int c, int32_t i
     bool rotated;
     const float* tab = rope_table_row(r, rc.axis, id, rotated) + rc.tab_off;
     if (!rotated) return;
+    const unsigned sm = rope_sign_mask(rc.is_x0 != 0, r.inverse != 0);
 #pragma unroll
-    for (int j = 0; j < 8; j++) {
-      const float cs = tab[2 * j], sn = r.inverse ? -tab[2 * j + 1] : tab[2 * j + 1];
-      self[j] = rope_mix(self[j], partner8[j], cs, sn, rc.is_x0);
-    }
+    for (int j = 0; j < 8; j++) self[j] = rope_mix_signed(self[j], partner8[j], tab[2 * j], tab[2 * j + 1], sm);
   } else if (rc.mode == 2) {
 #pragma unroll
     for (int j = 0; j < 8; j++) {

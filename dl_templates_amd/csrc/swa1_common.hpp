@@ -395,7 +395,7 @@ DLT_DEV void swa1_store_own(char* sW, const f32x4 (&acc)[D / 16], float mul, TIO
 #pragma unroll
         for (int j = 0; j < 8; j++) {
           const float cs = tv[it][j >> 1][2 * (j & 1)], sn_ = tv[it][j >> 1][2 * (j & 1) + 1];
-          self[j] = rope_mix(self[j], partner[j], cs, rope.inverse ? -sn_ : sn_, rc[it].is_x0);
+          self[j] = rope_mix_signed(self[j], partner[j], cs, sn_, rope_sign_mask(rc[it].is_x0 != 0, rope.inverse != 0));
         }
         v = pack8<CT>(self);
       }
