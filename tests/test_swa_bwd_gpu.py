@@ -194,3 +194,35 @@ def test_rotated_side_outputs_reject_aliasing():
     a[-2] = None
     assert lib.dlt_swa_fwd_rot(*a) == 1 and b"rope is NULL" in lib.dlt_last_error()
     del keep
+
+
+def test_rotated_side_outputs_with_awkward_strides():
+    """q_rot / k_rot that are not 16-byte-vector rows (a transposed buffer) or padded rows: the forward pass falls
+    back to the out-of-place rotation, the backward pass to the plain operator plus the standalone rotation."""
+    from dl_templates_amd import _lib, fused_rope2d as fr
+    sw = _swa()
+    B, H, th, tw, d, R, W = 1, 2, 10, 12, 64, 8, 2
+    N = th * tw
+    q, k, v, do = orc.make_qkv(77, B, H, N, N, d, d, torch.bfloat16)
+    idx = orc.make_rope_idx(5, th, tw, 0.1)
+    rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+    rope = (idx.cuda(), rcs.cuda(), ccs.cuda())
+    o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, W, W, 0.125)
+    qg, kg, vg, dog = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    shape = sw._shape(qg, kg, vg, 1, th, tw, W, W, 0.125)
+    desc, keep = _lib.rope_desc(*rope)
+    q2, k2 = fr.rope2d_qk_(q.cuda().clone(), k.cuda().clone(), *rope)
+    lib, P, S_ = _lib.load(), _lib.ptr, _lib.strides
+    for make in (lambda: torch.empty((B, H, d, N), dtype=torch.bfloat16, device="cuda").transpose(2, 3),      # element stride N
+                 lambda: torch.empty((B, H, N, d + 8), dtype=torch.bfloat16, device="cuda")[..., :d]):       # padded rows
+        q_rot, k_rot = make(), make()
+        o = torch.empty_like(vg)
+        lse = torch.empty((B, H, N), dtype=torch.float32, device="cuda")
+        _lib.check(lib.dlt_swa_fwd_rot(P(qg), S_(qg), P(kg), S_(kg), P(vg), S_(vg), P(o), S_(o), P(lse), S_(lse),
+                                       P(q_rot), S_(q_rot), P(k_rot), S_(k_rot), shape, desc, _lib.stream_of(qg)))
+        assert torch.equal(q_rot, q2) and torch.equal(k_rot, k2)
+        assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
+        dq, dk, dv = sw._backward_rot(q_rot, k_rot, vg, o, lse, dog, shape, rope)
+        errs = (_rel(dq, dq_w), _rel(dk, dk_w), _rel(dv, dv_w))
+        assert max(errs) <= GRAD_TOL, errs
+    del keep
