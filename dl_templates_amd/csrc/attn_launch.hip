@@ -340,12 +340,13 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
   if (rc != DLT_OK) return rc;
   const int es = dlt_elem_size(p.dtype);
   {
-    const bool streamed[2] = {tvec_ok(t.k, t.ks, p.dk, es), tvec_ok(t.v, t.vs, p.dv, es)};
+    // q is not streamed, but its own-token fragments are read as 16-byte pieces too
+    const bool streamed[3] = {tvec_ok(t.q, t.qs, p.dk, es), tvec_ok(t.k, t.ks, p.dk, es), tvec_ok(t.v, t.vs, p.dv, es)};
     Swa1Class c;
-    if (swa1_eligible(p, streamed, 2, c) && swa1_strides_fit(t)) {
+    if (swa1_eligible(p, streamed, 3, c) && swa1_strides_fit(t)) {
       // rotated side outputs come from the fused kernels only (16-byte rows); otherwise see below
       const bool side_ok = t.q_rot == nullptr || (c.rope_mode != 0 && tvec_ok(t.q_rot, t.qrs, p.dk, es) &&
-                                                  tvec_ok(t.k_rot, t.krs, p.dk, es) && tvec_ok(t.q, t.qs, p.dk, es));
+                                                  tvec_ok(t.k_rot, t.krs, p.dk, es));
       if (side_ok) {
         rc = swa1_forward(p, t, c, stream);
         if (rc != -1) return rc;

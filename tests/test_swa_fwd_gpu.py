@@ -125,3 +125,24 @@ def test_bad_arguments_raise():
     from dl_templates_amd._lib import DltError
     with pytest.raises(DltError):
         sw.tiled_swa_fwd(big, big, big, 1, 4, 4, 1, 1, 1.0)
+
+
+def test_token_grid_with_element_strided_operands():
+    """q, k or v whose head-dim elements are not adjacent in memory (a transposed buffer) cannot be read in
+    16-byte pieces: such calls must leave the token-grid kernels for the generic ones, forward and backward."""
+    sw = _swa()
+    B, H, th, tw, d, W = 1, 2, 12, 16, 64, 3
+    N = th * tw
+    q, k, v, do = orc.make_qkv(31, B, H, N, N, d, d, torch.bfloat16)
+    o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), 1, th, tw, W, W, 0.125)
+    tr = lambda t: t.transpose(2, 3).contiguous().cuda().transpose(2, 3)   # [B, H, N, D] view of a [B, H, D, N] buffer
+    for which in range(3):
+        ops = [t.cuda() for t in (q, k, v)]
+        ops[which] = tr((q, k, v)[which])
+        assert ops[which].stride(3) != 1
+        qg, kg, vg = (t.detach().requires_grad_(True) for t in ops)
+        o = sw.TiledSwa.apply(qg, kg, vg, 1, th, tw, W, W, 0.125)
+        o.backward(do.cuda())
+        assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL, which
+        rel = lambda g, w: ((g.float().cpu() - w).abs().max() / w.abs().max()).item()
+        assert max(rel(qg.grad, dq_w), rel(kg.grad, dk_w), rel(vg.grad, dv_w)) <= 5e-2, which
