@@ -149,10 +149,14 @@ void swa1_make_plan(const AttnProblem& p, const Swa1Class& c, int n_regions, int
   if (plan.lds_bytes < own_tile) plan.lds_bytes = own_tile;
 }
 
-// the token-grid kernels index a [N, D] slab with 32-bit element offsets
-bool swa1_strides_fit(const AttnTensors& t) {
-  const int64_t lim = (int64_t)1 << 20;
-  return t.qs[2] < lim && t.ks[2] < lim && t.vs[2] < lim && (t.d_o == nullptr || t.dos[2] < lim);
+// the token-grid kernels address the streamed tensors with 32-bit BYTE offsets inside a (batch, head) slab
+bool swa1_strides_fit(const AttnProblem& p, const AttnTensors& t) {
+  const int64_t ntok = (int64_t)p.g.TR * p.g.TC, lim = ((int64_t)1 << 31) - 1;
+  const int64_t row = 2 * (int64_t)(p.dk > p.dv ? p.dk : p.dv);   // bytes of the last row
+  auto fits = [&](const int64_t* st) { return st[2] >= 0 && (ntok - 1) * st[2] * 2 + row <= lim; };
+  // lse2 / delta of the halo tokens are fetched with 32-bit element offsets (backward)
+  const bool scalars_fit = t.ls[2] >= 0 && (ntok - 1) * t.ls[2] <= lim;
+  return fits(t.qs) && fits(t.ks) && fits(t.vs) && (t.d_o == nullptr || (fits(t.dos) && scalars_fit));
 }
 
 int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c_in, hipStream_t stream) {
@@ -343,7 +347,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
     // q is not streamed, but its own-token fragments are read as 16-byte pieces too
     const bool streamed[3] = {tvec_ok(t.q, t.qs, p.dk, es), tvec_ok(t.k, t.ks, p.dk, es), tvec_ok(t.v, t.vs, p.dv, es)};
     Swa1Class c;
-    if (swa1_eligible(p, streamed, 3, c) && swa1_strides_fit(t)) {
+    if (swa1_eligible(p, streamed, 3, c) && swa1_strides_fit(p, t)) {
       // rotated side outputs come from the fused kernels only (16-byte rows); otherwise see below
       const bool side_ok = t.q_rot == nullptr || (c.rope_mode != 0 && tvec_ok(t.q_rot, t.qrs, p.dk, es) &&
                                                   tvec_ok(t.k_rot, t.krs, p.dk, es));
@@ -403,7 +407,7 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
     const bool streamed[4] = {tvec_ok(t.q, t.qs, p.dk, es), tvec_ok(t.k, t.ks, p.dk, es),
                               tvec_ok(t.v, t.vs, p.dv, es), tvec_ok(t.d_o, t.dos, p.dv, es)};
     Swa1Class c;
-    if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(t)) return swa1_backward(p, t, c, stream);
+    if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(p, t)) return swa1_backward(p, t, c, stream);
   }
   if (p.rope_prerot && p.rope.enabled && p.rope.R > 0 && !p.tm.img) {
     // rotated q, k and no token-grid kernel: the plain operator (any kernel family) yields the gradients of the

@@ -146,3 +146,20 @@ def test_token_grid_with_element_strided_operands():
         assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL, which
         rel = lambda g, w: ((g.float().cpu() - w).abs().max() / w.abs().max()).item()
         assert max(rel(qg.grad, dq_w), rel(kg.grad, dk_w), rel(vg.grad, dv_w)) <= 5e-2, which
+
+
+def test_token_grid_offsets_beyond_32_bits_take_the_generic_kernels():
+    """A token stride so large that byte offsets inside a (batch, head) slab pass 2 GiB: the token-grid kernels
+    (32-bit offsets) must not be chosen.  The tensors are strided views of one byte-saving buffer: every token
+    row is re-used (stride 0 over a block of rows is not expressible), so the view steps over a 1.2 GiB buffer."""
+    sw = _swa()
+    B, H, th, tw, d, W = 1, 1, 32, 36, 64, 2
+    N = th * tw
+    big = (1 << 20) - 8                             # elements between tokens (16-byte aligned rows): (N - 1) * big * 2 bytes = 2.4 GB > 2 GiB
+    buf = torch.zeros((N - 1) * big + d, dtype=torch.bfloat16, device="cuda")
+    q, k, v, _ = orc.make_qkv(12, B, H, N, N, d, d, torch.bfloat16)
+    want = orc.tiled_swa_ref(q.float(), k.float(), v.float(), 1, th, tw, W, W, 0.125)
+    kview = torch.as_strided(buf, (B, H, N, d), (0, 0, big, 1))
+    kview.copy_(k.cuda())
+    got = sw.tiled_swa_fwd(q.cuda(), kview, v.cuda(), 1, th, tw, W, W, 0.125)
+    assert (got.float().cpu() - want).abs().max().item() <= FWD_TOL
