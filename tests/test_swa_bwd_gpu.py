@@ -226,3 +226,25 @@ def test_rotated_side_outputs_with_awkward_strides():
         errs = (_rel(dq, dq_w), _rel(dk, dk_w), _rel(dv, dv_w))
         assert max(errs) <= GRAD_TOL, errs
     del keep
+
+
+@pytest.mark.parametrize("d,dv,R,th,tw,W,save", [(32, 32, 8, 12, 20, 3, True), (32, 32, 8, 12, 20, 3, False), (32, 64, 8, 9, 9, 2, True),
+                                                  (96, 96, 8, 10, 12, 3, True), (96, 128, 16, 10, 12, 3, False),
+                                                  (64, 32, 16, 8, 8, 2, True), (128, 64, 8, 8, 12, 4, True)])
+def test_fused_rope_with_head_dims_below_the_padded_class(d, dv, R, th, tw, W, save, monkeypatch):
+    """dk / dv that do not fill their padded class (32 in the 64 class, 96 in the 128 class) and dk != dv, with the
+    rotation fused: staged pieces beyond the head dim stay zero, side outputs and gradients stop at the head dim."""
+    sw = _swa()
+    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save)
+    N = th * tw
+    q, k, v, do = orc.make_qkv(d + R, 1, 2, N, N, d, dv, torch.bfloat16)
+    idx = orc.make_rope_idx(2, th, tw, 0.1)
+    rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+    scale = 1 / math.sqrt(d)
+    o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, W, W, scale)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, W, W, scale)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert max(errs) <= GRAD_TOL, errs
