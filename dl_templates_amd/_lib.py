@@ -189,10 +189,19 @@ def require_cuda(*tensors: torch.Tensor) -> None:
             raise RuntimeError(f"all tensors must be on one device, got {dev} and {t.device}")
 
 
-def rope_desc(idx: torch.Tensor, row_cs: torch.Tensor, col_cs: torch.Tensor):
-    """(RopeDesc, keep-alive tuple).  Tables must be fp32 [len, R, 2] with a contiguous [R, 2] tail."""
+def rope_desc(idx: torch.Tensor, row_cs: torch.Tensor, col_cs: torch.Tensor, like: torch.Tensor = None,
+              n_tokens: int = None):
+    """(RopeDesc, keep-alive tuple).  Tables must be fp32 [len, R, 2] with a contiguous [R, 2] tail.
+
+    ``like``: the tensor the rotation is applied to; idx and both tables must live on its device (the kernels
+    dereference them: a host pointer would fault on the GPU instead of raising).  ``n_tokens``: idx must have
+    exactly one entry per token."""
     if idx.dtype != torch.int32 or idx.dim() != 1 or not idx.is_contiguous():
         raise TypeError("idx must be a contiguous 1-D int32 tensor")
+    if n_tokens is not None and idx.shape[0] != n_tokens:
+        raise ValueError(f"idx has {idx.shape[0]} entries for {n_tokens} tokens")
+    if like is not None:
+        require_cuda(like, idx, row_cs, col_cs)
     tabs = []
     for t in (row_cs, col_cs):
         if t.dim() != 3 or t.shape[2] != 2:

@@ -2,6 +2,7 @@
 // reference's call signatures into the attention-core problem description.
 #include "dlt_internal.hpp"
 #include <string.h>
+#include <cmath>
 
 static thread_local char g_err[512] = "";
 
@@ -120,6 +121,7 @@ int swa_problem(const char* who, const dlt_swa_shape_t* s, const dlt_rope_t* rop
   DLT_REQUIRE(s->row_size >= 0 && s->col_size >= 0, "%s: negative window (%d, %d)", who, s->row_size, s->col_size);
   DLT_REQUIRE(s->dk > 0 && s->dv > 0, "%s: dk=%d dv=%d must be positive", who, s->dk, s->dv);
   DLT_REQUIRE((int64_t)s->t_height * s->t_width * s->b_size <= 0x3fffffff, "%s: too many tokens", who);
+  DLT_REQUIRE(std::isfinite(s->sm_scale), "%s: sm_scale is not finite", who);
   p.g.mode = DLT_GEOM_SWA;
   p.g.TR = s->t_height;
   p.g.TC = s->t_width;
@@ -144,6 +146,7 @@ int flash_problem(const char* who, const dlt_flash_shape_t* s, AttnProblem& p) {
   DLT_REQUIRE(s->B > 0 && s->H > 0 && s->Lq > 0 && s->Lk > 0, "%s: B=%d H=%d Lq=%d Lk=%d must be positive", who, s->B, s->H, s->Lq, s->Lk);
   DLT_REQUIRE(s->dk > 0 && s->dv > 0, "%s: dk=%d dv=%d must be positive", who, s->dk, s->dv);
   DLT_REQUIRE(!s->causal || s->Lq == s->Lk, "%s: causal attention needs Lq == Lk (got %d, %d)", who, s->Lq, s->Lk);
+  DLT_REQUIRE(std::isfinite(s->sm_scale), "%s: sm_scale is not finite", who);
   p.g.mode = s->causal ? DLT_GEOM_CAUSAL : DLT_GEOM_DENSE;
   p.g.TR = 1; p.g.TC = 1; p.g.S = 1; p.g.WR = 0; p.g.WC = 0;
   p.g.XLq = s->Lq; p.g.XLk = s->Lk;

@@ -76,6 +76,27 @@ int DLT_CAT3(dlt_launch_delta_, DLT_DK, DLT_DV)(const BwdArgs& a, hipStream_t st
   }
 }
 
+#ifdef DLT_ONE_PATCH
+// head-dim classes whose accumulators leave no room for two query blocks per wave: np must be 1
+int DLT_CAT3(dlt_launch_bwd_, DLT_DK, DLT_DV)(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q, int np,
+                                              hipStream_t stream) {
+  if (np != 1) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward: this head-dim class takes one query block per wave");
+  switch (aq.p.dtype) {
+    case DLT_BF16: return launch_bwd_t<bf16_t, 1>(akv, grid_kv, aq, grid_q, stream);
+    case DLT_FP16: return launch_bwd_t<f16_t, 1>(akv, grid_kv, aq, grid_q, stream);
+    default: return launch_bwd_t<float, 1>(akv, grid_kv, aq, grid_q, stream);
+  }
+}
+
+int DLT_CAT3(dlt_launch_fwd_, DLT_DK, DLT_DV)(const FwdArgs& a, int np, int grid, hipStream_t stream) {
+  if (np != 1) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: this head-dim class takes one query block per wave");
+  switch (a.p.dtype) {
+    case DLT_BF16: return launch_fwd_t<bf16_t, 1>(a, grid, stream);
+    case DLT_FP16: return launch_fwd_t<f16_t, 1>(a, grid, stream);
+    default: return launch_fwd_t<float, 1>(a, grid, stream);
+  }
+}
+#else
 int DLT_CAT3(dlt_launch_bwd_, DLT_DK, DLT_DV)(const BwdArgs& akv, int grid_kv, const BwdArgs& aq, int grid_q, int np,
                                               hipStream_t stream) {
   switch (aq.p.dtype) {
@@ -92,3 +113,4 @@ int DLT_CAT3(dlt_launch_fwd_, DLT_DK, DLT_DV)(const FwdArgs& a, int np, int grid
     default: return np == 1 ? launch_fwd_t<float, 1>(a, grid, stream) : launch_fwd_t<float, 2>(a, grid, stream);
   }
 }
+#endif

@@ -10,11 +10,13 @@ int dlt_launch_fwd_32_32(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_64_64(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_128_128(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_64_128(const FwdArgs&, int, int, hipStream_t);
+int dlt_launch_fwd_256_256(const FwdArgs&, int, int, hipStream_t);
 
 int dlt_launch_bwd_32_32(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_64_64(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_128_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 int dlt_launch_bwd_64_128(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
+int dlt_launch_bwd_256_256(const BwdArgs&, int, const BwdArgs&, int, int, hipStream_t);
 
 int dlt_flash_launch_fwd_32_32(const FlashArgs&, int, int, hipStream_t);
 int dlt_flash_launch_fwd_64_64(const FlashArgs&, int, int, hipStream_t);
@@ -28,6 +30,7 @@ int dlt_launch_delta_32_32(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_64_64(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_128_128(const BwdArgs&, hipStream_t);
 int dlt_launch_delta_64_128(const BwdArgs&, hipStream_t);
+int dlt_launch_delta_256_256(const BwdArgs&, hipStream_t);
 int dlt_swa1_launch_bwd_64(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
 int dlt_swa1_launch_bwd_128(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
 int dlt_swa1_launch_fwd_64(const Swa1FwdArgs&, int, int, hipStream_t);
@@ -44,7 +47,8 @@ int pick_dims(const AttnProblem& p, DimClass& dc) {
   else if (p.dk <= 64 && p.dv <= 64) dc = {64, 64, 0};
   else if (p.dk <= 64 && p.dv <= 128) dc = {64, 128, 2};
   else if (p.dk <= 128 && p.dv <= 128) dc = {128, 128, 1};
-  else return dlt_set_error(DLT_ERR_UNSUPPORTED, "head dims dk=%d dv=%d: at most 128 is supported", p.dk, p.dv);
+  else if (p.dk <= 256 && p.dv <= 256) dc = {256, 256, 4};  // the largest head dim the reference admits (src/flash_attn.py:460-462): generic kernels only
+  else return dlt_set_error(DLT_ERR_UNSUPPORTED, "head dims dk=%d dv=%d: at most 256 is supported", p.dk, p.dv);
   return DLT_OK;
 }
 
@@ -111,6 +115,7 @@ struct Swa1Class { int D, wclass, pbit, rope_mode; };
 bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streamed, Swa1Class& c) {
   if (p.g.mode != DLT_GEOM_SWA || p.g.S != 1 || p.tm.img) return false;
   if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
+  if (!(p.sm_scale > 0.f)) return false;  // the running max is kept on raw scores: needs a positive scale
   if (p.dk % 32 != 0 || p.dv % 32 != 0) return false;  // 64-byte staging pieces
   if (p.dk <= 64 && p.dv <= 64) c.D = 64;
   else if (p.dk <= 128 && p.dv <= 128 && p.dk > 64 && p.dv > 64) c.D = 128;
@@ -131,6 +136,10 @@ bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streame
     // balanced staging map: the rotation covers exactly half of a fully used head dim, so there
     // are as many rotary chunk pairs per token as staging threads
     c.rope_mode = (2 * r8 == c.D / 32 && p.dk == c.D && p.dv == c.D) ? 2 : 1;
+    // plain staging map: a thread holds 4 neighbouring chunks of a token, so rotary partners must be 1 or 2
+    // chunks apart; farther partners (R = 32: 4 chunks) sit in another thread's piece.  Tensors that arrive
+    // rotated are staged without rotation and are not affected.
+    if (c.rope_mode == 1 && r8 > 2 && !p.rope_prerot) return false;
   }
   return true;
 }
@@ -241,6 +250,8 @@ bool flash_eligible(const AttnProblem& p, const AttnTensors& t, bool with_do) {
     if (p.rope.enabled && p.rope.R > 0) return false;
   }
   if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
+  if (!(p.sm_scale > 0.f)) return false;  // the running max is kept on raw scores: needs a positive scale
+  if (p.dk > 128 || p.dv > 128) return false;
   const int es = 2;
   if (!tvec_ok(t.q, t.qs, p.dk, es) || !tvec_ok(t.k, t.ks, p.dk, es) || !tvec_ok(t.v, t.vs, p.dv, es)) return false;
   if (with_do && !tvec_ok(t.d_o, t.dos, p.dv, es)) return false;
@@ -371,7 +382,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
     return dlt_attn_forward(p2, t2, stream);
   }
   if (flash_eligible(p, t, false)) return flash_forward(p, t, dc, stream);
-  const int np = p.g.mode == DLT_GEOM_SWA ? 1 : 2;
+  const int np = (p.g.mode == DLT_GEOM_SWA || dc.id == 4) ? 1 : 2;
   const int own = 64 * np;
   const int PQ = dc.DK * 2 + 16, PK = dc.DK * 2 + 16, PV = dc.DV * 2 + 16, PO = dc.DV * es + 16;
   FwdArgs a;
@@ -394,6 +405,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
     case 0: return dlt_launch_fwd_64_64(a, np, (int)grid, stream);
     case 1: return dlt_launch_fwd_128_128(a, np, (int)grid, stream);
     case 3: return dlt_launch_fwd_32_32(a, np, (int)grid, stream);
+    case 4: return dlt_launch_fwd_256_256(a, np, (int)grid, stream);
     default: return dlt_launch_fwd_64_128(a, np, (int)grid, stream);
   }
 }
@@ -478,6 +490,7 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
     case 0: return dlt_launch_bwd_64_64(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
     case 1: return dlt_launch_bwd_128_128(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
     case 3: return dlt_launch_bwd_32_32(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
+    case 4: return dlt_launch_bwd_256_256(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
     default: return dlt_launch_bwd_64_128(akv, (int)grid_kv, aq, (int)grid_q, np, stream);
   }
 }

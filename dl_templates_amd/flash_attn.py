@@ -22,19 +22,25 @@ def _shape(q, k, v, causal, sm_scale) -> _lib.FlashShape:
                            int(bool(causal)), _lib.dtype_code(q))
 
 
+def _forward(q, k, v, causal, sm_scale):
+    """(o, M): the output and the saved log2-domain log-sum-exp [B, H, Lq] (src/flash_attn.py:463-483)."""
+    shape = _shape(q, k, v, causal, sm_scale)
+    _lib.require_cuda(q, k, v)
+    lib = _lib.load()
+    o = torch.empty((q.shape[0], q.shape[1], q.shape[2], v.shape[-1]), dtype=q.dtype, device=q.device)
+    M = torch.empty((q.shape[0], q.shape[1], q.shape[2]), device=q.device, dtype=torch.float32)
+    with torch.cuda.device(q.device):
+        _lib.check(lib.dlt_flash_fwd(_lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v),
+                                     _lib.strides(v), _lib.ptr(o), _lib.strides(o), _lib.ptr(M), _lib.strides(M),
+                                     shape, _lib.stream_of(q)))
+    return o, M
+
+
 class _attention(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, q, k, v, causal, sm_scale):
-        shape = _shape(q, k, v, causal, sm_scale)
-        _lib.require_cuda(q, k, v)
-        lib = _lib.load()
-        o = torch.empty((q.shape[0], q.shape[1], q.shape[2], v.shape[-1]), dtype=q.dtype, device=q.device)
-        M = torch.empty((q.shape[0], q.shape[1], q.shape[2]), device=q.device, dtype=torch.float32)
-        with torch.cuda.device(q.device):
-            _lib.check(lib.dlt_flash_fwd(_lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v),
-                                         _lib.strides(v), _lib.ptr(o), _lib.strides(o), _lib.ptr(M), _lib.strides(M),
-                                         shape, _lib.stream_of(q)))
+        o, M = _forward(q, k, v, causal, sm_scale)
         ctx.save_for_backward(q, k, v, o, M)
         ctx.sm_scale = sm_scale
         ctx.causal = causal

@@ -39,7 +39,7 @@ def _forward(q, k, v, shape, rope):
     B, H, N, _ = q.shape
     o = torch.empty((B, H, N, v.shape[-1]), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
-    desc, keep = (None, None) if rope is None else _lib.rope_desc(*rope)
+    desc, keep = (None, None) if rope is None else _lib.rope_desc(*rope, like=q, n_tokens=q.shape[2])
     with torch.cuda.device(q.device):
         _lib.check(lib.dlt_swa_fwd(_lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v),
                                    _lib.strides(v), _lib.ptr(o), _lib.strides(o), _lib.ptr(lse), _lib.strides(lse),
@@ -55,7 +55,7 @@ def _backward(q, k, v, o, lse, do, shape, rope):
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
     delta = torch.empty_like(lse)
-    desc, keep = (None, None) if rope is None else _lib.rope_desc(*rope)
+    desc, keep = (None, None) if rope is None else _lib.rope_desc(*rope, like=q, n_tokens=q.shape[2])
     with torch.cuda.device(q.device):
         _lib.check(lib.dlt_swa_bwd(_lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v),
                                    _lib.strides(v), _lib.ptr(o), _lib.strides(o), _lib.ptr(do), _lib.strides(do),
@@ -101,9 +101,9 @@ def _forward_rot(q, k, v, shape, rope):
     B, H, N, _ = q.shape
     o = torch.empty((B, H, N, v.shape[-1]), dtype=q.dtype, device=q.device)
     lse = torch.empty((B, H, N), dtype=torch.float32, device=q.device)
+    desc, keep = _lib.rope_desc(*rope, like=q, n_tokens=q.shape[2])
     q_rot = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     k_rot = torch.empty(k.shape, dtype=k.dtype, device=k.device)
-    desc, keep = _lib.rope_desc(*rope)
     with torch.cuda.device(q.device):
         _lib.check(_lib.load().dlt_swa_fwd_rot(
             _lib.ptr(q), _lib.strides(q), _lib.ptr(k), _lib.strides(k), _lib.ptr(v), _lib.strides(v),
@@ -117,7 +117,7 @@ def _backward_rot(q_rot, k_rot, v, o, lse, do, shape, rope):
     _lib.require_cuda(q_rot, k_rot, v, o, lse, do)
     dq, dk, dv = torch.empty_like(q_rot), torch.empty_like(k_rot), torch.empty_like(v)
     delta = torch.empty_like(lse)
-    desc, keep = _lib.rope_desc(*rope)
+    desc, keep = _lib.rope_desc(*rope, like=v, n_tokens=v.shape[2])
     with torch.cuda.device(v.device):
         _lib.check(_lib.load().dlt_swa_bwd_rot(
             _lib.ptr(q_rot), _lib.strides(q_rot), _lib.ptr(k_rot), _lib.strides(k_rot), _lib.ptr(v), _lib.strides(v),

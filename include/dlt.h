@@ -80,7 +80,9 @@ typedef struct {
   int32_t B, H;
   int32_t b_size, t_height, t_width, row_size, col_size;
   int32_t dk, dv; /* q/k head dim, v/o head dim */
-  float sm_scale;
+  float sm_scale; /* must be finite (else DLT_ERR_INVALID); any sign is accepted as in the reference, which scales
+                     before taking the row max: the tuned kernels keep the max of the raw scores and take positive
+                     scales only, zero and negative scales run on the generic kernels */
   int32_t dtype;  /* dlt_dtype_t */
 } dlt_swa_shape_t;
 

@@ -17,9 +17,13 @@ of one reference function, cited as ``file:line`` relative to the reference tree
 * ``rope2d_ref``           - src/fused_rope2d.py:204-225
 * ``rope2d_bwd_ref``       - src/fused_rope2d.py:110-122 (transposed rotation)
 * ``flash_ref``            - src/flash_attn.py:625 (plain SDPA with scale)
-* ``rope_tables``          - src/fused_rope2d.py:236-246 gives the packing ([max_len, R, 2],
-                             cos then sin).  PARITY UNPINNED for the frequency formula: the
-                             file that defines it (src/rope2d.py) is absent from the reference.
+* ``rope_tables``          - src/fused_rope2d.py:236-246: the self-test's table construction
+                             (theta_i = base ** (-2 i / R), outer product with the positions,
+                             cos and sin stacked on the last axis: [max_len, R, 2]).  The file
+                             the module imports its tables from (src/rope2d.py) is absent from the
+                             reference; this construction is the only one the reference holds.
+                             Pinned in tests/test_oracle.py against the literal torch expression
+                             of those lines and against unit-circle / angle-addition identities.
 * ``swa_pairs``/``attn_flops`` - src/flash_attn.py:608-614 FLOP convention.
 * ``tokens_to_image``/``image_to_tokens`` - src/tiled_swa.py:753-755 (tile-major [B, H, N, D] to the
                              image layout [B, IH, IW, H, D] and back); ``image_token_index`` is the
@@ -248,11 +252,11 @@ def rope2d_bwd_ref(do, idx, cs_row_buffer, cs_col_buffer):
 # --------------------------------------------------------------------------- a7
 def rope_tables(n_rdim: int, max_len: int, base: float = 10000.0) -> torch.Tensor:
     """[max_len, n_rdim, 2] fp32, (cos, sin) on the last axis (packing per
-    src/fused_rope2d.py:238-240).  theta_i = base ** (-i / n_rdim).  PARITY UNPINNED (see header).
-    Angles are formed in float64 and rounded once to fp32."""
-    inv = np.power(float(base), -np.arange(n_rdim, dtype=np.float64) / n_rdim)
-    ang = np.outer(np.arange(max_len, dtype=np.float64), inv)
-    return torch.from_numpy(np.stack([np.cos(ang), np.sin(ang)], axis=-1).astype(np.float32))
+    src/fused_rope2d.py:236-240): theta_i = base ** (-2 i / n_rdim), entry [p, i] = exp(1j p theta_i).
+    Evaluated in float64 as a complex exponential and rounded once to fp32."""
+    theta = np.exp(-2.0 * np.log(float(base)) * np.arange(n_rdim, dtype=np.float64) / n_rdim)
+    z = np.exp(1j * np.arange(max_len, dtype=np.float64)[:, None] * theta[None, :])
+    return torch.from_numpy(np.stack([z.real, z.imag], axis=-1).astype(np.float32))
 
 
 # --------------------------------------------------------------------------- a9/a10
@@ -270,8 +274,13 @@ def flash_grads(q, k, v, do, causal, sm_scale):
     return o.detach(), q.grad, k.grad, v.grad
 
 
-def flash_lse2(q, k, sm_scale):
+def flash_lse2(q, k, sm_scale, causal: bool = False):
+    """log2-domain log-sum-exp of the scaled scores, the vector M the forward pass saves
+    (src/flash_attn.py:168-171: m_i + log2(l_i)); causal: keys up to the query's own index."""
     s = torch.matmul(q.float(), k.float().transpose(-1, -2)) * sm_scale
+    if causal:
+        Lq, Lk = s.shape[-2:]
+        s = s.masked_fill(torch.arange(Lk)[None, :] > torch.arange(Lq)[:, None], float("-inf"))
     return torch.logsumexp(s, dim=-1) * (1.0 / math.log(2.0))
 
 

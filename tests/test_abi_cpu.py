@@ -44,6 +44,11 @@ def test_argument_validation_happens_before_any_launch():
     shape = L.SwaShape(1, 1, 1, 4, 4, 1, 1, 512, 64, 1.0, 0)
     rc = lib.dlt_swa_fwd(one, st4, one, st4, one, st4, one, st4, one, st3, shape, None, None)
     assert rc == 2 and b"head dims" in lib.dlt_last_error()
+    shape = L.SwaShape(1, 1, 1, 4, 4, 1, 1, 64, 64, float("inf"), 0)
+    rc = lib.dlt_swa_fwd(one, st4, one, st4, one, st4, one, st4, one, st3, shape, None, None)
+    assert rc == 1 and b"sm_scale" in lib.dlt_last_error()
+    rc = lib.dlt_flash_fwd(one, st4, one, st4, one, st4, one, st4, one, st3, L.FlashShape(1, 1, 8, 8, 64, 64, float("nan"), 0, 0), None)
+    assert rc == 1 and b"sm_scale" in lib.dlt_last_error()
     st5 = (ctypes.c_int64 * 5)(1, 1, 1, 1, 1)
     shape = L.SwaShape(1, 1, 6, 4, 4, 1, 1, 64, 64, 1.0, 0)  # tile of 2 x 2 pixels is not 6 tokens
     rc = lib.dlt_swa_fwd_image(one, st5, one, st5, one, st5, one, st5, one, st3, shape, L.SwaTile(2, 2), None, None)
@@ -72,7 +77,29 @@ def test_table_context_matches_oracle_tables():
     from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
     from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as M
     from oracle import attn_oracle as orc
-    assert torch.equal(Ctx(16, 64).cs_components, orc.rope_tables(8, 64))
+    assert (Ctx(16, 64).cs_components - orc.rope_tables(8, 64)).abs().max().item() <= 1.2e-7
     assert torch.equal(M.encode_idx(5, 7), orc.encode_idx(5, 7))
     m = M(32, 8, 9)
     assert m.row_buffer.cs_components.shape == (8, 8, 2) and m.col_buffer.cs_components.shape == (9, 8, 2)
+
+
+def test_rope_operands_on_the_host_raise_before_any_launch():
+    """idx / tables are dereferenced by the kernels: the attention wrappers must refuse host tensors (what
+    encode_idx returns without a default device) instead of handing a host pointer to the GPU."""
+    import pytest
+    import torch
+    from dl_templates_amd import _lib
+    from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as M
+
+    class OnGpu:   # stands in for the CUDA tensor the rotation is applied to (no GPU in the CPU suite)
+        is_cuda = True
+        device = torch.device("cuda:0")
+
+    idx = M.encode_idx(4, 4)
+    tab = torch.zeros(4, 8, 2)
+    with pytest.raises(RuntimeError, match="ROCm GPU only"):
+        _lib.rope_desc(idx, tab, tab, like=OnGpu())
+    with pytest.raises(ValueError, match="entries for"):
+        _lib.rope_desc(idx, tab, tab, n_tokens=17)
+    with pytest.raises(TypeError):
+        _lib.rope_desc(idx.long(), tab, tab)

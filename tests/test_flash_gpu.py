@@ -67,6 +67,51 @@ def test_cross_attention_distinct_dims_and_lengths(Lq, Lk, dk, dv, dtype):
     assert max(errs) <= 5e-2, errs
 
 
+@pytest.mark.parametrize("causal,Lq,Lk,dk,dv,dtype", [
+    (False, 256, 512, 64, 128, torch.bfloat16), (False, 100, 333, 64, 64, torch.float16), (True, 300, 300, 128, 128, torch.bfloat16),
+    (True, 129, 129, 32, 32, torch.float16), (False, 77, 190, 48, 80, torch.float32), (False, 1, 1, 16, 16, torch.bfloat16)])
+def test_saved_log_sum_exp(causal, Lq, Lk, dk, dv, dtype):
+    """M = m + log2(l), the vector the forward pass saves for the backward pass (src/flash_attn.py:168-171),
+    directly against the oracle; 2e-2 in log2 units."""
+    q, k, v, _ = orc.make_qkv(Lq + 3 * Lk, 2, 2, Lq, Lk, dk, dv, dtype)
+    scale = 1 / math.sqrt(dk)
+    o, M = _fa()._forward(q.cuda(), k.cuda(), v.cuda(), causal, scale)
+    assert M.dtype == torch.float32 and M.shape == (2, 2, Lq)
+    want = orc.flash_lse2(q, k, scale, causal)
+    assert (M.cpu() - want).abs().max().item() <= 2e-2
+    assert (o.float().cpu() - orc.flash_ref(q.float(), k.float(), v.float(), causal, scale)).abs().max().item() <= 2e-2
+
+
+def test_negative_scale_matches_sdpa():
+    q, k, v, do = orc.make_qkv(91, 1, 2, 200, 320, 64, 64, torch.bfloat16)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), False, -0.125)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(qg, kg, vg, False, -0.125)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    assert max(_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w)) <= 5e-2
+
+
+@pytest.mark.parametrize("causal,Lq,Lk,dk,dv,dtype", [
+    (False, 256, 384, 256, 256, torch.bfloat16), (True, 200, 200, 256, 256, torch.float16), (False, 65, 130, 256, 64, torch.bfloat16),
+    (False, 100, 100, 64, 256, torch.float16), (True, 129, 129, 192, 160, torch.bfloat16), (False, 40, 70, 256, 256, torch.float32)])
+def test_head_dim_256(causal, Lq, Lk, dk, dv, dtype):
+    """The reference admits head dims up to 256 (src/flash_attn.py:460-462); forward, saved log-sum-exp and
+    gradients against SDPA."""
+    q, k, v, do = orc.make_qkv(Lq + dk, 1, 2, Lq, Lk, dk, dv, dtype)
+    scale = 1 / math.sqrt(dk)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), causal, scale)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(qg, kg, vg, causal, scale)
+    o.backward(do.cuda())
+    assert o.shape == (1, 2, Lq, dv) and o.dtype == dtype
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert max(errs) <= 5e-2, errs
+    _, M = _fa()._forward(q.cuda(), k.cuda(), v.cuda(), causal, scale)
+    assert (M.cpu() - orc.flash_lse2(q, k, scale, causal)).abs().max().item() <= 2e-2
+
+
 def test_c5_shape_reduced_batch():
     # benchmark config 5 shape with B=1, H=2 (CPU oracle time): Lq=4096, Lk=8192, 64/128
     q, k, v, do = orc.make_qkv(55, 1, 2, 4096, 8192, 64, 128, torch.bfloat16)

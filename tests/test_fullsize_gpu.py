@@ -7,7 +7,10 @@ properties and a cross-check between two independent GPU implementations.
   sum(dq * q) == sum(dk * k) per head; bit-reproducibility.
 * config 4 against the CPU oracle on a band of query rows of two heads (the window makes rows
   far from the band irrelevant, so a 60 x 128 sub-grid reproduces the interior rows exactly).
-* config 3 full batch, fused RoPE: equals the unfused composition bit for bit.
+* config 4's 96 x 160 grid against the CPU oracle on its top band of rows (windows truncated at the top,
+  left and right borders, partial workgroups in the last column block).
+* config 3 full batch, fused RoPE: equals the unfused composition bit for bit; one batch entry of it
+  (all 8 heads) directly against the CPU oracle's composition, forward and backward.
 * config 5 full size: flash kernels against the generic dense kernels (fp32 inputs route there).
 """
 import math
@@ -87,6 +90,58 @@ def test_c4_band_against_cpu_oracle():
     inner2_b = slice(2 * W * tw, (r1 - r0 - 2 * W) * tw)
     assert rel(kg.grad.float().cpu()[:, :, inner2], dk_w[:, :, inner2_b]) <= 5e-2
     assert rel(vg.grad.float().cpu()[:, :, inner2], dv_w[:, :, inner2_b]) <= 5e-2
+
+
+def test_c4_ragged_grid_border_band_against_cpu_oracle():
+    """Rows 0..39 of the 96 x 160 grid as a stand-alone 40 x 160 grid for the oracle (H = 2, d = 128, 21 x 21
+    window).  Queries of rows 0..29 have their whole (border-truncated) window inside the band: o, lse2 and dq
+    are exact there; keys of rows 0..19 are only seen by such queries: dk, dv exact there."""
+    sw, _, _ = _mods()
+    th, tw, d, W, band = 96, 160, 128, 10, 40
+    q, k, v, do = orc.make_qkv(42, 1, 2, th * tw, th * tw, d, d, torch.bfloat16)
+    scale = 1 / math.sqrt(d)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = sw.TiledSwa.apply(qg, kg, vg, 1, th, tw, W, W, scale)
+    o.backward(do.cuda())
+    sl = slice(0, band * tw)
+    o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q[:, :, sl].float(), k[:, :, sl].float(), v[:, :, sl].float(),
+                                                do[:, :, sl].float(), 1, band, tw, W, W, scale)
+    nq, nk = (band - W) * tw, (band - 2 * W) * tw
+    assert (o.float().cpu()[:, :, :nq] - o_w[:, :, :nq]).abs().max().item() <= 2e-2
+    rel = lambda a, b: ((a - b).abs().max() / b.abs().max()).item()
+    assert rel(qg.grad.float().cpu()[:, :, :nq], dq_w[:, :, :nq]) <= 5e-2
+    assert rel(kg.grad.float().cpu()[:, :, :nk], dk_w[:, :, :nk]) <= 5e-2
+    assert rel(vg.grad.float().cpu()[:, :, :nk], dv_w[:, :, :nk]) <= 5e-2
+    # the bottom band the same way (rows 56..95): windows truncated at the bottom border
+    sl = slice((th - band) * tw, th * tw)
+    o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q[:, :, sl].float(), k[:, :, sl].float(), v[:, :, sl].float(),
+                                                do[:, :, sl].float(), 1, band, tw, W, W, scale)
+    off = (th - band) * tw
+    assert (o.float().cpu()[:, :, off + W * tw:] - o_w[:, :, W * tw:]).abs().max().item() <= 2e-2
+    assert rel(qg.grad.float().cpu()[:, :, off + W * tw:], dq_w[:, :, W * tw:]) <= 5e-2
+    assert rel(kg.grad.float().cpu()[:, :, off + 2 * W * tw:], dk_w[:, :, 2 * W * tw:]) <= 5e-2
+    assert rel(vg.grad.float().cpu()[:, :, off + 2 * W * tw:], dv_w[:, :, 2 * W * tw:]) <= 5e-2
+
+
+@pytest.mark.parametrize("save_rotated", [True, False])
+def test_c3_one_batch_fused_rope_against_cpu_oracle(save_rotated, monkeypatch):
+    """Config 3 with B = 1 (all 8 heads, 64 x 64, d = 64, 13 x 13, rotary 32 of 64 dims, 5 % no-PE tokens): the fused
+    op directly against the oracle's composition rope -> attention and its autograd."""
+    sw, _, _ = _mods()
+    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save_rotated)
+    B, H, th, tw, d, W = 1, 8, 64, 64, 64, 6
+    N = th * tw
+    q, k, v, do = orc.make_qkv(31, B, H, N, N, d, d, torch.bfloat16)
+    idx = orc.make_rope_idx(32, th, tw, 0.05)
+    rcs, ccs = orc.rope_tables(8, th), orc.rope_tables(8, tw)
+    o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, W, W, 0.125)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, W, W, 0.125)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    rel = lambda a, b: ((a.float().cpu() - b).abs().max() / b.abs().max()).item()
+    errs = (rel(qg.grad, dq_w), rel(kg.grad, dk_w), rel(vg.grad, dv_w))
+    assert max(errs) <= 5e-2, errs
 
 
 @pytest.mark.parametrize("save_rotated", [True, False])

@@ -1,0 +1,135 @@
+"""Seeded random sweeps of the three operator families against the CPU oracle: a bounded number of cases each
+(the same generators found the boundary bugs fixed during development), stopping at the first failure and naming
+the case.  Bars as everywhere: forward max-abs <= 2e-2, dQ / dK / dV relative <= 5e-2.
+"""
+import math
+import random
+
+import pytest
+import torch
+
+from oracle import attn_oracle as orc
+
+pytestmark = pytest.mark.gpu
+N_CASES = 30
+
+
+def _rel(g, w):
+    return ((g.float().cpu() - w).abs().max() / w.abs().max().clamp_min(1e-3)).item()
+
+
+def _check(tag, o, o_w, grads, wants):
+    ef = (o.float().cpu() - o_w).abs().max().item()
+    eg = max(_rel(g, w) for g, w in zip(grads, wants))
+    assert ef <= 2e-2 and eg <= 5e-2, f"{tag}: fwd {ef:.3e} grad {eg:.3e}"
+
+
+def test_random_sliding_window_cases():
+    from dl_templates_amd import tiled_swa as sw
+    rng = random.Random(2)
+    done = 0
+    while done < N_CASES:
+        S = rng.choice([1, 1, 1, 16, 32])
+        th, tw = rng.randint(1, 24 if S == 1 else 6), rng.randint(1, 40 if S == 1 else 7)
+        WR, WC = rng.randint(0, 10 if S == 1 else 2), rng.randint(0, 10 if S == 1 else 2)
+        d = rng.choice([32, 64, 128])
+        dv = rng.choice([d, d, 64 if d == 32 else d])
+        if S == 1 and d == 32:
+            dv = 32
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        H = rng.randint(1, 2)
+        use_rope = S == 1 and rng.random() < 0.4 and d >= 64 and dv == d
+        R = rng.choice([8, 16, 32]) if d == 128 else 8
+        N = th * tw * S
+        if N > 4000:
+            continue
+        done += 1
+        tag = f"case {done}: S={S} grid={th}x{tw} W=({WR},{WC}) d={d}/{dv} {dt} rope={use_rope} R={R}"
+        print(tag, flush=True)
+        q, k, v, do = orc.make_qkv(done * 7 + 1, 1, H, N, N, d, dv, dt)
+        scale = 1 / math.sqrt(d)
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        if use_rope:
+            idx = orc.make_rope_idx(done, th, tw, 0.1)
+            rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+            o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, WR, WC, scale)
+            o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, WR, WC, scale)
+        else:
+            o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), S, th, tw, WR, WC, scale)
+            o = sw.TiledSwa.apply(qg, kg, vg, S, th, tw, WR, WC, scale)
+        o.backward(do.cuda())
+        _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
+
+
+def test_random_flash_cases():
+    from dl_templates_amd import flash_attn as fa
+    rng = random.Random(3)
+    for it in range(N_CASES):
+        causal = rng.random() < 0.5
+        Lq = rng.choice([1, 15, 64, 65, 127, 128, 129, 200, 511, 700])
+        Lk = Lq if causal else rng.choice([1, 31, 64, 100, 257, 640, 900])
+        dk = rng.choice([16, 32, 48, 64, 96, 128, 256])
+        dv = rng.choice([16, 32, 64, 80, 128, 256])
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        tag = f"case {it}: causal={causal} L=({Lq},{Lk}) d={dk}/{dv} {dt}"
+        print(tag, flush=True)
+        q, k, v, do = orc.make_qkv(it * 3 + 5, 1, 2, Lq, Lk, dk, dv, dt)
+        scale = 1 / math.sqrt(dk)
+        o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), causal, scale)
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        o = fa.attention(qg, kg, vg, causal, scale)
+        o.backward(do.cuda())
+        _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
+
+
+def test_random_image_layout_cases():
+    from dl_templates_amd import tiled_swa as sw
+    rng = random.Random(4)
+    done = 0
+    while done < N_CASES:
+        bh, bw = rng.choice([(1, 1), (2, 2), (4, 4), (8, 2), (2, 8), (4, 8), (8, 8), (3, 5), (1, 16), (16, 2), (6, 8)])
+        S = bh * bw
+        th, tw = rng.randint(1, 10 if S < 16 else 6), rng.randint(1, 12 if S < 16 else 7)
+        WR, WC = rng.randint(0, 3), rng.randint(0, 3)
+        d = rng.choice([32, 64, 128])
+        dv = rng.choice([d, d, 128 if d == 64 else d])
+        dt = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+        B, H = rng.randint(1, 2), rng.randint(1, 3)
+        N = th * tw * S
+        if N > 3000 or (S == 1 and WR + WC == 0):   # self-only attention: dq = dk = 0, nothing to compare against
+            continue
+        pad = rng.choice([0, 0, 2])        # extra pixel columns in the allocation (cropped view)
+        packed = rng.random() < 0.5        # q, k, v as slices of one [.., 3, H, d] tensor (needs dk == dv)
+        if packed:
+            dv = d
+        done += 1
+        tag = f"case {done}: tile={bh}x{bw} grid={th}x{tw} W=({WR},{WC}) d={d}/{dv} {dt} B={B} H={H} pad={pad} packed={packed}"
+        print(tag, flush=True)
+        q, k, v, do = orc.make_qkv(done * 11 + 3, B, H, N, N, d, dv, dt)
+        scale = 1 / math.sqrt(d)
+        o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), S, th, tw, WR, WC, scale)
+        to_img = lambda t: orc.tokens_to_image(t, th, tw, bh, bw)
+        IH, IW = th * bh, tw * bw
+        if packed:
+            buf = torch.zeros((B, IH, IW + pad, 3, H, d), dtype=dt)
+            for j, t in enumerate((q, k, v)):
+                buf[:, :, :IW, j] = to_img(t)
+            buf = buf.cuda().requires_grad_(True)
+            qi, ki, vi = (buf[:, :, :IW, j] for j in range(3))
+        else:
+            leaves = []
+            for t, dd in ((q, d), (k, d), (v, dv)):
+                b_ = torch.zeros((B, IH, IW + pad, H, dd), dtype=dt)
+                b_[:, :, :IW] = to_img(t)
+                leaves.append(b_.cuda().requires_grad_(True))
+            qi, ki, vi = (b_[:, :, :IW] for b_ in leaves)
+        o = sw.TiledSwaImage.apply(qi, ki, vi, bh, bw, WR, WC, scale)
+        o.backward(to_img(do).cuda())
+        if packed:
+            grads = tuple(buf.grad[:, :, :IW, j] for j in range(3))
+        else:
+            grads = tuple(b_.grad[:, :, :IW] for b_ in leaves)
+        _check(tag, o, to_img(o_w), grads, (to_img(dq_w), to_img(dk_w), to_img(dv_w)))
+        if pad:
+            g_all = buf.grad if packed else leaves[0].grad
+            assert g_all[:, :, IW:].abs().max().item() == 0.0, tag

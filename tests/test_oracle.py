@@ -167,7 +167,7 @@ def test_rope_is_a_rotation_and_identity_on_nope():
     r, c = 3, 6
     n = r * 8 + c
     if idx[n] >= 0:
-        th = 10000.0 ** (-np.arange(R) / R)
+        th = 10000.0 ** (-2 * np.arange(R) / R)
         z = (x[0, n, :R].double().numpy() + 1j * x[0, n, R:2 * R].double().numpy()) * np.exp(1j * r * th)
         assert np.allclose(z.real, y[0, n, :R].numpy(), atol=1e-5) and np.allclose(z.imag, y[0, n, R:2 * R].numpy(), atol=1e-5)
         z = (x[0, n, 2 * R:3 * R].double().numpy() + 1j * x[0, n, 3 * R:4 * R].double().numpy()) * np.exp(1j * c * th)
@@ -182,6 +182,42 @@ def test_rope_backward_is_autograd_of_forward():
     do = torch.randn(2, 12, 16, generator=g)
     orc.rope2d_ref(x, idx, rcs, ccs).backward(do)
     assert torch.allclose(x.grad, orc.rope2d_bwd_ref(do, idx, rcs, ccs), atol=1e-6)
+
+
+def test_rope_tables_match_the_reference_self_test_construction():
+    """The only table construction in the reference is its self-test, src/fused_rope2d.py:236-246; it is typed
+    here as those lines have it (fp32 torch ops, base 1000, R = 8, 8 positions) and compared with the oracle's
+    generator and with the product's table holder.  A schedule of another form (exponent -i/R, another base, sin
+    and cos swapped, [R, len] instead of [len, R]) fails."""
+    from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
+    for n_rdim, n_max in ((8, 8), (4, 33), (16, 64)):
+        bases = torch.pow(1000, -2 * (torch.arange(n_rdim) / n_rdim))
+        indices = torch.arange(0, n_max)
+        cos_c = torch.cos(torch.outer(indices, bases))
+        sin_c = torch.sin(torch.outer(indices, bases))
+        literal = torch.dstack([cos_c, sin_c])
+        assert literal.shape == (n_max, n_rdim, 2)
+        mine = orc.rope_tables(n_rdim, n_max, base=1000.0)
+        prod = Ctx(2 * n_rdim, n_max, base=1000.0).cs_components
+        assert mine.shape == literal.shape and prod.shape == literal.shape and prod.dtype == torch.float32
+        # the literal expression forms its angles in fp32: half an ulp of the largest angle (< 64) is 4e-6
+        assert (mine - literal).abs().max().item() <= 8e-6
+        assert (prod - literal).abs().max().item() <= 8e-6
+        # oracle (complex exponential) and product (cos / sin), both from float64 angles, agree to an fp32 ulp
+        assert (mine - prod).abs().max().item() <= 1.2e-7
+        other_form = torch.cos(torch.outer(indices.double(), torch.pow(torch.tensor(1000.0, dtype=torch.float64), -(torch.arange(n_rdim) / n_rdim))))
+        assert (mine[..., 0].double() - other_form).abs().max().item() > 1e-2
+
+
+def test_rope_tables_identities():
+    # unit circle; position p is p steps of position 1 (angle addition); position 0 is the identity
+    t = orc.rope_tables(8, 40).double()
+    assert torch.allclose(t[..., 0] ** 2 + t[..., 1] ** 2, torch.ones(40, 8, dtype=torch.float64), atol=1e-6)
+    z = torch.complex(t[..., 0], t[..., 1])
+    assert torch.allclose(z[17] * z[5], z[22], atol=1e-6) and torch.allclose(z[1] ** 3, z[3], atol=1e-6)
+    # successive pairs slow down by the constant factor base ** (-2 / R)
+    ang = torch.atan2(t[1, :, 1], t[1, :, 0])
+    assert torch.allclose(ang[1:] / ang[:-1], torch.full((7,), 10000.0 ** (-2 / 8), dtype=torch.float64), rtol=1e-5)
 
 
 def test_rope_table_packing_and_golden():

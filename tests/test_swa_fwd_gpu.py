@@ -13,6 +13,7 @@ from oracle import attn_oracle as orc
 
 pytestmark = pytest.mark.gpu
 FWD_TOL = 2e-2
+LSE_TOL = 2e-2   # saved log-sum-exp, in log2 units
 
 
 def _swa():
@@ -26,15 +27,22 @@ def test_neighbor_sets_bit_exact(th, tw, wr, wc):
     assert np.array_equal(got, orc.neighbor_mask(th, tw, wr, wc))
 
 
-def _run(seed, B, H, b_size, th, tw, wr, wc, dk, dv, dtype, scale=None, check_lse=True):
+def _run(seed, B, H, b_size, th, tw, wr, wc, dk, dv, dtype, scale=None):
+    """o and the saved log-sum-exp lse2 (src/tiled_swa.py:129-133) of dlt_swa_fwd against the oracle."""
+    sw = _swa()
     N = b_size * th * tw
     q, k, v, _ = orc.make_qkv(seed, B, H, N, N, dk, dv, dtype)
     scale = 1.0 / math.sqrt(dk) if scale is None else scale
     want, lse_w = orc.tiled_swa_explicit(q.float(), k.float(), v.float(), b_size, th, tw, wr, wc, scale, return_lse2=True)
-    got = _swa().tiled_swa_fwd(q.cuda(), k.cuda(), v.cuda(), b_size, th, tw, wr, wc, scale)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    got, lse = sw._forward(qg, kg, vg, sw._shape(qg, kg, vg, b_size, th, tw, wr, wc, scale), None)
     assert got.dtype == dtype and got.shape == want.shape
     err = (got.float().cpu() - want).abs().max().item()
     assert err <= FWD_TOL, f"max abs err {err}"
+    assert lse.dtype == torch.float32 and lse.shape == lse_w.shape
+    lerr = (lse.cpu() - lse_w).abs().max().item()
+    assert lerr <= LSE_TOL, f"lse2 max abs err {lerr}"
+    assert torch.equal(sw.tiled_swa_fwd(qg, kg, vg, b_size, th, tw, wr, wc, scale), got)
     return err
 
 
@@ -116,12 +124,56 @@ def test_fused_rope_forward_equals_composition():
     assert torch.equal(comp, got)
 
 
+@pytest.mark.parametrize("d,R", [(64, 8), (128, 32), (128, 16)])
+def test_fused_rope_forward_lse_and_head_dim_fully_rotated(d, R):
+    """lse2 of the fused forward against the oracle's composition; (128, 32) rotates the whole head dim with
+    partners four 16-byte chunks apart (beyond one staging thread's piece)."""
+    from dl_templates_amd import fused_rope2d as fr
+    sw = _swa()
+    B, H, th, tw, W = 1, 2, 12, 20, 3
+    N = th * tw
+    q, k, v, _ = orc.make_qkv(80 + R, B, H, N, N, d, d, torch.bfloat16)
+    idx = orc.make_rope_idx(81, th, tw, 0.1)
+    rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+    scale = 1 / math.sqrt(d)
+    qr = orc.rope2d_ref(q.float().reshape(-1, N, d), idx, rcs, ccs).reshape(q.shape)
+    kr = orc.rope2d_ref(k.float().reshape(-1, N, d), idx, rcs, ccs).reshape(k.shape)
+    want, lse_w = orc.tiled_swa_explicit(qr, kr, v.float(), 1, th, tw, W, W, scale, return_lse2=True)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    rope = (idx.cuda(), rcs.cuda(), ccs.cuda())
+    shape = sw._shape(qg, kg, vg, 1, th, tw, W, W, scale)
+    q2, k2 = fr.rope2d_qk_(qg.clone(), kg.clone(), *rope)
+    comp, lse_c = sw._forward(q2, k2, vg, shape, None)
+    for which, (o, lse) in enumerate((sw._forward(qg, kg, vg, shape, rope), sw._forward_rot(qg, kg, vg, shape, rope)[:2])):
+        assert (o.float().cpu() - want).abs().max().item() <= FWD_TOL
+        assert (lse.cpu() - lse_w).abs().max().item() <= LSE_TOL
+        if not (R == 32 and which == 0):   # R = 32 rotating inside the tile loads: generic kernels, another summation order
+            assert torch.equal(o, comp) and torch.equal(lse, lse_c)
+
+
+@pytest.mark.parametrize("scale", [-0.125, 0.0])
+def test_zero_and_negative_scale(scale):
+    """The reference multiplies by sm_scale before taking the row max (src/tiled_swa.py:113-117), so any sign
+    works there; the kernels that keep the max of raw scores must not be chosen for these calls."""
+    sw = _swa()
+    q, k, v, _ = orc.make_qkv(90, 1, 2, 16 * 16, 16 * 16, 64, 64, torch.bfloat16)
+    want, lse_w = orc.tiled_swa_explicit(q.float(), k.float(), v.float(), 1, 16, 16, 3, 3, scale, return_lse2=True)
+    qg, kg, vg = q.cuda(), k.cuda(), v.cuda()
+    got, lse = sw._forward(qg, kg, vg, sw._shape(qg, kg, vg, 1, 16, 16, 3, 3, scale), None)
+    assert torch.isfinite(got.float()).all()
+    assert (got.float().cpu() - want).abs().max().item() <= FWD_TOL
+    assert (lse.cpu() - lse_w).abs().max().item() <= LSE_TOL
+    from dl_templates_amd._lib import DltError
+    with pytest.raises(DltError):
+        sw.tiled_swa_fwd(qg, kg, vg, 1, 16, 16, 3, 3, float("nan"))
+
+
 def test_bad_arguments_raise():
     sw = _swa()
     q = torch.randn(1, 1, 16, 64, dtype=torch.bfloat16).cuda()
     with pytest.raises(AssertionError):
         sw.tiled_swa_fwd(q, q, q, 1, 4, 5, 1, 1, 1.0)
-    big = torch.randn(1, 1, 16, 256, dtype=torch.bfloat16).cuda()
+    big = torch.randn(1, 1, 16, 512, dtype=torch.bfloat16).cuda()
     from dl_templates_amd._lib import DltError
     with pytest.raises(DltError):
         sw.tiled_swa_fwd(big, big, big, 1, 4, 4, 1, 1, 1.0)
