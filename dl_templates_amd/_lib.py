@@ -27,7 +27,9 @@ EXPORTS = (
     "dlt_swa_fwd", "dlt_swa_bwd", "dlt_swa_neighbors", "dlt_flash_fwd", "dlt_flash_bwd",
     "dlt_timing_enable", "dlt_timing_collect", "dlt_debug_copy",
     "dlt_swa_fwd_image", "dlt_swa_bwd_image", "dlt_swa_image_offsets", "dlt_swa_fwd_rot", "dlt_swa_bwd_rot",
+    "dlt_swa_bwd_noalloc",
 )
+NOALLOC_MAX_DELTA = 1 << 20  # DLT_NOALLOC_MAX_DELTA of include/dlt.h
 KERNEL_NAMES = ("rope2d", "attn_fwd", "attn_delta", "attn_bwd_kv", "attn_bwd_q")
 
 
@@ -106,6 +108,9 @@ def _declare(lib) -> None:
     lib.dlt_swa_fwd.argtypes = fwd + [POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
     lib.dlt_swa_bwd.restype = c_int
     lib.dlt_swa_bwd.argtypes = bwd + [POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
+    lib.dlt_swa_bwd_noalloc.restype = c_int
+    lib.dlt_swa_bwd_noalloc.argtypes = [c_void_p, P64] * 5 + [c_void_p, P64] + [c_void_p, P64] * 3 + [
+        POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
     lib.dlt_swa_fwd_rot.restype = c_int
     lib.dlt_swa_fwd_rot.argtypes = fwd + [c_void_p, P64, c_void_p, P64, POINTER(SwaShape), POINTER(RopeDesc), c_void_p]
     lib.dlt_swa_bwd_rot.restype = c_int

@@ -16,6 +16,7 @@ int dlt_set_error(int code, const char* fmt, ...) {
 
 // ---- per-kernel timing ------------------------------------------------------------------
 #include <vector>
+#include <mutex>
 namespace {
 struct TimedLaunch { int kernel; hipEvent_t e0, e1; };
 thread_local bool g_timing = false;
@@ -280,6 +281,63 @@ extern "C" int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void
   if (rc != DLT_OK) return rc;
   AttnTensors t;
   rc = fill_bwd("swa_bwd", t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, d_o, do_strides, lse2, delta,
+                lse_strides, dq, dq_strides, dk, dk_strides, dv, dv_strides);
+  if (rc != DLT_OK) return rc;
+  return dlt_attn_backward(p, t, (hipStream_t)stream);
+}
+
+// ---- backward without a caller-provided scratch buffer ------------------------------------------
+// The array's name is a host-side stand-in, not a device address: host code uses the pointer that
+// hipGetSymbolAddress returns for the current device (each GPU holds its own copy at its own address).
+static __device__ __align__(256) float g_delta_scratch[DLT_NOALLOC_MAX_DELTA];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[MAX_DEVICES] = {};
+
+// device address of the scratch array on the CURRENT device, looked up once per device
+int delta_scratch(const char* who, float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(e));
+  if (dev < 0 || dev >= MAX_DEVICES) return dlt_set_error(DLT_ERR_UNSUPPORTED, "%s: device %d is out of range", who, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_delta_scratch));
+    if (e != hipSuccess || p == nullptr)
+      return dlt_set_error(DLT_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) on device %d: %s", who, dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = static_cast<float*>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return DLT_OK;
+}
+}  // namespace
+
+extern "C" int dlt_swa_bwd_noalloc(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                                   const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],
+                                   const void* d_o, const int64_t do_strides[4],
+                                   const float* lse2, const int64_t lse_strides[3],
+                                   void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                                   void* dv, const int64_t dv_strides[4],
+                                   const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream) {
+  const char* who = "swa_bwd_noalloc";
+  AttnProblem p;
+  int rc = swa_problem(who, shape, rope, p);
+  if (rc != DLT_OK) return rc;
+  DLT_REQUIRE(lse_strides != nullptr, "%s: lse_strides is NULL", who);
+  DLT_REQUIRE(lse_strides[0] >= 0 && lse_strides[1] >= 0 && lse_strides[2] >= 0, "%s: negative lse2 stride", who);
+  const int64_t n_tok = (int64_t)shape->t_height * shape->t_width * shape->b_size;
+  const int64_t last = (shape->B - 1) * lse_strides[0] + (shape->H - 1) * lse_strides[1] + (n_tok - 1) * lse_strides[2];
+  DLT_REQUIRE(last < DLT_NOALLOC_MAX_DELTA,
+              "%s: the scratch for delta holds %d floats, this call needs %lld (B * H * N with the strides of lse2); "
+              "use dlt_swa_bwd with a caller-provided buffer", who, DLT_NOALLOC_MAX_DELTA, (long long)(last + 1));
+  float* delta = nullptr;
+  rc = delta_scratch(who, &delta);
+  if (rc != DLT_OK) return rc;
+  AttnTensors t;
+  rc = fill_bwd(who, t, q, q_strides, k, k_strides, v, v_strides, o, o_strides, d_o, do_strides, lse2, delta,
                 lse_strides, dq, dq_strides, dk, dk_strides, dv, dv_strides);
   if (rc != DLT_OK) return rc;
   return dlt_attn_backward(p, t, (hipStream_t)stream);

@@ -111,6 +111,25 @@ int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void* k, const 
                 void* dv, const int64_t dv_strides[4],
                 const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream);
 
+/* dlt_swa_bwd without the `delta` argument: the fp32 scratch lives in a buffer inside the library
+ * (one static device array per GPU, DLT_NOALLOC_MAX_DELTA floats = 4 MiB, held until the process
+ * ends) and the call allocates nothing: no hipMalloc / hipFree, no allocating library routine.
+ * No counterpart in the reference (TiledSwa.backward allocates delta with torch, src/tiled_swa.py:663);
+ * it is for callers that cannot allocate: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  The scratch is addressed with `lse_strides`, so the call is
+ * rejected (DLT_ERR_INVALID, nothing launched) when a stride is negative or the largest offset
+ * (B-1) s0 + (H-1) s1 + (N-1) s2 reaches DLT_NOALLOC_MAX_DELTA.  Every call on a GPU shares that GPU's
+ * buffer and overwrites all of it that it reads: calls that overlap in time on one GPU (two streams,
+ * two threads) race and must be serialised by the caller; results equal dlt_swa_bwd's bit for bit. */
+#define DLT_NOALLOC_MAX_DELTA (1 << 20)
+int dlt_swa_bwd_noalloc(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
+                        const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],
+                        const void* d_o, const int64_t do_strides[4],
+                        const float* lse2, const int64_t lse_strides[3],
+                        void* dq, const int64_t dq_strides[4], void* dk, const int64_t dk_strides[4],
+                        void* dv, const int64_t dv_strides[4],
+                        const dlt_swa_shape_t* shape, const dlt_rope_t* rope, void* stream);
+
 /* The fused call with the rotated tensors kept: forward as dlt_swa_fwd with `rope`, which in addition
  * stores the rotated q and k into q_rot / k_rot (shapes and element type of q / k, own strides; must
  * not alias q, k or each other).  These are the tensors RotaryPE2D leaves behind in the reference's
