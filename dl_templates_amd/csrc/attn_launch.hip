@@ -5,6 +5,8 @@
 #include "swa1_fwd_kernel.hpp"
 #include "swa1_bwd_kernel.hpp"
 #include "flash_kernel.hpp"
+#include "swam_bwd_kernel.hpp"
+#include <stdlib.h>
 
 int dlt_launch_fwd_32_32(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_64_64(const FwdArgs&, int, int, hipStream_t);
@@ -35,6 +37,8 @@ int dlt_swa1_launch_bwd_64(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
 int dlt_swa1_launch_bwd_128(const Swa1BwdArgs&, int, int, int, int, hipStream_t);
 int dlt_swa1_launch_fwd_64(const Swa1FwdArgs&, int, int, hipStream_t);
 int dlt_swa1_launch_fwd_128(const Swa1FwdArgs&, int, int, hipStream_t);
+int dlt_swam_launch_fwd(const SwamFwdArgs&, int, int, hipStream_t);
+int dlt_swam_launch_bwd(const SwamBwdArgs&, int, int, hipStream_t);
 
 namespace {
 
@@ -241,6 +245,72 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
                    : dlt_swa1_launch_fwd_128(a, c.wclass, (int)grid, stream);
 }
 
+// ---- marching token-grid kernels: head dim 64 exactly, windows up to 13 x 13, no rotation or R = 8 ----------
+constexpr int GPU_CUS = 256;   // MI355X
+
+bool swam_eligible(const AttnProblem& p, const Swa1Class& c) {
+  static const bool off = getenv("DLT_NO_MARCH") != nullptr;
+  if (off) return false;
+  if (c.D != 64 || p.dk != 64 || p.dv != 64) return false;
+  if (p.g.WR > 6 || p.g.WC > 6) return false;
+  if (c.rope_mode != 0 && !(c.rope_mode == 2 && p.rope.R == 8)) return false;
+  return true;
+}
+
+// rows per workgroup: the longest band (fewest re-fetched halo rows) that still gives every CU a workgroup
+void swam_make_plan(const AttnProblem& p, SwamPlan& plan) {
+  plan.nstrips = (p.g.TC + 15) / 16;
+  const int steps = (p.g.TR + 7) / 8;
+  const int64_t cols = (int64_t)p.B * p.H * plan.nstrips;
+  int ns = 1;
+  for (int cand = 2; cand <= 8 && cand <= steps; cand++)
+    if (cols * ((steps + cand - 1) / cand) >= GPU_CUS) ns = cand;
+  plan.band = 8 * ns;
+  plan.nbands = (steps + ns - 1) / ns;
+  dlt_fastdiv_make((uint32_t)(plan.nbands * plan.nstrips), plan.m_bh, plan.s_bh);
+  dlt_fastdiv_make((uint32_t)plan.nstrips, plan.m_st, plan.s_st);
+  dlt_fastdiv_make((uint32_t)p.H, plan.m_h, plan.s_h);
+}
+
+int swam_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c, hipStream_t stream) {
+  SwamFwdArgs a;
+  a.p = p;
+  swam_make_plan(p, a.plan);
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
+  for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.q_rot = c.rope_mode != 0 ? t.q_rot : nullptr;
+  a.k_rot = c.rope_mode != 0 ? t.k_rot : nullptr;
+  for (int i = 0; i < 4; i++) { a.qrs[i] = t.qrs[i]; a.krs[i] = t.krs[i]; }
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  const int64_t grid = (int64_t)p.B * p.H * a.plan.nbands * a.plan.nstrips;
+  if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: grid too large");
+  return dlt_swam_launch_fwd(a, c.rope_mode != 0, (int)grid, stream);
+}
+
+// backward on the marching kernels: plain inputs, or rotated inputs with the gradients rotated back on store
+int swam_backward(const AttnProblem& p, const AttnTensors& t, bool rot, hipStream_t stream) {
+  SwamBwdArgs a;
+  a.p = p;
+  swam_make_plan(p, a.plan);
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.o; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
+  for (int i = 0; i < 4; i++) {
+    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; a.dos[i] = t.dos[i];
+    a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
+  }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  const int64_t grid = (int64_t)p.B * p.H * a.plan.nbands * a.plan.nstrips;
+  if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward: grid too large");
+  return dlt_swam_launch_bwd(a, rot, (int)grid, stream);
+}
+
+// 16-byte row pieces and 32-bit byte offsets inside a (batch, head) slab of head dim 64
+bool swam_rows_ok(const AttnProblem& p, const void* ptr, const int64_t* st) {
+  return tvec_ok(ptr, st, 64, 2) && st[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * st[2] * 2 + 128 <= (((int64_t)1 << 31) - 1);
+}
+
 // ---- flash fast path: dense, causal, and sliding windows over tiles of 16 k tokens -----------
 // needs 2-byte elements, 16-byte vector access to q, k, v and 32-bit byte offsets inside a slab;
 // tile mode takes no fused rotation (those calls use the generic kernels)
@@ -363,6 +433,10 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
       const bool side_ok = t.q_rot == nullptr || (c.rope_mode != 0 && tvec_ok(t.q_rot, t.qrs, p.dk, es) &&
                                                   tvec_ok(t.k_rot, t.krs, p.dk, es));
       if (side_ok) {
+        // the marching kernels store o in 16-byte pieces and address every tensor with 32-bit offsets
+        const bool rows_fit = swam_rows_ok(p, t.out_o, t.os) &&
+                              (t.q_rot == nullptr || (swam_rows_ok(p, t.q_rot, t.qrs) && swam_rows_ok(p, t.k_rot, t.krs)));
+        if (swam_eligible(p, c) && rows_fit) return swam_forward(p, t, c, stream);
         rc = swa1_forward(p, t, c, stream);
         if (rc != -1) return rc;
       }
@@ -419,7 +493,15 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
     const bool streamed[4] = {tvec_ok(t.q, t.qs, p.dk, es), tvec_ok(t.k, t.ks, p.dk, es),
                               tvec_ok(t.v, t.vs, p.dv, es), tvec_ok(t.d_o, t.dos, p.dv, es)};
     Swa1Class c;
-    if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(p, t)) return swa1_backward(p, t, c, stream);
+    if (swa1_eligible(p, streamed, 4, c) && swa1_strides_fit(p, t)) {
+      Swa1Class cm = c;
+      if (p.rope_prerot && cm.rope_mode != 0) cm.rope_mode = 2;   // the marching kernels rotate dq / dk back on store
+      const bool plain_or_prerot = c.rope_mode == 0 || p.rope_prerot;
+      if (plain_or_prerot && swam_eligible(p, cm) && swam_rows_ok(p, t.o, t.os) && swam_rows_ok(p, t.dq, t.dqs) &&
+          swam_rows_ok(p, t.dk, t.dks) && swam_rows_ok(p, t.dv, t.dvs))
+        return swam_backward(p, t, c.rope_mode != 0, stream);
+      return swa1_backward(p, t, c, stream);
+    }
   }
   if (p.rope_prerot && p.rope.enabled && p.rope.R > 0 && !p.tm.img) {
     // rotated q, k and no token-grid kernel: the plain operator (any kernel family) yields the gradients of the
