@@ -11,7 +11,9 @@ store them (dlt_swa_fwd_rot / dlt_swa_bwd_rot).  `value` is the effective TFLOP/
 step (in-window FLOPs only: fwd 2*pairs*(dk+dv), bwd 2*pairs*(3dk+2dv)).  The JSON line also
 carries the roofline of the dominant kernel (per-kernel HIP-event durations taken inside the
 timed steps), the standalone RoPE-2D bandwidth (config 2), configs 4 / 5 as extras, and a CPU
-baseline: the eager-PyTorch oracle of the same step timed on the host cores.
+baseline: the eager-PyTorch oracle of the same step timed on the host cores, whose outputs also check the GPU
+results of the same seeded inputs (`accuracy`).  `ms_per_step` is the median of 5 repeats of >= 100 back-to-back
+steps whatever --steps says (the mean over the requested steps is reported in `extra`).
 
 Only one GPU is used; --gpus N with N > 1 exits with a message.
 """
@@ -70,6 +72,16 @@ class Timer:
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return e0.elapsed_time(e1) / steps, wall
+
+
+def median_of_repeats(fn, launches=100, repeats=5, warmup=10):
+    """Median (and all samples) of `repeats` timings of `launches` back-to-back repetitions each."""
+    samples = []
+    for i in range(repeats):
+        ms, _ = Timer.run(fn, launches, warmup if i == 0 else 0)
+        samples.append(ms)
+    srt = sorted(samples)
+    return srt[len(srt) // 2], samples
 
 
 def kernel_breakdown(fn, steps):
@@ -281,25 +293,87 @@ def bench_rope(steps, warmup):
 
 
 # ------------------------------------------------------------------------------------------ CPU baseline
-def cpu_baseline_c3():
-    """The oracle (eager PyTorch, fp32) of the same fused step on the host cores: one repetition of
-    the whole config-3 step after one warm-up on a quarter of the heads."""
+def gpu_results_for_accuracy():
+    """GPU outputs the CPU-baseline leg checks: the fused config-3 step on the inputs of seed 0 (the same draws
+    make_qkv(0, ...) yields on the host), config-2 rotation of a seeded tensor, neighbour sets and no-PE masks."""
+    from dl_templates_amd import fused_rope2d, tiled_swa
+    from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
+    from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as Rope
+    dev = torch.device("cuda:0")
+    B, H, th, tw, W, d = 2, 8, 64, 64, 6, 64
+    N = th * tw
+    q, k, v, do = make_inputs(0, B, H, N, N, d, d, torch.bfloat16, dev)
+    g = torch.Generator().manual_seed(1000)
+    idx = Rope.encode_idx(th, tw).clone()
+    idx[torch.rand(N, generator=g) < 0.05] = -1
+    rcs, ccs = Ctx(16, th).cs_components.to(dev), Ctx(16, tw).cs_components.to(dev)
+    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+    o = tiled_swa.TiledSwaRope.apply(qg, kg, vg, idx.to(dev), rcs, ccs, 1, th, tw, W, W, 1.0 / math.sqrt(d))
+    o.backward(do)
+    out = {"idx": idx, "o": o.detach().float().cpu(), "dq": qg.grad.float().cpu(), "dk": kg.grad.float().cpu(),
+           "dv": vg.grad.float().cpu()}
+    # config 2: B=4, H=8 -> 32 batch rows, 64 x 64 tokens, C = 64, R = 8, 5 % no-PE
+    g2 = torch.Generator().manual_seed(2)
+    idx2 = Rope.encode_idx(64, 64).clone()
+    idx2[torch.rand(N, generator=g2) < 0.05] = -1
+    x = torch.randn(32, N, 64, generator=g2).to(torch.bfloat16)
+    xr = fused_rope2d.RotaryPE2D.apply(x.to(dev).clone(), idx2.to(dev), rcs, ccs)
+    out.update({"idx2": idx2, "x": x, "x_rot": xr.cpu(), "rcs": rcs.cpu(), "ccs": ccs.cpu()})
+    out["neighbors"] = tiled_swa.swa_neighbors(16, 16, 3, 3).cpu().numpy()
+    from dl_templates_amd import _lib
+    bits = torch.empty(N, dtype=torch.uint8, device=dev)
+    _lib.check(_lib.load().dlt_rope_pe_mask(_lib.ptr(idx2.to(dev)), N, _lib.ptr(bits), _lib.stream_of(bits)))
+    out["pe_bits"] = bits.cpu().numpy()
+    return out
+
+
+def cpu_baseline_c3(gpu):
+    """The CPU leg: the oracle (eager PyTorch, fp32) of the same fused config-3 step on the host cores, three
+    repetitions after a warm-up on a quarter of the heads; its outputs then serve as the checker for the GPU
+    results of the same seeded inputs (`gpu`, from gpu_results_for_accuracy): returns (cpu_baseline, accuracy)."""
+    import numpy as np
     from oracle import attn_oracle as orc
     B, H, th, tw, W, d = 2, 8, 64, 64, 6, 64
     N = th * tw
-    q, k, v, do = orc.make_qkv(0, B, H, N, N, d, d, torch.float32)
-    idx = orc.make_rope_idx(1000, th, tw, 0.05)
+    q, k, v, do = orc.make_qkv(0, B, H, N, N, d, d, torch.bfloat16)
+    q, k, v, do = (t.float() for t in (q, k, v, do))
+    idx = gpu["idx"]
     rcs, ccs = orc.rope_tables(8, th), orc.rope_tables(8, tw)
     args = (idx, rcs, ccs, 1, th, tw, W, W, 1.0 / math.sqrt(d))
     orc.rope_swa_grads(q[:, :2], k[:, :2], v[:, :2], do[:, :2], *args)
-    t0 = time.perf_counter()
-    orc.rope_swa_grads(q, k, v, do, *args)
-    dt = time.perf_counter() - t0
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q, k, v, do, *args)
+        times.append(time.perf_counter() - t0)
+    dt = sorted(times)[1]
     pairs = swa_pairs(B, H, 1, th, tw, W, W)
     flops = 2 * pairs * (d + d) + 2 * pairs * (5 * d)
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"whole config-3 step (B=2,H=8,64x64,d=64,13x13, fp32 eager masked SDPA + autograd), 1 repetition, {dt * 1e3:.0f} ms",
-            "ms_per_step": dt * 1e3, "host_cpus": os.cpu_count()}
+    cpu = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"whole config-3 step (B=2,H=8,64x64,d=64,13x13, fp32 eager masked SDPA + autograd), median of 3 repetitions "
+                     f"({', '.join(f'{t * 1e3:.0f}' for t in times)} ms)",
+           "ms_per_step": dt * 1e3, "host_cpus": os.cpu_count()}
+
+    def rel(got, want):
+        return ((got - want).abs().max() / want.abs().max()).item()
+
+    def frob(got, want):
+        return ((got - want).norm() / want.norm()).item()
+
+    y = orc.rope2d_ref(gpu["x"].float(), gpu["idx2"], gpu["rcs"], gpu["ccs"]).to(torch.bfloat16)
+    acc = {
+        "workload": "config 3 fused step on the inputs of seed 0 (B=2, H=8: all of it), config 2 rotation, 16x16 grid 7x7 window "
+                    "neighbour sets, config 2 no-PE mask; checked against the CPU oracle outside the timed region",
+        "fwd_max_abs": (gpu["o"] - o_w).abs().max().item(), "fwd_max_abs_bar": 2e-2,
+        "dq_rel": rel(gpu["dq"], dq_w), "dk_rel": rel(gpu["dk"], dk_w), "dv_rel": rel(gpu["dv"], dv_w), "grad_rel_bar": 5e-2,
+        "dq_frobenius_rel": frob(gpu["dq"], dq_w), "dk_frobenius_rel": frob(gpu["dk"], dk_w), "dv_frobenius_rel": frob(gpu["dv"], dv_w),
+        "rope_max_bf16_ulp": int(orc.bf16_ulp_diff(gpu["x_rot"], y).max()), "rope_ulp_bar": 1,
+        "neighbor_sets_bit_exact": bool(np.array_equal(gpu["neighbors"], orc.neighbor_mask(16, 16, 3, 3))),
+        "no_pe_mask_bit_exact": bool(np.array_equal(gpu["pe_bits"], orc.pe_mask(gpu["idx2"].numpy()))),
+    }
+    acc["within_bars"] = bool(acc["fwd_max_abs"] <= 2e-2 and max(acc["dq_rel"], acc["dk_rel"], acc["dv_rel"]) <= 5e-2 and
+                              acc["rope_max_bf16_ulp"] <= 1 and acc["neighbor_sets_bit_exact"] and acc["no_pe_mask_bit_exact"])
+    return cpu, acc
 
 
 def calibration_copy():
@@ -327,7 +401,9 @@ def copy_bandwidth():
         st = _lib.stream_of(a)
         fn = lambda: _lib.check(lib.dlt_debug_copy(_lib.ptr(b), _lib.ptr(a), nbytes, st))
         ms, _ = Timer.run(fn, reps, 2)
-        out[name] = {"ms": ms, "gbps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9}
+        ms_t, _ = Timer.run(lambda: b.copy_(a), reps, 2)   # PyTorch's own device copy: an independent yardstick
+        out[name] = {"ms": ms, "gbps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9,
+                     "torch_copy_ms": ms_t, "torch_copy_gbps_read_plus_write": 2 * nbytes / (ms_t * 1e-3) / 1e9}
         del a, b
     # a copy with the real traffic of one RoPE C2 launch (about 48 MiB), cold: 13 buffer pairs cycled (624 MiB)
     nbytes, npairs = 24 << 20, 13
@@ -342,7 +418,15 @@ def copy_bandwidth():
         _lib.check(lib.dlt_debug_copy(_lib.ptr(b), _lib.ptr(a), nbytes, st))
 
     ms, _ = Timer.run(cold, 5 * npairs, npairs)
-    out["24MiB_cold"] = {"ms": ms, "gbps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9}
+
+    def cold_torch():
+        a, b = bufs[state["i"] % npairs]
+        state["i"] += 1
+        b.copy_(a)
+
+    ms_t, _ = Timer.run(cold_torch, 5 * npairs, npairs)
+    out["24MiB_cold"] = {"ms": ms, "gbps_read_plus_write": 2 * nbytes / (ms * 1e-3) / 1e9,
+                         "torch_copy_ms": ms_t, "torch_copy_gbps_read_plus_write": 2 * nbytes / (ms_t * 1e-3) / 1e9}
     return out
 
 
@@ -409,10 +493,12 @@ def main():
     # ---- main workload: config 3, fused RoPE, 4 input sets cycled (about 400 MB touched per cycle)
     wl = SwaWorkload("C3", 2, 8, 64, 64, 6, 64, fused_rope=True, nsets=4)
     ms_eager, wall_eager = Timer.run(wl.step, K, W)
-    kb = kernel_breakdown(wl.step, K)
+    kb = kernel_breakdown(wl.step, max(K, 20))
     ms_graph = try_graph(wl, K, W)
-    # the same K steps were run twice, as eager launches and replayed from a HIP graph: the faster one counts
-    ms_step = min(ms_graph, ms_eager) if ms_graph is not None else ms_eager
+    # headline: median of 5 repeats of >= 100 back-to-back steps (eager launches), whatever --steps says; the mean over the
+    # K requested steps and the HIP-graph replay of the same steps are reported beside it
+    ms_median, ms_samples = median_of_repeats(wl.step, launches=max(100, K), repeats=5, warmup=W)
+    ms_step = ms_median
     flops_step = wl.flops_fwd + wl.flops_bwd
     value = flops_step / (ms_step * 1e-3) / 1e12
 
@@ -421,6 +507,7 @@ def main():
     ach = kflops[dom] / (kb[dom]["avg_ms"] * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": dom, "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": ach / PEAK_BF16_TFLOPS, "traffic": recorded_traffic(dom),
+                "traffic_source": "recorded in profiles/c3_kernels_hbm_traffic.json (rocprofv3 --pmc runs of this script), not measured by this run",
                 "avg_launch_ms": kb[dom]["avg_ms"], "alg_flops_per_launch": kflops[dom]}
     kernels = {}
     for k_, v_ in kb.items():
@@ -429,8 +516,9 @@ def main():
             kernels[k_]["eff_tflops"] = kflops[k_] / (v_["avg_ms"] * 1e-3) / 1e12
             kernels[k_]["frac_mfma_peak"] = kernels[k_]["eff_tflops"] / PEAK_BF16_TFLOPS
 
-    extra = {"ms_per_step_eager_events": ms_eager, "ms_per_step_eager_wall": wall_eager, "ms_per_step_graph": ms_graph,
-             "step_source": "hip graph replay" if ms_graph is not None and ms_graph <= ms_eager else "eager launches",
+    extra = {"ms_per_step_mean_of_requested_steps": ms_eager, "ms_per_step_eager_wall": wall_eager, "ms_per_step_graph": ms_graph,
+             "ms_per_step_median_of_5x100": ms_median, "ms_per_step_samples_5x100": ms_samples,
+             "step_source": "median of 5 repeats of >= 100 eager back-to-back steps",
              "frac_mfma_peak_effective": value / PEAK_BF16_TFLOPS, "kernels": kernels,
              "hbm_floor_ms": 101e6 / (PEAK_HBM_GBPS * 1e9) * 1e3}
 
@@ -499,7 +587,7 @@ def main():
                              "kernels_ms": {k_: v_["avg_ms"] for k_, v_ in kb5.items()}}
         del w5
 
-    cpu = None if args.quick else cpu_baseline_c3()
+    cpu, accuracy = (None, None) if args.quick else cpu_baseline_c3(gpu_results_for_accuracy())
 
     line = {
         "metric": "swa2d_fwd_bwd_effective_tflops", "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": K,
@@ -508,7 +596,7 @@ def main():
         "config": {"workload": "C3: fused RoPE-2D + tiled 2D SWA fwd+bwd, B=2 H=8 64x64 grid b_size=1 d=64 13x13 window, "
                                "bf16, 5% no-PE tokens, 4 input sets cycled; rotated q, k kept by the forward pass for the backward pass",
                    "peak_bf16_tflops": PEAK_BF16_TFLOPS, "peak_hbm_gbps": PEAK_HBM_GBPS},
-        "roofline": roofline, "cpu_baseline": cpu,
+        "roofline": roofline, "cpu_baseline": cpu, "accuracy": accuracy,
         "rope2d_gbps": rope["cold"]["gbps"], "rope2d_frac_hbm": rope["cold"]["frac_of_hbm_peak"],
         "extra": extra,
     }

@@ -276,11 +276,12 @@ int rope_impl(void* const x[2], const int64_t* const st[2], const int64_t nb[2],
     if (nb[z] > maxb) maxb = nb[z];
   }
   if (N == 0 || maxb == 0 || a.r.R == 0) return DLT_OK;
-  // enough blocks to cover the chip several times over, few enough table reloads
   const int items = vec ? 2 * (a.r.R / 8) : 2 * a.r.R;
   const int64_t bx = ((int64_t)N * items + 255) / 256;
   int bb = (int)maxb;
-  while (bb > UNR && bx * ((maxb + bb - 1) / bb) * ntens < 2048) bb = (bb + 1) / 2;
+  // two workgroups per CU: measured optimum on the benchmark shape (a thread's token index -> table row chain is paid once
+  // per workgroup, so more, shorter workgroups re-read the tables more often: 1024 blocks +2 %, 2048 blocks +16 %, 256 +10 %)
+  while (bb > 1 && bx * ((maxb + bb - 1) / bb) * ntens < 512) bb = (bb + 1) / 2;
   a.bb = bb < 1 ? 1 : bb;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {

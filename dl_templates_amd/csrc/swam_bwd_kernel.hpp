@@ -130,11 +130,13 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
 #pragma unroll
     for (int c = 0; c < SWAM_NSLOT; c++) swam_issue(it[c], st, G, c, side[c & 1]);
     own_issue(cur, G.r0 + 4 * rg);
+    // chunk by chunk (loads return in order): the LDS writes of a chunk overlap the arrival of the later ones
 #pragma unroll
-    for (int c = 0; c < SWAM_NSLOT; c++) swam_pin(it[c]);
+    for (int c = 0; c < SWAM_NSLOT; c++) {
+      swam_pin(it[c]);
+      commit_chunk(it[c], c);
+    }
     own_pin(cur);
-#pragma unroll
-    for (int c = 0; c < SWAM_NSLOT; c++) commit_chunk(it[c], c);
     del_n = own_delta(cur);
   }
   __syncthreads();
@@ -344,12 +346,13 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
       if (kpar + 2 * i < SWAM_NSLOT) sc[i] = scalar_issue(kpar + 2 * i);
     own_issue(cur, G.r0 + 4 * rg);
 #pragma unroll
-    for (int c = 0; c < SWAM_NSLOT; c++) swam_pin(it[c]);
+    for (int c = 0; c < SWAM_NSLOT; c++) {
+      swam_pin(it[c]);
+      commit_chunk(it[c], c);
+    }
 #pragma unroll
     for (int i = 0; i < 3; i++) pin_loaded(sc[i]);
     own_pin(cur);
-#pragma unroll
-    for (int c = 0; c < SWAM_NSLOT; c++) commit_chunk(it[c], c);
 #pragma unroll
     for (int i = 0; i < 3; i++)
       if (kpar + 2 * i < SWAM_NSLOT) scalar_commit(sc[i], kpar + 2 * i);

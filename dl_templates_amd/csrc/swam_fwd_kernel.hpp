@@ -165,23 +165,40 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
         if (kpar + 2 * i < SWAM_NSLOT) swam_tab_issue(tb[i], idk[i], st.qd, rope);
       swam_tab_issue(tbq, idq, g >> 1, rope);
     }
+    if (!ROT) {
+      // chunk by chunk (loads return in order): the LDS writes of a chunk overlap the arrival of the later ones
 #pragma unroll
-    for (int c = 0; c < SWAM_NSLOT; c++) swam_pin(it[c]);
-    swam_own_pin(qo, ROT);
+      for (int c = 0; c < SWAM_NSLOT; c++) {
+        swam_pin(it[c]);
+        commit_chunk(it[c], c);
+      }
+    }
     if (ROT) {
-      // static register indexing: the K items of this half are chunks kpar, kpar + 2, kpar + 4
+      // V chunks need no rotation and are written as they arrive; the K chunks wait for their table rows, which were
+      // requested last (static register indexing: the K items of this half are chunks kpar, kpar + 2, kpar + 4)
       if (kpar == 0) {
-        rotate_k(it[0], tb[0]);
-        rotate_k(it[2], tb[1]);
-        rotate_k(it[4], tb[2]);
+        swam_pin(it[1]); commit_chunk(it[1], 1);
+        swam_pin(it[3]); commit_chunk(it[3], 3);
       } else {
-        rotate_k(it[1], tb[0]);
-        rotate_k(it[3], tb[1]);
+        swam_pin(it[0]); commit_chunk(it[0], 0);
+        swam_pin(it[2]); commit_chunk(it[2], 2);
+        swam_pin(it[4]); commit_chunk(it[4], 4);
+      }
+#pragma unroll
+      for (int c = 0; c < SWAM_NSLOT; c++) swam_pin(it[c]);
+      swam_own_pin(qo, ROT);
+      if (kpar == 0) {
+        rotate_k(it[0], tb[0]); commit_chunk(it[0], 0);
+        rotate_k(it[2], tb[1]); commit_chunk(it[2], 2);
+        rotate_k(it[4], tb[2]); commit_chunk(it[4], 4);
+      } else {
+        rotate_k(it[1], tb[0]); commit_chunk(it[1], 1);
+        rotate_k(it[3], tb[1]); commit_chunk(it[3], 3);
       }
       rotate_q(qo, tbq);
+    } else {
+      swam_own_pin(qo, ROT);
     }
-#pragma unroll
-    for (int c = 0; c < SWAM_NSLOT; c++) commit_chunk(it[c], c);
   }
   __syncthreads();
 
