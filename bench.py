@@ -478,6 +478,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="skip the extra configs and the CPU baseline")
+    ap.add_argument("--workload", choices=("all", "c4", "c4b", "c5"), default="all",
+                    help="c4 / c4b / c5: run only config 4 (128x128 / 96x160) or config 5 and print its timing (for profiler runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the hot path shards over batch*heads with no exchange); "
@@ -489,6 +491,20 @@ def main():
     torch.cuda.set_device(0)
     K, W = args.steps, args.warmup
     calibration_copy()
+    if args.workload != "all":
+        # one extra config alone, for rocprofv3 runs: the calibration copy above, then W + K steps
+        if args.workload == "c5":
+            w = FlashWorkload(2, 16, 4096, 8192, 64, 128)
+        else:
+            th, tw = (128, 128) if args.workload == "c4" else (96, 160)
+            w = SwaWorkload(args.workload, 1, 16, th, tw, 10, 128, fused_rope=False, nsets=1)
+        ms, _ = Timer.run(w.step, K, W)
+        kbw = kernel_breakdown(w.step, max(K // 2, 2))
+        fl = w.flops_fwd + w.flops_bwd
+        print(json.dumps({"workload": args.workload, "ms_per_step": ms, "eff_tflops": fl / (ms * 1e-3) / 1e12,
+                          "frac_mfma_peak": fl / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+                          "kernels_ms": {k_: v_["avg_ms"] for k_, v_ in kbw.items()}}))
+        return
 
     # ---- main workload: config 3, fused RoPE, 4 input sets cycled (about 400 MB touched per cycle)
     wl = SwaWorkload("C3", 2, 8, 64, 64, 6, 64, fused_rope=True, nsets=4)

@@ -58,14 +58,14 @@ constexpr int flash_ck_fwd(int dk, int dv) { return FLASH_CK_FWD(dk, dv); }
 constexpr int flash_ck_q(int dk, int dv) { return FLASH_CK_Q(dk, dv); }
 constexpr int flash_ck_kv(int dk, int dv) { return FLASH_CK_KV(dk, dv); }
 // key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
-constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 128 ? 1 : 2; }
+constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 192 ? 1 : 2; }
 // query blocks per wave in the dQ kernel: one at 128/128 (accumulators, q and dO fragments of two blocks do not fit 256 registers)
 constexpr int flash_np_q(int dk, int dv) { return dk + dv > 192 ? 1 : FLASH_NP_DEF; }
 // resident workgroups per CU the register allocation aims for (spill-free at these settings)
 constexpr int flash_occ_fwd(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 3 : 2); }
 constexpr int flash_occ_q(int dk, int dv) { return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 3 : 2); }
 constexpr int flash_occ_kv(int dk, int dv, int mode) {
-  return dk + dv <= 64 ? 4 : (dk + dv <= 128 ? 2 : (dk + dv <= 192 && mode < 2 ? 3 : 2));
+  return dk + dv <= 64 ? 4 : 2;
 }
 
 // One chunk of streamed tokens: first token (index inside the [N, D] slab), its x inside the grid
@@ -351,12 +351,13 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
 #pragma unroll
       for (int p = 0; p < NP; p++) {
         if (!any[p]) continue;
-        float mloc = -INFINITY;
+        // four independent chains, two new values per instruction (v_max3_f32)
+        float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++)
-          mloc = fmaxf(mloc, fmaxf(fmaxf(fmaxf(t[p][kb][0], t[p][kb][1]), fmaxf(t[p][kb][2], t[p][kb][3])),
-                                   fmaxf(fmaxf(t[p][kb][4], t[p][kb][5]), fmaxf(t[p][kb][6], t[p][kb][7]))));
-        mloc = wave_max4(mloc);
+#pragma unroll
+          for (int i = 0; i < 4; i++) mx[i] = fmaxf(fmaxf(mx[i], t[p][kb][2 * i]), t[p][kb][2 * i + 1]);
+        float mloc = wave_max4(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])));
         const float m_new = fmaxf(m_run[p], mloc);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a block that has seen no key yet
         const float alpha = fast_exp2((m_run[p] - m_use) * scale);
@@ -779,49 +780,45 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
         need = need || bv[p];
       }
       if (!need) continue;
-      u32x4 qa[2][KC], da[2][VC];
-      f32x4 lq[2], dl[2];
+      // the first products run over one 16-query half at a time (operands of a half: KC + VC vectors), the second
+      // products contract over the whole block
+      float pr[NP][8], ds[NP][8];
 #pragma unroll
       for (int mb = 0; mb < 2; mb++) {
+        u32x4 qa[KC], da[VC];
 #pragma unroll
-        for (int c_ = 0; c_ < KC; c_++) qa[mb][c_] = lds_read16(sQ + (32 * qb_ + 16 * mb + n) * PQ + (32 * c_ + 8 * g) * 2);
+        for (int c_ = 0; c_ < KC; c_++) qa[c_] = lds_read16(sQ + (32 * qb_ + 16 * mb + n) * PQ + (32 * c_ + 8 * g) * 2);
 #pragma unroll
-        for (int c_ = 0; c_ < VC; c_++) da[mb][c_] = lds_read16(sDO + (32 * qb_ + 16 * mb + n) * PD + (32 * c_ + 8 * g) * 2);
-        lq[mb] = *reinterpret_cast<const f32x4*>(sLse + 32 * qb_ + 16 * mb + 4 * g);
-        dl[mb] = *reinterpret_cast<const f32x4*>(sDel + 32 * qb_ + 16 * mb + 4 * g);
-      }
-      u32x4 pb[NP], dsb[NP];
+        for (int c_ = 0; c_ < VC; c_++) da[c_] = lds_read16(sDO + (32 * qb_ + 16 * mb + n) * PD + (32 * c_ + 8 * g) * 2);
+        const f32x4 lq = *reinterpret_cast<const f32x4*>(sLse + 32 * qb_ + 16 * mb + 4 * g);
+        const f32x4 dl = *reinterpret_cast<const f32x4*>(sDel + 32 * qb_ + 16 * mb + 4 * g);
 #pragma unroll
-      for (int p = 0; p < NP; p++) {
-        if (!bv[p]) continue;
-        f32x4 s[2], dp[2];
+        for (int p = 0; p < NP; p++) {
+          if (!bv[p]) continue;
+          f32x4 sv = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++) {
-          s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-          dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+          for (int c_ = 0; c_ < KC; c_++) sv = Mma<CT>::mfma(qa[c_], kf[p][c_], sv);
 #pragma unroll
-          for (int c_ = 0; c_ < KC; c_++) s[mb] = Mma<CT>::mfma(qa[mb][c_], kf[p][c_], s[mb]);
-#pragma unroll
-          for (int c_ = 0; c_ < VC; c_++) dp[mb] = Mma<CT>::mfma(da[mb][c_], vf[p][c_], dp[mb]);
-        }
-        float pr[8], ds[8];
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++) {
+          for (int c_ = 0; c_ < VC; c_++) dp = Mma<CT>::mfma(da[c_], vf[p][c_], dp);
           const bool hv = !TILE || (q0 + 32 * qb_ + 16 * mb >= vlo[p] && q0 + 32 * qb_ + 16 * mb < vhi[p]);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            float pv = fast_exp2(fmaf(s[mb][i], scale, -lq[mb][i]));
+            float pv = fast_exp2(fmaf(sv[i], scale, -lq[i]));
             if (tail) {
               const int qi = q0 + 32 * qb_ + 16 * mb + 4 * g + i;
               pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
             }
             if (TILE) pv = hv ? pv : 0.f;
-            pr[4 * mb + i] = pv;
-            ds[4 * mb + i] = pv * (dp[mb][i] - dl[mb][i]);
+            pr[p][4 * mb + i] = pv;
+            ds[p][4 * mb + i] = pv * (dp[i] - dl[i]);
           }
         }
-        pb[p] = pack8<CT>(pr);
-        dsb[p] = pack8<CT>(ds);
+      }
+      u32x4 pb[NP], dsb[NP];
+#pragma unroll
+      for (int p = 0; p < NP; p++) {
+        pb[p] = pack8<CT>(pr[p]);
+        dsb[p] = pack8<CT>(ds[p]);
       }
 #pragma unroll
       for (int d = 0; d < VB; d++) {
