@@ -104,15 +104,34 @@ DLT_DEV u32x4 lds_read_tokens_as_k(const char* tile, int pitch, int row0, int di
   return r;
 }
 
-DLT_DEV float wave_max4(float v) {  // max over the 4 lanes that share n (lane ^ 16, lane ^ 32)
-  v = fmaxf(v, __shfl_xor(v, 16));
-  v = fmaxf(v, __shfl_xor(v, 32));
-  return v;
+// Reductions over the 4 lanes that share n (lanes n, n + 16, n + 32, n + 48), every lane receiving the result.  The two
+// exchanges are lane-swap VALU instructions (rows 2,3 <-> rows 0,1, then odd rows <-> even rows), not LDS permutes:
+// those queue behind the operand reads of every wave on the CU.
+DLT_DEV void wave_rows_swap32(float v, float& a, float& b) {
+  typedef unsigned pair_t __attribute__((ext_vector_type(2)));
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  const pair_t r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  a = __builtin_bit_cast(float, (unsigned)r.x); b = __builtin_bit_cast(float, (unsigned)r.y);
+}
+DLT_DEV void wave_rows_swap16(float v, float& a, float& b) {
+  typedef unsigned pair_t __attribute__((ext_vector_type(2)));
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  const pair_t r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  a = __builtin_bit_cast(float, (unsigned)r.x); b = __builtin_bit_cast(float, (unsigned)r.y);
+}
+DLT_DEV float wave_max4(float v) {
+  float a, b;
+  wave_rows_swap32(v, a, b);
+  v = fmaxf(a, b);
+  wave_rows_swap16(v, a, b);
+  return fmaxf(a, b);
 }
 DLT_DEV float wave_sum4(float v) {
-  v += __shfl_xor(v, 16);
-  v += __shfl_xor(v, 32);
-  return v;
+  float a, b;
+  wave_rows_swap32(v, a, b);
+  v = a + b;
+  wave_rows_swap16(v, a, b);
+  return a + b;
 }
 
 // ---- global <-> register moves of 8 consecutive head dims -------------------------------

@@ -6,7 +6,7 @@
 #include "swa1_bwd_kernel.hpp"
 #include "flash_kernel.hpp"
 #include "swam_bwd_kernel.hpp"
-#include <stdlib.h>
+#include "swa2_bwd_kernel.hpp"
 
 int dlt_launch_fwd_32_32(const FwdArgs&, int, int, hipStream_t);
 int dlt_launch_fwd_64_64(const FwdArgs&, int, int, hipStream_t);
@@ -39,6 +39,8 @@ int dlt_swa1_launch_fwd_64(const Swa1FwdArgs&, int, int, hipStream_t);
 int dlt_swa1_launch_fwd_128(const Swa1FwdArgs&, int, int, hipStream_t);
 int dlt_swam_launch_fwd(const SwamFwdArgs&, int, int, hipStream_t);
 int dlt_swam_launch_bwd(const SwamBwdArgs&, int, int, hipStream_t);
+int dlt_swa2_launch_fwd(const Swa2FwdArgs&, int, hipStream_t);
+int dlt_swa2_launch_bwd(const Swa2BwdArgs&, int, hipStream_t);
 
 namespace {
 
@@ -249,8 +251,6 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
 constexpr int GPU_CUS = 256;   // MI355X
 
 bool swam_eligible(const AttnProblem& p, const Swa1Class& c) {
-  static const bool off = getenv("DLT_NO_MARCH") != nullptr;
-  if (off) return false;
   if (c.D != 64 || p.dk != 64 || p.dv != 64) return false;
   if (p.g.WR > 6 || p.g.WC > 6) return false;
   if (c.rope_mode != 0 && !(c.rope_mode == 2 && p.rope.R == 8)) return false;
@@ -286,6 +286,53 @@ int swam_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
   const int64_t grid = (int64_t)p.B * p.H * a.plan.nbands * a.plan.nstrips;
   if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: grid too large");
   return dlt_swam_launch_fwd(a, c.rope_mode != 0, (int)grid, stream);
+}
+
+// ---- streaming kernels for head dim 128 exactly, no rotation, windows up to 21 columns -------------------------------
+bool swa2_eligible(const AttnProblem& p, const Swa1Class& c) {
+  return c.D == 128 && p.dk == 128 && p.dv == 128 && c.rope_mode == 0 && p.g.WC <= 10;
+}
+
+void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan) {
+  plan.nblk_r = (p.g.TR + 7) / 8;
+  plan.nblk_c = (p.g.TC + 15) / 16;
+  dlt_fastdiv_make((uint32_t)(plan.nblk_r * plan.nblk_c), plan.m_bh, plan.s_bh);
+  dlt_fastdiv_make((uint32_t)plan.nblk_c, plan.m_c, plan.s_c);
+  dlt_fastdiv_make((uint32_t)p.H, plan.m_h, plan.s_h);
+}
+
+bool swa2_rows_ok(const AttnProblem& p, const void* ptr, const int64_t* st) {
+  return tvec_ok(ptr, st, 128, 2) && st[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * st[2] * 2 + 256 <= (((int64_t)1 << 31) - 1);
+}
+
+int swa2_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
+  Swa2FwdArgs a;
+  a.p = p;
+  swa2_make_plan(p, a.plan);
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
+  for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
+  if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: grid too large");
+  return dlt_swa2_launch_fwd(a, (int)grid, stream);
+}
+
+int swa2_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
+  Swa2BwdArgs a;
+  a.p = p;
+  swa2_make_plan(p, a.plan);
+  a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.o; a.d_o = t.d_o; a.lse = t.lse; a.delta = t.delta;
+  a.dq = t.dq; a.dk = t.dk; a.dv = t.dv;
+  for (int i = 0; i < 4; i++) {
+    a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; a.dos[i] = t.dos[i];
+    a.dqs[i] = t.dqs[i]; a.dks[i] = t.dks[i]; a.dvs[i] = t.dvs[i];
+  }
+  for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];
+  a.scale_log2 = p.sm_scale * 1.4426950408889634f;
+  const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
+  if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward: grid too large");
+  return dlt_swa2_launch_bwd(a, (int)grid, stream);
 }
 
 // backward on the marching kernels: plain inputs, or rotated inputs with the gradients rotated back on store
@@ -437,6 +484,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
         const bool rows_fit = swam_rows_ok(p, t.out_o, t.os) &&
                               (t.q_rot == nullptr || (swam_rows_ok(p, t.q_rot, t.qrs) && swam_rows_ok(p, t.k_rot, t.krs)));
         if (swam_eligible(p, c) && rows_fit) return swam_forward(p, t, c, stream);
+        if (swa2_eligible(p, c) && t.q_rot == nullptr && swa2_rows_ok(p, t.out_o, t.os)) return swa2_forward(p, t, stream);
         rc = swa1_forward(p, t, c, stream);
         if (rc != -1) return rc;
       }
@@ -500,6 +548,10 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
       if (plain_or_prerot && swam_eligible(p, cm) && swam_rows_ok(p, t.o, t.os) && swam_rows_ok(p, t.dq, t.dqs) &&
           swam_rows_ok(p, t.dk, t.dks) && swam_rows_ok(p, t.dv, t.dvs))
         return swam_backward(p, t, c.rope_mode != 0, stream);
+      // lse2 / delta rows are copied with 32-bit byte offsets inside a (batch, head) slab
+      if (swa2_eligible(p, c) && swa2_rows_ok(p, t.o, t.os) && swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) &&
+          swa2_rows_ok(p, t.dv, t.dvs) && t.ls[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * t.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1))
+        return swa2_backward(p, t, stream);
       return swa1_backward(p, t, c, stream);
     }
   }

@@ -413,7 +413,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   // ---- epilogue: normalise, O^T fragments -> LDS tile -> coalesced rows
 #pragma unroll
   for (int p = 0; p < NP; p++) {
-    const float lt = __shfl(acc_l[p][0], n);
+    const float lt = wave_sum4(acc_l[p][0]);   // only row 0 of the ones operand is set: the other lane groups hold zeros
     const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
     TL* orow = reinterpret_cast<TL*>(smem + (wave * 16 * NP + 16 * p + n) * PO);
 #pragma unroll

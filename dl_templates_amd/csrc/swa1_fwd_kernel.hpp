@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   typedef typename TileOf<TIO>::type TL;
   constexpr int PO = D * (int)sizeof(TL) + 16;
   // row 0 of the ones product lives in lane group 0; per-lane partial sums are added over the 4 groups
-  const float lt = ONES ? __shfl(acc_l[0], n) : wave_sum4(l_run);
+  const float lt = wave_sum4(ONES ? acc_l[0] : l_run);   // ones product: only lane group 0 is non-zero
   const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
   const int64_t tq = own_token(16 * wave + n);
   if (g == 0 && tq >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq * a.ls[2]] = m_run * scale + fast_log2(lt);

@@ -285,7 +285,7 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
       acc_l = Mma<CT>::mfma(ones, pb, acc_l);
     }
     // row 0 of the ones product (lane group 0) = sum over keys of P[key][query n]
-    const float lt = __shfl(acc_l[0], n);
+    const float lt = wave_sum4(acc_l[0]);   // only row 0 of the ones operand is set: the other lane groups hold zeros
     SwamFwdOut r;
 #pragma unroll
     for (int d = 0; d < 4; d++) r.acc[d] = acc[d];

@@ -147,7 +147,9 @@ def test_fused_rope_forward_lse_and_head_dim_fully_rotated(d, R):
     for which, (o, lse) in enumerate((sw._forward(qg, kg, vg, shape, rope), sw._forward_rot(qg, kg, vg, shape, rope)[:2])):
         assert (o.float().cpu() - want).abs().max().item() <= FWD_TOL
         assert (lse.cpu() - lse_w).abs().max().item() <= LSE_TOL
-        if not (R == 32 and which == 0):   # R = 32 rotating inside the tile loads: generic kernels, another summation order
+        # bit equality only where both runs use one kernel family: at head dim 128 the unrotated composition runs on the
+        # streaming kernels (another summation order and softmax reference), the fused rotation on the tile kernels
+        if d != 128:
             assert torch.equal(o, comp) and torch.equal(lse, lse_c)
 
 
