@@ -289,6 +289,26 @@ extern "C" int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void
 // ---- backward without a caller-provided scratch buffer ------------------------------------------
 // The array's name is a host-side stand-in, not a device address: host code uses the pointer that
 // hipGetSymbolAddress returns for the current device (each GPU holds its own copy at its own address).
+int dlt_ensure_lds(const void* kern, int bytes) {
+  if (bytes <= 48 * 1024) return DLT_OK;   // within the default limit
+  struct Entry { const void* kern; int dev; int bytes; };
+  static std::mutex mu;
+  static std::vector<Entry> seen;
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  std::lock_guard<std::mutex> lock(mu);
+  Entry* hit = nullptr;
+  for (Entry& en : seen)
+    if (en.kern == kern && en.dev == dev) { hit = &en; break; }
+  if (hit != nullptr && hit->bytes >= bytes) return DLT_OK;
+  e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
+  if (hit != nullptr) hit->bytes = bytes;
+  else seen.push_back(Entry{kern, dev, bytes});
+  return DLT_OK;
+}
+
 static __device__ __align__(256) float g_delta_scratch[DLT_NOALLOC_MAX_DELTA];
 
 namespace {

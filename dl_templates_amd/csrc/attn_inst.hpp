@@ -8,14 +8,7 @@
 
 namespace {
 template <typename KernT>
-int set_lds_limit(KernT kern, int bytes) {
-  // dynamic LDS above the default limit must be opted into once per kernel
-  if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
-  }
-  return DLT_OK;
-}
+int set_lds_limit(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cast<const void*>(kern), bytes); }
 
 template <typename TIO, int NP>
 int launch_fwd_t(const FwdArgs& a, int grid, hipStream_t stream) {

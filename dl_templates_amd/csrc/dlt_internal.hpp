@@ -10,6 +10,10 @@
 
 // ---- error reporting ---------------------------------------------------------------
 int dlt_set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+// Raises a kernel's limit of dynamic LDS to `bytes` on the current device.  The runtime call is made only when a larger
+// size than any before is asked for (per kernel and device): it costs tens of microseconds of host time, which would
+// otherwise sit in front of every launch.
+int dlt_ensure_lds(const void* kern, int bytes);
 
 #define DLT_REQUIRE(cond, ...)                                   \
   do {                                                           \

@@ -9,9 +9,9 @@ namespace {
 template <typename TIO, int MODE>
 int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
   auto kern = flash_fwd_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, flash_ck_fwd(DLT_DK, DLT_DV), MODE>;
-  if (a.lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, a.lds_bytes);
-    if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", a.lds_bytes, hipGetErrorString(e));
+  {
+    const int rc = dlt_ensure_lds(reinterpret_cast<const void*>(kern), a.lds_bytes);
+    if (rc != DLT_OK) return rc;
   }
   dlt_timing_before(DLT_K_FWD, stream);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(256), a.lds_bytes, stream, a);
@@ -27,13 +27,7 @@ int flash_launch_fwd_t(const FlashArgs& a, int grid, hipStream_t stream) {
 }
 
 template <typename KernT>
-int flash_set_lds(KernT kern, int bytes) {
-  if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
-  }
-  return DLT_OK;
-}
+int flash_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cast<const void*>(kern), bytes); }
 
 template <typename TIO, int MODE>
 int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {

@@ -7,13 +7,7 @@
 
 namespace {
 template <typename KernT>
-int swa1_set_lds(KernT kern, int bytes) {
-  if (bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
-  }
-  return DLT_OK;
-}
+int swa1_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cast<const void*>(kern), bytes); }
 
 template <typename TIO, int NCGMAX, int ROPE>
 int swa1_launch_fwd_r(const Swa1FwdArgs& a, int grid, hipStream_t stream) {

@@ -195,12 +195,23 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_q_kernel(const Swa2BwdA
     }
   };
 
-  for (int ch = G.ch_first; ch < G.ch_last; ch++) {
-    if (ch >= W.ch_lo && ch <= W.ch_hi) consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF, smem + ((ch + 1) & 1) * SWA2_BUF, std::true_type{});
-    else swa2_issue(st, G, ch + 1, sbase, srow, smem + ((ch + 1) & 1) * SWA2_BUF, wave);
+  // Every wave runs ch_last - ch_first rounds of (work, wait for its copies, workgroup barrier).  The chunks that hold
+  // visible rows of its patch are contiguous; the rounds before and after them only copy.  Three loops instead of one
+  // with a branch keep the accumulators in place (a branch inside the loop had them copied on every round).
+  const int act_lo = dlt_imax(G.ch_first, W.ch_lo), act_hi = dlt_imin(G.ch_last - 1, W.ch_hi);
+  auto copy_only = [&](int ch) {
+    swa2_issue(st, G, ch + 1, sbase, srow, smem + ((ch + 1) & 1) * SWA2_BUF, wave);
+    swa2_wait_copies();
+    __syncthreads();
+  };
+  int ch = G.ch_first;
+  for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
+  for (; ch <= act_hi; ch++) {
+    consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF, smem + ((ch + 1) & 1) * SWA2_BUF, std::true_type{});
     swa2_wait_copies();
     __syncthreads();
   }
+  for (; ch < G.ch_last; ch++) copy_only(ch);
   if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
     consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * SWA2_BUF, smem + ((G.ch_last + 1) & 1) * SWA2_BUF, std::false_type{});
   __syncthreads();
@@ -239,7 +250,7 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_kv_kernel(const Swa2Bwd
   const char* sbase = stage_q ? qb : dob;
   const int ssn2 = (int)(stage_q ? a.qs[2] : a.dos[2]) * 2;
   const uint32_t srow = (uint32_t)(G.TC * ssn2);
-  Swa2StageLean st;   // this kernel is short of registers
+  Swa2Stage st;
   swa2_stage_init(st, G, wave, lane, ssn2);
   const float* scal_base = stage_q ? lseb : delb;
   const int ls2 = (int)a.ls[2];
@@ -406,16 +417,23 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_kv_kernel(const Swa2Bwd
     }
   };
 
-  for (int ch = G.ch_first; ch < G.ch_last; ch++) {
+  // three loops, as in the dQ kernel
+  const int act_lo = dlt_imax(G.ch_first, W.ch_lo), act_hi = dlt_imin(G.ch_last - 1, W.ch_hi);
+  auto copy_only = [&](int ch) {
     char* nxt = smem + ((ch + 1) & 1) * SWA2_BUF_KV;
-    if (ch >= W.ch_lo && ch <= W.ch_hi) consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF_KV, nxt, std::true_type{});
-    else {
-      swa2_issue(st, G, ch + 1, sbase, srow, nxt, wave);
-      issue_scalars(ch + 1, nxt);
-    }
+    swa2_issue(st, G, ch + 1, sbase, srow, nxt, wave);
+    issue_scalars(ch + 1, nxt);
+    swa2_wait_copies();
+    __syncthreads();
+  };
+  int ch = G.ch_first;
+  for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
+  for (; ch <= act_hi; ch++) {
+    consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF_KV, smem + ((ch + 1) & 1) * SWA2_BUF_KV, std::true_type{});
     swa2_wait_copies();
     __syncthreads();
   }
+  for (; ch < G.ch_last; ch++) copy_only(ch);
   if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
     consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * SWA2_BUF_KV, smem + ((G.ch_last + 1) & 1) * SWA2_BUF_KV, std::false_type{});
   __syncthreads();

@@ -101,36 +101,6 @@ DLT_DEV const char* swa2_issue_row(const Swa2Geom& G, int ch, const char* base, 
 }
 DLT_DEV char* swa2_issue_dst(char* buf, int wave) { return buf + (wave >> 2) * SWA2_REGION + (wave & 3) * (SWA2_HCW * SWA2_ROW); }
 
-// The same copies with the nine offsets recomputed per instruction from two lane constants (four vector instructions
-// each) instead of held in nine registers: for the kernel that has none to spare.
-struct Swa2StageLean {
-  int cb;         // grid column of the lane's token in instruction 0 (may lie outside the grid: clamped per instruction)
-  uint32_t swz;   // swizzled piece offset of instruction 0; instructions alternate between swz and swz ^ 128
-  int sn2, tc1;   // bytes between tokens, TC - 1
-};
-DLT_DEV void swa2_stage_init(Swa2StageLean& st, const Swa2Geom& G, int wave, int lane, int sn2) {
-  st.cb = G.c0 - G.WC + (lane >> 4);
-  // token & 7 = (lane >> 4) + 4 ((wave + i) & 1)  (36 = 4 mod 8, four tokens per instruction)
-  st.swz = (uint32_t)(16 * ((lane & 15) ^ (2 * (lane >> 4)) ^ (8 * (wave & 1))));
-  st.sn2 = sn2;
-  st.tc1 = G.TC - 1;
-}
-template <int I>
-DLT_DEV void swa2_issue_one(const Swa2StageLean& st, const char* row, char* dst) {
-  int cb = st.cb;
-  asm volatile("" : "+v"(cb));   // keeps the nine offsets from being hoisted out of the chunk loop into registers
-  const int cc = dlt_imax(0, dlt_imin(cb + 4 * I, st.tc1));
-  const uint32_t off = (uint32_t)(cc * st.sn2) + ((I & 1) ? (st.swz ^ 128u) : st.swz);
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(row + off), (DLT_LDS void*)(dst + 1024 * I), 16, 0, 0);
-}
-DLT_DEV void swa2_issue(const Swa2StageLean& st, const Swa2Geom& G, int ch, const char* base, uint32_t rowstride, char* buf, int wave) {
-  const char* row = swa2_issue_row(G, ch, base, rowstride, wave);
-  char* dst = swa2_issue_dst(buf, wave);
-  swa2_issue_one<0>(st, row, dst); swa2_issue_one<1>(st, row, dst); swa2_issue_one<2>(st, row, dst);
-  swa2_issue_one<3>(st, row, dst); swa2_issue_one<4>(st, row, dst); swa2_issue_one<5>(st, row, dst);
-  swa2_issue_one<6>(st, row, dst); swa2_issue_one<7>(st, row, dst); swa2_issue_one<8>(st, row, dst);
-}
-
 // every copy this wave issued has landed in LDS (the workgroup barrier that follows makes all of them visible)
 DLT_DEV void swa2_wait_copies() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 

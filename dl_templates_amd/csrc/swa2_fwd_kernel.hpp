@@ -207,12 +207,23 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_fwd_kernel(const Swa2FwdArg
   };
 
   // chunk ch + 1 travels HBM -> LDS (other buffer) while chunk ch is consumed; one barrier per chunk
-  for (int ch = G.ch_first; ch < G.ch_last; ch++) {
-    if (ch >= W.ch_lo && ch <= W.ch_hi) consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF, smem + ((ch + 1) & 1) * SWA2_BUF, std::true_type{});
-    else swa2_issue(st, G, ch + 1, sbase, srow, smem + ((ch + 1) & 1) * SWA2_BUF, wave);
+  // Every wave runs ch_last - ch_first rounds of (work, wait for its copies, workgroup barrier).  The chunks that hold
+  // visible rows of its patch are contiguous; the rounds before and after them only copy.  Three loops instead of one
+  // with a branch keep the accumulators in place (a branch inside the loop had them copied on every round).
+  const int act_lo = dlt_imax(G.ch_first, W.ch_lo), act_hi = dlt_imin(G.ch_last - 1, W.ch_hi);
+  auto copy_only = [&](int ch) {
+    swa2_issue(st, G, ch + 1, sbase, srow, smem + ((ch + 1) & 1) * SWA2_BUF, wave);
+    swa2_wait_copies();
+    __syncthreads();
+  };
+  int ch = G.ch_first;
+  for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
+  for (; ch <= act_hi; ch++) {
+    consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF, smem + ((ch + 1) & 1) * SWA2_BUF, std::true_type{});
     swa2_wait_copies();
     __syncthreads();
   }
+  for (; ch < G.ch_last; ch++) copy_only(ch);
   if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi) consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * SWA2_BUF, smem + ((G.ch_last + 1) & 1) * SWA2_BUF, std::false_type{});
   __syncthreads();
 

@@ -3,11 +3,7 @@
 
 namespace {
 template <typename KernT>
-int swa2_set_lds(KernT kern, int bytes) {
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-  if (e != hipSuccess) return dlt_set_error(DLT_ERR_LAUNCH, "hipFuncSetAttribute(%d bytes of LDS): %s", bytes, hipGetErrorString(e));
-  return DLT_OK;
-}
+int swa2_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cast<const void*>(kern), bytes); }
 
 template <typename TIO>
 int swa2_launch_fwd_t(const Swa2FwdArgs& a, int grid, hipStream_t stream) {
