@@ -18,6 +18,7 @@
 // sums produced by one extra MFMA against a row of ones.  Keys past Lk are clamped loads
 // masked by an additive -inf bias that only the last chunk applies.
 #pragma once
+#include <type_traits>
 #include "swa1_common.hpp"
 
 // Streamed chunks in LDS: rows of 2 D + 32 bytes.  16-byte LDS accesses of a wave are served 16
@@ -285,11 +286,17 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   pin_loaded(qf);
 
   // products and softmax update of the chunk resident in LDS
-  auto consume = [&](const int ci) {
+  // `tail` (dense / causal): some keys of the chunk lie past the end or (causal) above the wave's first query, and every
+  // pair is tested.  A compile-time tag: without a causal mask only the last chunk can be short, and the loop body then
+  // holds no test at all.
+  auto chunk_tail = [&](const int ci) {
+    const FlashChunk c = W.at(ci);
+    return !TILE && (c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0));
+  };
+  auto consume_t = [&](const int ci, auto tail_tag) {
+    constexpr bool tail = decltype(tail_tag)::value;
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
-    // dense / causal: some keys of this chunk lie past the end or (causal) above the wave's first query
-    const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && k0 + CK - 1 > wq0));
     // causal: every key of the chunk lies above every query of this wave (wave-uniform)
     bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
     // tile mode: which 32-key blocks hold a 16-key half that query block p sees (wave-uniform)
@@ -358,22 +365,24 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
 #pragma unroll
           for (int i = 0; i < 4; i++) mx[i] = fmaxf(fmaxf(mx[i], t[p][kb][2 * i]), t[p][kb][2 * i + 1]);
         float mloc = wave_max4(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])));
-        const float m_new = fmaxf(m_run[p], mloc);
-        const float m_use = m_new == -INFINITY ? 0.f : m_new;   // a block that has seen no key yet
-        const float alpha = fast_exp2((m_run[p] - m_use) * scale);
-        const float neg_m2 = -m_use * scale;
-        m_run[p] = m_new;
+        // The reference maximum only moves when a score exceeds it by more than 2^8 after scaling: p stays below 2^8,
+        // well inside the range of the 16-bit operand and of the fp32 sums, and most chunks skip the rescaling of the
+        // accumulators.  o and lse do not depend on which reference was used.
+        if (__builtin_amdgcn_ballot_w64((mloc - m_run[p]) * scale > 8.f)) {
+          keep_branch();
+          const float m_new = fmaxf(m_run[p], mloc);   // finite here
+          const float alpha = fast_exp2((m_run[p] - m_new) * scale);
+          m_run[p] = m_new;
+#pragma unroll
+          for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
+          acc_l[p] *= alpha;
+        }
+        const float neg_m2 = m_run[p] == -INFINITY ? 0.f : -m_run[p] * scale;   // -inf: a block that has seen no key yet
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
           for (int i = 0; i < 8; i++) t[p][kb][i] = fast_exp2(fmaf(t[p][kb][i], scale, neg_m2));
           pb[p][kb] = pack8<CT>(t[p][kb]);
-        }
-        if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
-          keep_branch();
-#pragma unroll
-          for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
-          acc_l[p] *= alpha;
         }
       }
     }
@@ -400,9 +409,14 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   // The last chunk is peeled off so that prefetch and commit are unconditional inside the loop:
   // with `if (has_next)` around each, the compiler sees a path on which loads stay pending across
   // the back edge and guards every later load with a full vmcnt(0) wait.
+  auto consume = [&](const int ci) {
+    if (chunk_tail(ci)) consume_t(ci, std::true_type{});
+    else consume_t(ci, std::false_type{});
+  };
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
     issue(W.at(ci + 1));
-    consume(ci);
+    if (CAUSAL) consume(ci);
+    else consume_t(ci, std::false_type{});
     __syncthreads();
     commit();
     __syncthreads();
@@ -604,10 +618,16 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
 #pragma unroll
   for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
 
-  auto consume = [&](const int ci) {
+  // `tail`: some keys of the chunk lie past the end or (causal) above the wave's first query, and every pair is tested.
+  // It is a compile-time tag: as a run-time flag the test was folded into a select per element of every chunk.
+  auto chunk_tail = [&](const int ci) {
+    const FlashChunk c = W.at(ci);
+    return !TILE && (c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0));
+  };
+  auto consume_t = [&](const int ci, auto tail_tag) {
+    constexpr bool tail = decltype(tail_tag)::value;
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
-    const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && k0 + CK - 1 > wq0));
     const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
 #pragma unroll
     for (int kb = 0; kb < NKB; kb++) {
@@ -664,10 +684,16 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
       }
     }
   };
-  // last chunk peeled off: unconditional prefetch and commit inside the loop (see the forward kernel)
+  auto consume = [&](const int ci) {
+    if (chunk_tail(ci)) consume_t(ci, std::true_type{});
+    else consume_t(ci, std::false_type{});
+  };
+  // last chunk peeled off: unconditional prefetch and commit inside the loop (see the forward kernel); without a causal
+  // mask only the last chunk can be short
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
     st.issue(kb_, ak, vb_, av, W.at(ci + 1));
-    consume(ci);
+    if (CAUSAL) consume(ci);
+    else consume_t(ci, std::false_type{});
     __syncthreads();
     st.commit(sK, PK, sV, PV);
     __syncthreads();
@@ -763,11 +789,16 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
   pin_loaded(kf);
   pin_loaded(vf);
 
-  auto consume = [&](const int ci) {
+  // `tail`: some queries of the chunk lie past the end or (causal) below the wave's last own key (a compile-time tag, as
+  // in the dQ kernel)
+  auto chunk_tail = [&](const int ci) {
+    const FlashChunk c = W.at(ci);
+    return !TILE && (c.nvalid < CK || (CAUSAL && c.x < wk0 + 16 * NP - 1));
+  };
+  auto consume_t = [&](const int ci, auto tail_tag) {
+    constexpr bool tail = decltype(tail_tag)::value;
     const FlashChunk c = W.at(ci);
     const int q0 = c.x;
-    // some queries of the chunk lie past the end or (causal) below the wave's last own key
-    const bool tail = !TILE && (c.nvalid < CK || (CAUSAL && q0 < wk0 + 16 * NP - 1));
     // causal: every query of the chunk lies below every own key of this wave
     const bool live = !CAUSAL || q0 + CK - 1 >= wk0;
 #pragma unroll
@@ -836,11 +867,16 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
       }
     }
   };
+  auto consume = [&](const int ci) {
+    if (chunk_tail(ci)) consume_t(ci, std::true_type{});
+    else consume_t(ci, std::false_type{});
+  };
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
     const FlashChunk cn = W.at(ci + 1);
     st.issue(qb, aq, dob, ad, cn);
     issue_scalars(cn);
-    consume(ci);
+    if (CAUSAL) consume(ci);
+    else consume_t(ci, std::false_type{});   // without a causal mask only the last chunk can be short
     __syncthreads();
     st.commit(sQ, PQ, sDO, PD);
     pin_loaded(r_lse);
