@@ -39,8 +39,10 @@ int dlt_swa1_launch_fwd_64(const Swa1FwdArgs&, int, int, hipStream_t);
 int dlt_swa1_launch_fwd_128(const Swa1FwdArgs&, int, int, hipStream_t);
 int dlt_swam_launch_fwd(const SwamFwdArgs&, int, int, hipStream_t);
 int dlt_swam_launch_bwd(const SwamBwdArgs&, int, int, hipStream_t);
-int dlt_swa2_launch_fwd(const Swa2FwdArgs&, int, hipStream_t);
-int dlt_swa2_launch_bwd(const Swa2BwdArgs&, int, hipStream_t);
+int dlt_swa2_launch_fwd_64(const Swa2FwdArgs&, int, int, hipStream_t);
+int dlt_swa2_launch_bwd_64(const Swa2BwdArgs&, int, int, hipStream_t);
+int dlt_swa2_launch_fwd_128(const Swa2FwdArgs&, int, int, hipStream_t);
+int dlt_swa2_launch_bwd_128(const Swa2BwdArgs&, int, int, hipStream_t);
 
 namespace {
 
@@ -288,10 +290,12 @@ int swam_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
   return dlt_swam_launch_fwd(a, c.rope_mode != 0, (int)grid, stream);
 }
 
-// ---- streaming kernels for head dim 128 exactly, no rotation, windows up to 21 columns -------------------------------
+// ---- streaming kernels: head dim 64 or 128 exactly, no rotation, windows up to 21 columns ---------------------------
 bool swa2_eligible(const AttnProblem& p, const Swa1Class& c) {
-  return c.D == 128 && p.dk == 128 && p.dv == 128 && c.rope_mode == 0 && p.g.WC <= 10;
+  return (c.D == 64 || c.D == 128) && p.dk == c.D && p.dv == c.D && c.rope_mode == 0 && p.g.WC <= 10;
 }
+// column groups of a wave's window: 4 x 4 columns cover windows up to 13 columns, 6 x 4 up to 21
+int swa2_ncg(const AttnProblem& p) { return p.g.WC <= 6 ? 4 : 6; }
 
 void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan) {
   plan.nblk_r = (p.g.TR + 7) / 8;
@@ -302,7 +306,7 @@ void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan) {
 }
 
 bool swa2_rows_ok(const AttnProblem& p, const void* ptr, const int64_t* st) {
-  return tvec_ok(ptr, st, 128, 2) && st[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * st[2] * 2 + 256 <= (((int64_t)1 << 31) - 1);
+  return tvec_ok(ptr, st, p.dk, 2) && st[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * st[2] * 2 + 2 * p.dk <= (((int64_t)1 << 31) - 1);
 }
 
 int swa2_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
@@ -315,7 +319,7 @@ int swa2_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream)
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
   if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention forward: grid too large");
-  return dlt_swa2_launch_fwd(a, (int)grid, stream);
+  return p.dk == 64 ? dlt_swa2_launch_fwd_64(a, swa2_ncg(p), (int)grid, stream) : dlt_swa2_launch_fwd_128(a, swa2_ncg(p), (int)grid, stream);
 }
 
 int swa2_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
@@ -332,7 +336,7 @@ int swa2_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream
   a.scale_log2 = p.sm_scale * 1.4426950408889634f;
   const int64_t grid = (int64_t)p.B * p.H * a.plan.nblk_r * a.plan.nblk_c;
   if (grid > 0x7fffffff) return dlt_set_error(DLT_ERR_UNSUPPORTED, "attention backward: grid too large");
-  return dlt_swa2_launch_bwd(a, (int)grid, stream);
+  return p.dk == 64 ? dlt_swa2_launch_bwd_64(a, swa2_ncg(p), (int)grid, stream) : dlt_swa2_launch_bwd_128(a, swa2_ncg(p), (int)grid, stream);
 }
 
 // backward on the marching kernels: plain inputs, or rotated inputs with the gradients rotated back on store

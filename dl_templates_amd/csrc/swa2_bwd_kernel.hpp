@@ -1,5 +1,5 @@
-// Backward kernels for token grids at head dim 128 (b_size == 1, no rotation): the decoupled dQ and dK/dV passes of
-// tiled_swa_bwd_large_kernel_decoupled_q (src/tiled_swa.py:407-562) on the streaming structure of swa2_common.hpp.
+// Backward kernels for token grids at head dim 64 / 128 (b_size == 1, no rotation): the decoupled dQ and dK/dV passes
+// of tiled_swa_bwd_large_kernel_decoupled_q (src/tiled_swa.py:407-562) on the streaming structure of swa2_common.hpp.
 //
 //   dQ   : a wave owns a 4x4 patch of queries; K and V stream through LDS.  It runs first and computes
 //          delta = rowsum(o * dO) of its own queries on the way (the reference's pre-pass, src/tiled_swa.py:253-282),
@@ -22,22 +22,17 @@ struct Swa2BwdArgs {
   float scale_log2;
 };
 
-// own-token fragments in B-operand layout: lane (n, g) holds head dims 32 c + 8 g .. + 7 of token n
-DLT_DEV void swa2_own_frags(u32x4 (&f)[4], const char* base, int sn2, int tok, int g) {
-  const char* p = base + ((uint32_t)((tok >= 0 ? tok : 0) * sn2) + 16 * g);
-#pragma unroll
-  for (int c = 0; c < 4; c++) f[c] = *reinterpret_cast<const u32x4*>(p + 64 * c);
-}
-
-// visibility of the streamed token (halo row `hrow`, window column 4 cg + i) from the lane's own token
-DLT_DEV bool swa2_visible(const Swa2Win& W, bool row_vis, int cg, int i, int ncg) {
-  return row_vis & (cg < ncg) & ((unsigned)(4 * cg + i - W.clo) <= (unsigned)W.cspan);
-}
+// waves per SIMD the register budget is sized for
+constexpr int swa2_occ_bwd_q(int D) { return D == 64 ? 4 : 2; }
+constexpr int swa2_occ_bwd_kv(int D) { return 2; }
 
 // =============================================================================================== dQ
-template <typename TIO>
-__global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_q_kernel(const Swa2BwdArgs a) {
+template <typename TIO, int D, int NCG>
+__global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_kernel(const Swa2BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
+  typedef Swa2Cfg<D, NCG> C;
+  constexpr int KC = C::KC, VB = C::VB, NKB = C::NKB;
+  constexpr int NG = VB / 4;   // groups of four 16-dim blocks of dQ
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -60,24 +55,24 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_q_kernel(const Swa2BwdA
   const char* sbase = stage_k ? kb_ : vb_;
   const int ssn2 = (int)(stage_k ? a.ks[2] : a.vs[2]) * 2;
   const uint32_t srow = (uint32_t)(G.TC * ssn2);
-  Swa2Stage st;
+  Swa2Stage<C> st;
   swa2_stage_init(st, G, wave, lane, ssn2);
-  swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * SWA2_BUF, wave);
+  swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF, wave);
 
   const int r_p = G.r0 + 4 * rg, c_p = G.c0 + 4 * pc;
   const int tq = (r_p + (n >> 2) < G.TR && c_p + (n & 3) < G.TC) ? (r_p + (n >> 2)) * G.TC + c_p + (n & 3) : -1;
-  u32x4 qf[4], dof[4];
+  u32x4 qf[KC], dof[KC];
   float neg_lse, del_n;
   {
-    u32x4 of[4];
-    swa2_own_frags(qf, qb, (int)a.qs[2] * 2, tq, g);
-    swa2_own_frags(dof, dob, (int)a.dos[2] * 2, tq, g);
-    swa2_own_frags(of, ob, (int)a.os[2] * 2, tq, g);
+    u32x4 of[KC];
+    swa2_own_frags<KC>(qf, qb, (int)a.qs[2] * 2, tq, g);
+    swa2_own_frags<KC>(dof, dob, (int)a.dos[2] * 2, tq, g);
+    swa2_own_frags<KC>(of, ob, (int)a.os[2] * 2, tq, g);
     neg_lse = tq >= 0 ? -lseb[(int64_t)tq * a.ls[2]] : -INFINITY;
-    // delta = rowsum(o * dO) of the own token: 32 head dims per lane, summed over the four lanes of the token
+    // delta = rowsum(o * dO) of the own token: D / 4 head dims per lane, summed over the four lanes of the token
     float part = 0.f;
 #pragma unroll
-    for (int c = 0; c < 4; c++)
+    for (int c = 0; c < KC; c++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         part = fmaf(unpack_lo<CT>(of[c][j]), unpack_lo<CT>(dof[c][j]), part);
@@ -87,12 +82,12 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_q_kernel(const Swa2BwdA
     if (g == 0 && tq >= 0) delb[(int64_t)tq * a.ls[2]] = del_n;
   }
   const Swa2Win W = swa2_window(G, rg, pc, n);
-  Swa2Lane L;
+  Swa2Lane<C> L;
   swa2_lane_init(L, pc, n, g);
 
-  f32x4 acc[8];
+  f32x4 acc[VB];
 #pragma unroll
-  for (int d = 0; d < 8; d++) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int d = 0; d < VB; d++) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int ncg = (4 + 2 * G.WC + 3) >> 2;
 
   swa2_wait_copies();   // also: the own fragments have arrived
@@ -102,15 +97,15 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_q_kernel(const Swa2BwdA
   auto consume = [&](const int ch, Swa2Lds __restrict__ cur, char* __restrict__ nxt, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     Swa2Lds sK = cur;
-    Swa2Lds sV = sK + SWA2_REGION;
+    Swa2Lds sV = sK + C::REGION;
     const char* nrow = swa2_issue_row(G, ch + 1, sbase, srow, wave);
-    char* ndst = swa2_issue_dst(nxt, wave);
+    char* ndst = swa2_issue_dst<C>(nxt, wave);
     const int hrow = 4 * ch + g;
     const bool row_vis = (hrow >= W.rlo) & (hrow <= W.rhi);
-    u32x4 xk[2][4], xv[2][4], kt[2][4];
-    swa2_read_a<0>(sK, L, xk[0]);
-#pragma unroll
-    for (int kb = 0; kb < 3; kb++) {
+    u32x4 xk[2][KC], xv[2][KC], kt[2][4];
+    swa2_read_a<C, 0>(sK, L, xk[0]);
+    swa2_for<0, NKB>([&](auto kbc) {
+      constexpr int kb = decltype(kbc)::value;
       f32x4 s[2], dp[2];
       float t[8];
       // dS^T of one column group: p = exp2(s scale - lse2) where visible, dS = p (dP - delta)
@@ -124,110 +119,87 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_q_kernel(const Swa2BwdA
         }
       };
       // ---- stage 1: S of the even column group
-      if (more) {
-        if (kb == 0) swa2_issue_one<0>(st, nrow, ndst);
-        if (kb == 1) swa2_issue_one<3>(st, nrow, ndst);
-        if (kb == 2) swa2_issue_one<6>(st, nrow, ndst);
-      }
-      if (kb == 0) swa2_read_a<0>(sV, L, xv[0]);
-      if (kb == 1) swa2_read_a<2>(sV, L, xv[0]);
-      if (kb == 2) swa2_read_a<4>(sV, L, xv[0]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb>(st, nrow, ndst);
+      swa2_read_a<C, 2 * kb>(sV, L, xv[0]);
       __builtin_amdgcn_sched_barrier(0);
       s[0] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 4; c++) s[0] = Mma<CT>::mfma(xk[0][c], qf[c], s[0]);
+      for (int c = 0; c < KC; c++) s[0] = Mma<CT>::mfma(xk[0][c], qf[c], s[0]);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 2: dP of the even column group
-      if (kb == 0) swa2_read_a<1>(sK, L, xk[1]);
-      if (kb == 1) swa2_read_a<3>(sK, L, xk[1]);
-      if (kb == 2) swa2_read_a<5>(sK, L, xk[1]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb + 1>(st, nrow, ndst);
+      swa2_read_a<C, 2 * kb + 1>(sK, L, xk[1]);
       __builtin_amdgcn_sched_barrier(0);
       dp[0] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 4; c++) dp[0] = Mma<CT>::mfma(xv[0][c], dof[c], dp[0]);
+      for (int c = 0; c < KC; c++) dp[0] = Mma<CT>::mfma(xv[0][c], dof[c], dp[0]);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 3: S of the odd column group
-      if (more) {
-        if (kb == 0) swa2_issue_one<1>(st, nrow, ndst);
-        if (kb == 1) swa2_issue_one<4>(st, nrow, ndst);
-        if (kb == 2) swa2_issue_one<7>(st, nrow, ndst);
-      }
-      if (kb == 0) swa2_read_a<1>(sV, L, xv[1]);
-      if (kb == 1) swa2_read_a<3>(sV, L, xv[1]);
-      if (kb == 2) swa2_read_a<5>(sV, L, xv[1]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb + 2>(st, nrow, ndst);
+      swa2_read_a<C, 2 * kb + 1>(sV, L, xv[1]);
       __builtin_amdgcn_sched_barrier(0);
       s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 4; c++) s[1] = Mma<CT>::mfma(xk[1][c], qf[c], s[1]);
+      for (int c = 0; c < KC; c++) s[1] = Mma<CT>::mfma(xk[1][c], qf[c], s[1]);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 4: dP of the odd column group, with the elementwise work of the even one between the products
-      if (kb == 0) swa2_read_tr<0, 0, 4>(sK, L, kt[0]);
-      if (kb == 1) swa2_read_tr<1, 0, 4>(sK, L, kt[0]);
-      if (kb == 2) swa2_read_tr<2, 0, 4>(sK, L, kt[0]);
+      swa2_read_tr<C, kb, 0, 4>(sK, L, kt[0]);
       __builtin_amdgcn_sched_barrier(0);
       dp[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 4; c++) dp[1] = Mma<CT>::mfma(xv[1][c], dof[c], dp[1]);
+      for (int c = 0; c < KC; c++) dp[1] = Mma<CT>::mfma(xv[1][c], dof[c], dp[1]);
       elementwise(0);
-      SWA2_MIX(4, 4)
+      SWA2_MIX(KC, 16 / KC)
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 5: elementwise work of the odd column group
-      if (more) {
-        if (kb == 0) swa2_issue_one<2>(st, nrow, ndst);
-        if (kb == 1) swa2_issue_one<5>(st, nrow, ndst);
-        if (kb == 2) swa2_issue_one<8>(st, nrow, ndst);
-      }
-      if (kb == 0) swa2_read_tr<0, 4, 4>(sK, L, kt[1]);
-      if (kb == 1) swa2_read_tr<1, 4, 4>(sK, L, kt[1]);
-      if (kb == 2) swa2_read_tr<2, 4, 4>(sK, L, kt[1]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb + 3>(st, nrow, ndst);
+      if constexpr (NG == 2) swa2_read_tr<C, kb, 4, 4>(sK, L, kt[1]);
       elementwise(1);
       const u32x4 pk = pack8<CT>(t);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stages 6, 7: dQ^T += K^T dS^T
-      if (kb == 0) swa2_read_a<2>(sK, L, xk[0]);
-      if (kb == 1) swa2_read_a<4>(sK, L, xk[0]);
+      if constexpr (kb + 1 < NKB) swa2_read_a<C, 2 * kb + 2>(sK, L, xk[0]);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int d = 0; d < 4; d++) acc[d] = Mma<CT>::mfma(kt[0][d], pk, acc[d]);
+      if constexpr (NG == 2) {
 #pragma unroll
-      for (int d = 0; d < 4; d++) acc[4 + d] = Mma<CT>::mfma(kt[1][d], pk, acc[4 + d]);
+        for (int d = 0; d < 4; d++) acc[4 + d] = Mma<CT>::mfma(kt[1][d], pk, acc[4 + d]);
+      }
       __builtin_amdgcn_sched_barrier(0);
-    }
+    });
   };
 
-  // Every wave runs ch_last - ch_first rounds of (work, wait for its copies, workgroup barrier).  The chunks that hold
-  // visible rows of its patch are contiguous; the rounds before and after them only copy.  Three loops instead of one
-  // with a branch keep the accumulators in place (a branch inside the loop had them copied on every round).
+  // three loops: copy-only rounds before and after the rounds with visible rows (see the forward kernel)
   const int act_lo = dlt_imax(G.ch_first, W.ch_lo), act_hi = dlt_imin(G.ch_last - 1, W.ch_hi);
   auto copy_only = [&](int ch) {
-    swa2_issue(st, G, ch + 1, sbase, srow, smem + ((ch + 1) & 1) * SWA2_BUF, wave);
+    swa2_issue(st, G, ch + 1, sbase, srow, smem + ((ch + 1) & 1) * C::BUF, wave);
     swa2_wait_copies();
     __syncthreads();
   };
   int ch = G.ch_first;
   for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
   for (; ch <= act_hi; ch++) {
-    consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF, smem + ((ch + 1) & 1) * SWA2_BUF, std::true_type{});
+    consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF, smem + ((ch + 1) & 1) * C::BUF, std::true_type{});
     swa2_wait_copies();
     __syncthreads();
   }
   for (; ch < G.ch_last; ch++) copy_only(ch);
   if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
-    consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * SWA2_BUF, smem + ((G.ch_last + 1) & 1) * SWA2_BUF, std::false_type{});
+    consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF, smem + ((G.ch_last + 1) & 1) * C::BUF, std::false_type{});
   __syncthreads();
 
-  swa2_store_own<TIO, CT>(smem + wave * 4096, acc, a.p.sm_scale, dqb, a.dqs[2], G, r_p, c_p, lane);
+  swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, acc, a.p.sm_scale, dqb, a.dqs[2], G, r_p, c_p, lane);
 }
 
 // =============================================================================================== dK / dV
-// A chunk buffer holds Q, dO and a table of per-token scalars: lse2 then delta, [4 halo rows][36 halo columns] each.
-constexpr int SWA2_SCAL = 2 * SWA2_TOK * 4;
-constexpr int SWA2_BUF_KV = SWA2_BUF + SWA2_SCAL;
-constexpr int SWA2_LDS_KV = 2 * SWA2_BUF_KV;
-
-template <typename TIO>
-__global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_kv_kernel(const Swa2BwdArgs a) {
+// A chunk buffer holds Q, dO and a table of per-token scalars: lse2 then delta, [4 halo rows][HCW halo columns] each.
+template <typename TIO, int D, int NCG>
+__global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_kernel(const Swa2BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
+  typedef Swa2Cfg<D, NCG> C;
+  constexpr int KC = C::KC, VB = C::VB, NKB = C::NKB;
+  constexpr int NP2 = VB / 2;   // pairs of 16-dim blocks per gradient
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -250,36 +222,36 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_kv_kernel(const Swa2Bwd
   const char* sbase = stage_q ? qb : dob;
   const int ssn2 = (int)(stage_q ? a.qs[2] : a.dos[2]) * 2;
   const uint32_t srow = (uint32_t)(G.TC * ssn2);
-  Swa2Stage st;
+  Swa2Stage<C> st;
   swa2_stage_init(st, G, wave, lane, ssn2);
   const float* scal_base = stage_q ? lseb : delb;
   const int ls2 = (int)a.ls[2];
-  // lane l < 36 copies the scalar of halo column l (clamped like the rows: positions outside the grid are masked)
+  // lane l < HCW copies the scalar of halo column l (clamped like the rows: positions outside the grid are masked)
   const uint32_t scal_off = (uint32_t)(dlt_imax(0, dlt_imin(G.c0 - G.WC + lane, G.TC - 1)) * ls2) * 4u;
   auto issue_scalars = [&](int ch, char* buf) {
     const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + 4 * ch + (wave & 3), G.TR - 1));
     const char* row = reinterpret_cast<const char*>(scal_base) + (uint32_t)(r * G.TC * ls2) * 4u;   // wave-uniform
-    char* dst = buf + SWA2_BUF + (wave >> 2) * (SWA2_TOK * 4) + (wave & 3) * (SWA2_HCW * 4);
-    if (lane < SWA2_HCW)
+    char* dst = buf + C::BUF + (wave >> 2) * (C::TOK * 4) + (wave & 3) * (C::HCW * 4);
+    if (lane < C::HCW)
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(row + scal_off), (DLT_LDS void*)dst, 4, 0, 0);
   };
-  swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * SWA2_BUF_KV, wave);
-  issue_scalars(G.ch_first, smem + (G.ch_first & 1) * SWA2_BUF_KV);
+  swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF_KV, wave);
+  issue_scalars(G.ch_first, smem + (G.ch_first & 1) * C::BUF_KV);
 
   const int r_p = G.r0 + 4 * rg, c_p = G.c0 + 4 * pc;
   const int tk = (r_p + (n >> 2) < G.TR && c_p + (n & 3) < G.TC) ? (r_p + (n >> 2)) * G.TC + c_p + (n & 3) : -1;
-  u32x4 kf[4], vf[4];
-  swa2_own_frags(kf, kb_, (int)a.ks[2] * 2, tk, g);
-  swa2_own_frags(vf, vb_, (int)a.vs[2] * 2, tk, g);
+  u32x4 kf[KC], vf[KC];
+  swa2_own_frags<KC>(kf, kb_, (int)a.ks[2] * 2, tk, g);
+  swa2_own_frags<KC>(vf, vb_, (int)a.vs[2] * 2, tk, g);
   const Swa2Win W = swa2_window(G, rg, pc, n);
-  Swa2Lane L;
+  Swa2Lane<C> L;
   swa2_lane_init(L, pc, n, g);
   // scalars of the queries (halo row g, window columns 4 cg .. 4 cg + 3) of a chunk
-  const int scal_lane = (g * SWA2_HCW + 4 * pc) * 4;
+  const int scal_lane = (g * C::HCW + 4 * pc) * 4;
 
-  f32x4 acck[8], accv[8];
+  f32x4 acck[VB], accv[VB];
 #pragma unroll
-  for (int d = 0; d < 8; d++) { acck[d] = f32x4{0.f, 0.f, 0.f, 0.f}; accv[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
+  for (int d = 0; d < VB; d++) { acck[d] = f32x4{0.f, 0.f, 0.f, 0.f}; accv[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
   const int ncg = (4 + 2 * G.WC + 3) >> 2;
 
   swa2_wait_copies();
@@ -288,20 +260,20 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_kv_kernel(const Swa2Bwd
   auto consume = [&](const int ch, Swa2Lds __restrict__ cur, char* __restrict__ nxt, auto more_tag) {
     constexpr bool more = decltype(more_tag)::value;
     Swa2Lds sQ = cur;
-    Swa2Lds sD = sQ + SWA2_REGION;
-    Swa2Lds sLse = cur + SWA2_BUF + scal_lane;
-    Swa2Lds sDel = sLse + SWA2_TOK * 4;
+    Swa2Lds sD = sQ + C::REGION;
+    Swa2Lds sLse = cur + C::BUF + scal_lane;
+    Swa2Lds sDel = sLse + C::TOK * 4;
     const char* nrow = swa2_issue_row(G, ch + 1, sbase, srow, wave);
-    char* ndst = swa2_issue_dst(nxt, wave);
-    if (more) issue_scalars(ch + 1, nxt);
+    char* ndst = swa2_issue_dst<C>(nxt, wave);
+    if constexpr (more) issue_scalars(ch + 1, nxt);
     const int hrow = 4 * ch + g;
     const bool row_vis = (hrow >= W.rlo) & (hrow <= W.rhi);
     // two A-operand buffers: a buffer is free again once the products that read it have been issued, one stage before
     // the next read into it returns.  Transposed operands come in pairs of 16-dim blocks, one pair ahead of its products.
-    u32x4 x[2][4], tr[2][2];
-    swa2_read_a<0>(sQ, L, x[0]);
-#pragma unroll
-    for (int kb = 0; kb < 3; kb++) {
+    u32x4 x[2][KC], tr[2][2];
+    swa2_read_a<C, 0>(sQ, L, x[0]);
+    swa2_for<0, NKB>([&](auto kbc) {
+      constexpr int kb = decltype(kbc)::value;
       u32x4 pp, pd;
       // P and dS of one column group, packed: p = exp2(s scale - lse2) where visible, dS = p (dP - delta)
       auto elementwise = [&](const int half, const f32x4& sv, const f32x4& dpv, const f32x4& lse4, const f32x4& del4) {
@@ -323,104 +295,79 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_kv_kernel(const Swa2Bwd
         }
       };
       // ---- stage 1: S of the even column group (rows: queries, columns: own keys)
-      if (more) {
-        if (kb == 0) swa2_issue_one<0>(st, nrow, ndst);
-        if (kb == 1) swa2_issue_one<3>(st, nrow, ndst);
-        if (kb == 2) swa2_issue_one<6>(st, nrow, ndst);
-      }
-      if (kb == 0) swa2_read_a<0>(sD, L, x[1]);
-      if (kb == 1) swa2_read_a<2>(sD, L, x[1]);
-      if (kb == 2) swa2_read_a<4>(sD, L, x[1]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb>(st, nrow, ndst);
+      swa2_read_a<C, 2 * kb>(sD, L, x[1]);
       const f32x4 lse_e = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 32 * kb));
       const f32x4 del_e = __builtin_bit_cast(f32x4, swa2_lds16(sDel + 32 * kb));
       __builtin_amdgcn_sched_barrier(0);
       f32x4 s0 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; j++) s0 = Mma<CT>::mfma(x[0][j], kf[j], s0);
+      for (int c = 0; c < KC; c++) s0 = Mma<CT>::mfma(x[0][c], kf[c], s0);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 2: dP of the even column group
-      if (kb == 0) swa2_read_a<1>(sQ, L, x[0]);
-      if (kb == 1) swa2_read_a<3>(sQ, L, x[0]);
-      if (kb == 2) swa2_read_a<5>(sQ, L, x[0]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb + 1>(st, nrow, ndst);
+      swa2_read_a<C, 2 * kb + 1>(sQ, L, x[0]);
       __builtin_amdgcn_sched_barrier(0);
       f32x4 dp0 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; j++) dp0 = Mma<CT>::mfma(x[1][j], vf[j], dp0);
+      for (int c = 0; c < KC; c++) dp0 = Mma<CT>::mfma(x[1][c], vf[c], dp0);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 3: S of the odd column group, with the elementwise work of the even one between the products
-      if (more) {
-        if (kb == 0) swa2_issue_one<1>(st, nrow, ndst);
-        if (kb == 1) swa2_issue_one<4>(st, nrow, ndst);
-        if (kb == 2) swa2_issue_one<7>(st, nrow, ndst);
-      }
-      if (kb == 0) swa2_read_a<1>(sD, L, x[1]);
-      if (kb == 1) swa2_read_a<3>(sD, L, x[1]);
-      if (kb == 2) swa2_read_a<5>(sD, L, x[1]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb + 2>(st, nrow, ndst);
+      swa2_read_a<C, 2 * kb + 1>(sD, L, x[1]);
       __builtin_amdgcn_sched_barrier(0);
       f32x4 s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; j++) s1 = Mma<CT>::mfma(x[0][j], kf[j], s1);
+      for (int c = 0; c < KC; c++) s1 = Mma<CT>::mfma(x[0][c], kf[c], s1);
       elementwise(0, s0, dp0, lse_e, del_e);
-      SWA2_MIX(4, 5)
+      SWA2_MIX(KC, 20 / KC)
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 4: dP of the odd column group
-      if (kb == 0) swa2_read_tr<0, 0, 2>(sD, L, tr[0]);
-      if (kb == 1) swa2_read_tr<1, 0, 2>(sD, L, tr[0]);
-      if (kb == 2) swa2_read_tr<2, 0, 2>(sD, L, tr[0]);
+      swa2_read_tr<C, kb, 0, 2>(sD, L, tr[0]);
       const f32x4 lse_o = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 32 * kb + 16));
       const f32x4 del_o = __builtin_bit_cast(f32x4, swa2_lds16(sDel + 32 * kb + 16));
       __builtin_amdgcn_sched_barrier(0);
       f32x4 dp1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int j = 0; j < 4; j++) dp1 = Mma<CT>::mfma(x[1][j], vf[j], dp1);
+      for (int c = 0; c < KC; c++) dp1 = Mma<CT>::mfma(x[1][c], vf[c], dp1);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 5: elementwise work of the odd column group
-      if (more) {
-        if (kb == 0) swa2_issue_one<2>(st, nrow, ndst);
-        if (kb == 1) swa2_issue_one<5>(st, nrow, ndst);
-        if (kb == 2) swa2_issue_one<8>(st, nrow, ndst);
-      }
-      if (kb == 0) swa2_read_tr<0, 2, 2>(sD, L, tr[1]);
-      if (kb == 1) swa2_read_tr<1, 2, 2>(sD, L, tr[1]);
-      if (kb == 2) swa2_read_tr<2, 2, 2>(sD, L, tr[1]);
+      if constexpr (more) swa2_issue_one<C, 4 * kb + 3>(st, nrow, ndst);
+      swa2_read_tr<C, kb, 2, 2>(sD, L, tr[1]);
       elementwise(1, s1, dp1, lse_o, del_o);
       __builtin_amdgcn_sched_barrier(0);
-      // ---- stage 6: dV^T += dO^T P, then dK^T += Q^T dS: eight pairs of 16-dim blocks
-      auto rd = [&](Swa2Lds reg, auto d0c, u32x4 (&dst)[2]) {
-        constexpr int D0 = decltype(d0c)::value;
-        if (kb == 0) swa2_read_tr<0, D0, 2>(reg, L, dst);
-        if (kb == 1) swa2_read_tr<1, D0, 2>(reg, L, dst);
-        if (kb == 2) swa2_read_tr<2, D0, 2>(reg, L, dst);
-        __builtin_amdgcn_sched_barrier(0);
-      };
-      auto pair = [&](f32x4 (&acc)[8], auto d0c, const u32x4& pk) {
-        constexpr int D0 = decltype(d0c)::value;
+      // ---- stage 6: dV^T += dO^T P over NP2 pairs of 16-dim blocks, then dK^T += Q^T dS over NP2 pairs.  Pair j of the
+      //      sequence sits in tr[j & 1]; pair j + 2 is requested once the products of pair j are issued, and the first
+      //      operands of the next 32 queries before the last pair.
+      swa2_for<0, 2 * NP2>([&](auto jc) {
+        constexpr int j = decltype(jc)::value;
+        constexpr int d0 = 2 * (j % NP2);
+        if constexpr (j == 2 * NP2 - 1 && kb + 1 < NKB) {
+          swa2_read_a<C, 2 * kb + 2>(sQ, L, x[0]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (j < NP2) {
 #pragma unroll
-        for (int d = 0; d < 2; d++) acc[D0 + d] = Mma<CT>::mfma(tr[(D0 >> 1) & 1][d], pk, acc[D0 + d]);
+          for (int d = 0; d < 2; d++) accv[d0 + d] = Mma<CT>::mfma(tr[j & 1][d], pp, accv[d0 + d]);
+        } else {
+#pragma unroll
+          for (int d = 0; d < 2; d++) acck[d0 + d] = Mma<CT>::mfma(tr[j & 1][d], pd, acck[d0 + d]);
+        }
         __builtin_amdgcn_sched_barrier(0);
-      };
-      typedef std::integral_constant<int, 0> I0;
-      typedef std::integral_constant<int, 2> I2;
-      typedef std::integral_constant<int, 4> I4;
-      typedef std::integral_constant<int, 6> I6;
-      pair(accv, I0{}, pp); rd(sD, I4{}, tr[0]);
-      pair(accv, I2{}, pp); rd(sD, I6{}, tr[1]);
-      pair(accv, I4{}, pp); rd(sQ, I0{}, tr[0]);
-      pair(accv, I6{}, pp); rd(sQ, I2{}, tr[1]);
-      pair(acck, I0{}, pd); rd(sQ, I4{}, tr[0]);
-      pair(acck, I2{}, pd); rd(sQ, I6{}, tr[1]);
-      pair(acck, I4{}, pd);
-      if (kb == 0) swa2_read_a<2>(sQ, L, x[0]);
-      if (kb == 1) swa2_read_a<4>(sQ, L, x[0]);
-      __builtin_amdgcn_sched_barrier(0);
-      pair(acck, I6{}, pd);
-    }
+        if constexpr (j + 2 < 2 * NP2) {
+          constexpr int j2 = j + 2;
+          if constexpr (j2 < NP2) swa2_read_tr<C, kb, 2 * j2, 2>(sD, L, tr[j & 1]);
+          else swa2_read_tr<C, kb, 2 * (j2 - NP2), 2>(sQ, L, tr[j & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+    });
   };
 
   // three loops, as in the dQ kernel
   const int act_lo = dlt_imax(G.ch_first, W.ch_lo), act_hi = dlt_imin(G.ch_last - 1, W.ch_hi);
   auto copy_only = [&](int ch) {
-    char* nxt = smem + ((ch + 1) & 1) * SWA2_BUF_KV;
+    char* nxt = smem + ((ch + 1) & 1) * C::BUF_KV;
     swa2_issue(st, G, ch + 1, sbase, srow, nxt, wave);
     issue_scalars(ch + 1, nxt);
     swa2_wait_copies();
@@ -429,15 +376,15 @@ __global__ __launch_bounds__(SWA2_THREADS) void swa2_bwd_kv_kernel(const Swa2Bwd
   int ch = G.ch_first;
   for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
   for (; ch <= act_hi; ch++) {
-    consume(ch, (Swa2Lds)smem + (ch & 1) * SWA2_BUF_KV, smem + ((ch + 1) & 1) * SWA2_BUF_KV, std::true_type{});
+    consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF_KV, smem + ((ch + 1) & 1) * C::BUF_KV, std::true_type{});
     swa2_wait_copies();
     __syncthreads();
   }
   for (; ch < G.ch_last; ch++) copy_only(ch);
   if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
-    consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * SWA2_BUF_KV, smem + ((G.ch_last + 1) & 1) * SWA2_BUF_KV, std::false_type{});
+    consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF_KV, smem + ((G.ch_last + 1) & 1) * C::BUF_KV, std::false_type{});
   __syncthreads();
 
-  swa2_store_own<TIO, CT>(smem + wave * 4096, accv, 1.f, dvb, a.dvs[2], G, r_p, c_p, lane);
-  swa2_store_own<TIO, CT>(smem + wave * 4096, acck, a.p.sm_scale, dkb, a.dks[2], G, r_p, c_p, lane);
+  swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, accv, 1.f, dvb, a.dvs[2], G, r_p, c_p, lane);
+  swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, acck, a.p.sm_scale, dkb, a.dks[2], G, r_p, c_p, lane);
 }

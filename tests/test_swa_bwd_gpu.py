@@ -51,6 +51,14 @@ def test_ragged_and_boundary_grids(th, tw, wr, wc):
     _run(2, 1, 3, 1, th, tw, wr, wc, 64, 64, torch.bfloat16)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("th,tw,wr,wc", [(7, 9, 2, 3), (9, 130, 3, 10), (20, 5, 6, 1), (6, 6, 8, 8), (33, 40, 10, 7), (17, 18, 0, 6)])
+def test_ragged_and_boundary_grids_head_dim_128(th, tw, wr, wc, dtype):
+    """Streaming kernels (head dim 128; windows up to 13 columns take four column groups per wave, wider ones six):
+    grids that are no multiple of the 8 x 16 band, windows wider than the grid, a window of one row."""
+    _run(22, 1, 2, 1, th, tw, wr, wc, 128, 128, dtype)
+
+
 def test_reference_demo_shape_b16():
     # src/tiled_swa.py:736-750: S=16 (4x4 px), 16x16 tiles, W=1, d=32, scale 0.25; B, H reduced
     _run(3, 1, 2, 16, 16, 16, 1, 1, 32, 32, torch.float16, scale=0.25)
