@@ -542,6 +542,9 @@ def main():
     extra["rope2d_c2"] = rope
     extra["copy_bandwidth"] = copy_bandwidth()
 
+    # the extra configs: long enough runs (tens of milliseconds of GPU time behind a warm-up) that the clock ramp after an
+    # idle phase does not weigh on the mean
+    XK, XW = max(K, 40), 8
     if not args.quick:
         # the same step when nothing but the caller's q, k is kept: every K / Q tile load of the backward
         # kernels rotates again (dlt_swa_fwd / dlt_swa_bwd with the rotary operands)
@@ -553,8 +556,8 @@ def main():
         del wl2
         for name, (B, H, th, tw, Wn, d) in {"C4_128x128": (1, 16, 128, 128, 10, 128), "C4_96x160": (1, 16, 96, 160, 10, 128)}.items():
             w4 = SwaWorkload(name, B, H, th, tw, Wn, d, fused_rope=False, nsets=1)
-            ms4, _ = Timer.run(w4.step, max(K // 5, 3), 2)
-            kb4 = kernel_breakdown(w4.step, 3)
+            ms4, _ = Timer.run(w4.step, XK, XW)
+            kb4 = kernel_breakdown(w4.step, 10)
             f4 = w4.flops_fwd + w4.flops_bwd
             extra[name] = {"ms_per_step": ms4, "eff_tflops": f4 / (ms4 * 1e-3) / 1e12,
                            "frac_mfma_peak": f4 / (ms4 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
@@ -562,7 +565,7 @@ def main():
             del w4
         # the reference's own demo shape (src/tiled_swa.py:736-750): 16-token tiles, generic kernels
         wd = SwaWorkload("ref_demo", 4, 8, 16, 16, 1, 32, fused_rope=False, nsets=1, dtype=torch.float16, b_size=16, scale=0.25)
-        msd, _ = Timer.run(wd.step, max(K // 5, 3), 2)
+        msd, _ = Timer.run(wd.step, XK, XW)
         fd = wd.flops_fwd + wd.flops_bwd
         extra["ref_demo_b16"] = {"ms_per_step": msd, "eff_tflops": fd / (msd * 1e-3) / 1e12,
                                  "workload": "B=4 H=8 16x16 tiles of 16 tokens, d=32, 3x3 window, fp16, fwd+bwd (src/tiled_swa.py:736-750)"}
@@ -573,8 +576,8 @@ def main():
         extra["ref_demo_image_layout"] = image_layout_demo(max(K // 5, 3))
         # larger tiles: B=2, H=8, 16x16 tiles of 64 tokens (N = 16384), d=64, 3x3 tile window, bf16
         wt = SwaWorkload("tiles_b64", 2, 8, 16, 16, 1, 64, fused_rope=False, nsets=1, b_size=64)
-        mst, _ = Timer.run(wt.step, max(K // 5, 3), 2)
-        kbt = kernel_breakdown(wt.step, 3)
+        mst, _ = Timer.run(wt.step, XK, XW)
+        kbt = kernel_breakdown(wt.step, 10)
         ft = wt.flops_fwd + wt.flops_bwd
         extra["tiles_b64_d64"] = {"ms_per_step": mst, "eff_tflops": ft / (mst * 1e-3) / 1e12,
                                   "frac_mfma_peak": ft / (mst * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
@@ -586,8 +589,8 @@ def main():
         ref = {}
         for causal in (False, True):
             wr = FlashWorkload(4, 32, 4096, 4096, 64, 64, dtype=torch.float16, causal=causal, scale=1.3)
-            ms_f, _ = Timer.run(wr.fwd_only, max(K // 5, 3), 2)
-            ms_s, _ = Timer.run(wr.step, max(K // 5, 3), 2)
+            ms_f, _ = Timer.run(wr.fwd_only, XK, XW)
+            ms_s, _ = Timer.run(wr.step, XK, XW)
             ref["causal" if causal else "non_causal"] = {
                 "fwd_ms": ms_f, "fwd_tflops": wr.flops_fwd / (ms_f * 1e-3) / 1e12,
                 "bwd_ms": ms_s - ms_f, "bwd_tflops": wr.flops_bwd / ((ms_s - ms_f) * 1e-3) / 1e12}
@@ -595,8 +598,8 @@ def main():
         ref["published_triton_fp16_unstated_hw_tflops"] = {"fwd_non_causal": 73.56, "fwd_causal": 71.11, "bwd_causal": 38.22}
         extra["flash_ref_b4_h32_d64_n4096_fp16"] = ref
         w5 = FlashWorkload(2, 16, 4096, 8192, 64, 128)
-        ms5, _ = Timer.run(w5.step, max(K // 5, 3), 2)
-        kb5 = kernel_breakdown(w5.step, 3)
+        ms5, _ = Timer.run(w5.step, XK, XW)
+        kb5 = kernel_breakdown(w5.step, 10)
         f5 = w5.flops_fwd + w5.flops_bwd
         extra["C5_flash"] = {"ms_per_step": ms5, "eff_tflops": f5 / (ms5 * 1e-3) / 1e12,
                              "frac_mfma_peak": f5 / (ms5 * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,

@@ -21,6 +21,8 @@
 #include <type_traits>
 #include "swa1_common.hpp"
 
+struct FlashTailDyn {};   // tag: whether a chunk needs the per-pair bound test is decided at run time
+
 // Streamed chunks in LDS: rows of 2 D + 32 bytes.  16-byte LDS accesses of a wave are served 16
 // lanes at a time, lanes {0-7, 16-23}, {8-15, 24-31}, ... together; with 64 banks a pitch of 16 k
 // bytes keeps the operand reads (16 rows x 16 bytes, and the transposing 8-byte reads) of such a group
@@ -293,8 +295,11 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
     const FlashChunk c = W.at(ci);
     return !TILE && (c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0));
   };
-  auto consume_t = [&](const int ci, auto tail_tag) {
-    constexpr bool tail = decltype(tail_tag)::value;
+  auto consume_t = [&](const int ci, auto tail_tag) __attribute__((always_inline)) {
+    // the tag is true_type / false_type (dense: known per call site) or FlashTailDyn (causal: tested per chunk)
+    bool tail;
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    else tail = decltype(tail_tag)::value;
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
     // causal: every key of the chunk lies above every query of this wave (wave-uniform)
@@ -409,8 +414,9 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   // The last chunk is peeled off so that prefetch and commit are unconditional inside the loop:
   // with `if (has_next)` around each, the compiler sees a path on which loads stay pending across
   // the back edge and guards every later load with a full vmcnt(0) wait.
-  auto consume = [&](const int ci) {
-    if (chunk_tail(ci)) consume_t(ci, std::true_type{});
+  auto consume = [&](const int ci) __attribute__((always_inline)) {
+    if (CAUSAL) consume_t(ci, FlashTailDyn{});
+    else if (chunk_tail(ci)) consume_t(ci, std::true_type{});
     else consume_t(ci, std::false_type{});
   };
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
@@ -624,8 +630,11 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
     const FlashChunk c = W.at(ci);
     return !TILE && (c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0));
   };
-  auto consume_t = [&](const int ci, auto tail_tag) {
-    constexpr bool tail = decltype(tail_tag)::value;
+  auto consume_t = [&](const int ci, auto tail_tag) __attribute__((always_inline)) {
+    // the tag is true_type / false_type (dense: known per call site) or FlashTailDyn (causal: tested per chunk)
+    bool tail;
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    else tail = decltype(tail_tag)::value;
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
     const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
@@ -684,8 +693,9 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
       }
     }
   };
-  auto consume = [&](const int ci) {
-    if (chunk_tail(ci)) consume_t(ci, std::true_type{});
+  auto consume = [&](const int ci) __attribute__((always_inline)) {
+    if (CAUSAL) consume_t(ci, FlashTailDyn{});
+    else if (chunk_tail(ci)) consume_t(ci, std::true_type{});
     else consume_t(ci, std::false_type{});
   };
   // last chunk peeled off: unconditional prefetch and commit inside the loop (see the forward kernel); without a causal
@@ -795,8 +805,11 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
     const FlashChunk c = W.at(ci);
     return !TILE && (c.nvalid < CK || (CAUSAL && c.x < wk0 + 16 * NP - 1));
   };
-  auto consume_t = [&](const int ci, auto tail_tag) {
-    constexpr bool tail = decltype(tail_tag)::value;
+  auto consume_t = [&](const int ci, auto tail_tag) __attribute__((always_inline)) {
+    // the tag is true_type / false_type (dense: known per call site) or FlashTailDyn (causal: tested per chunk)
+    bool tail;
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    else tail = decltype(tail_tag)::value;
     const FlashChunk c = W.at(ci);
     const int q0 = c.x;
     // causal: every query of the chunk lies below every own key of this wave
@@ -867,8 +880,9 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
       }
     }
   };
-  auto consume = [&](const int ci) {
-    if (chunk_tail(ci)) consume_t(ci, std::true_type{});
+  auto consume = [&](const int ci) __attribute__((always_inline)) {
+    if (CAUSAL) consume_t(ci, FlashTailDyn{});
+    else if (chunk_tail(ci)) consume_t(ci, std::true_type{});
     else consume_t(ci, std::false_type{});
   };
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
