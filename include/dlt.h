@@ -79,7 +79,7 @@ int dlt_rope_pe_mask(const int32_t* idx, int64_t n_tokens, uint8_t* bits, void* 
 typedef struct {
   int32_t B, H;
   int32_t b_size, t_height, t_width, row_size, col_size;
-  int32_t dk, dv; /* q/k head dim, v/o head dim */
+  int32_t dk, dv; /* q/k head dim, v/o head dim: 1..256 each (larger: DLT_ERR_UNSUPPORTED) */
   float sm_scale; /* must be finite (else DLT_ERR_INVALID); any sign is accepted as in the reference, which scales
                      before taking the row max: the tuned kernels keep the max of the raw scores and take positive
                      scales only, zero and negative scales run on the generic kernels */
