@@ -61,7 +61,10 @@ constexpr int flash_ck_fwd(int dk, int dv) { return FLASH_CK_FWD(dk, dv); }
 constexpr int flash_ck_q(int dk, int dv) { return FLASH_CK_Q(dk, dv); }
 constexpr int flash_ck_kv(int dk, int dv) { return FLASH_CK_KV(dk, dv); }
 // key blocks per wave in the dK/dV kernel: its two accumulator sets only fit twice for small dims
-constexpr int flash_np_kv(int dk, int dv) { return dk + dv > 192 ? 1 : 2; }
+#ifndef FLASH_NP_KV
+#define FLASH_NP_KV(dk, dv) ((dk) + (dv) > 192 ? 1 : 2)
+#endif
+constexpr int flash_np_kv(int dk, int dv) { return FLASH_NP_KV(dk, dv); }
 // query blocks per wave in the dQ kernel: one at 128/128 (accumulators, q and dO fragments of two blocks do not fit 256 registers)
 constexpr int flash_np_q(int dk, int dv) { return dk + dv > 192 ? 1 : FLASH_NP_DEF; }
 // resident workgroups per CU the register allocation aims for (spill-free at these settings)
