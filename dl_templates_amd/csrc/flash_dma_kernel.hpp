@@ -78,18 +78,19 @@ struct FlashDStage {
       const int t = tok0 + R::TPI * i;
       const uint32_t off = ad(c, dlt_imin(t, c.nvalid - 1)) + 16u * (uint32_t)(lp ^ (R::SWZ * (t & 7)));
       char* dst = region + (wave * (CK / 4) + R::TPI * i) * R::ROW;   // wave-uniform
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + off), (DLT_LDS void*)dst, 16, 0, 0);
+      dlt_copy16_to_lds(base, off, dst);
     }
   }
 };
 
-// per-token fp32 scalars of a chunk: 64 tokens per instruction, 4 bytes per lane
+// per-token fp32 scalars of a chunk: 64 tokens per instruction, 4 bytes per lane (32-bit byte offsets inside a
+// (batch, head) slab: checked by the host)
 template <int CK>
-DLT_DEV void flashd_issue_scalars(const float* base, int64_t stride, const FlashChunk& c, char* dst, int lane) {
+DLT_DEV void flashd_issue_scalars(const float* base, int stride, const FlashChunk& c, char* dst, int lane) {
 #pragma unroll
   for (int j = 0; j < CK / 64; j++) {
-    const int64_t tok = c.tok0 + dlt_imin(64 * j + lane, c.nvalid - 1);
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(base + tok * stride), (DLT_LDS void*)(dst + 256 * j), 4, 0, 0);
+    const uint32_t off = (uint32_t)((c.tok0 + dlt_imin(64 * j + lane, c.nvalid - 1)) * stride) * 4u;
+    dlt_copy4_to_lds(reinterpret_cast<const char*>(base), off, dst + 256 * j);
   }
 }
 
@@ -155,7 +156,7 @@ __global__ __launch_bounds__(256, NP >= 4 ? 1 : 2) void flashd_bwd_kv_kernel(con
   auto issue = [&](const FlashChunk& c, char* buf) {
     stq.issue(qb, aq, c, buf, wave);
     std_.issue(dob, ad, c, buf + B::REG_A, wave);
-    if (wave < 2) flashd_issue_scalars<CK>(scal_base, a.ls[2], c, buf + B::REG_A + B::REG_B + wave * (CK * 4), lane);
+    if (wave < 2) flashd_issue_scalars<CK>(scal_base, (int)a.ls[2], c, buf + B::REG_A + B::REG_B + wave * (CK * 4), lane);
   };
   constexpr int NBUF = flashd_nbuf(DK, DV), AHEAD = NBUF - 1;
   constexpr int PER_CHUNK = FlashDStage<DK, CK>::NI + FlashDStage<DV, CK>::NI;   // copies per wave and chunk (waves 0, 1: more)

@@ -233,7 +233,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
     const char* row = reinterpret_cast<const char*>(scal_base) + (uint32_t)(r * G.TC * ls2) * 4u;   // wave-uniform
     char* dst = buf + C::BUF + (wave >> 2) * (C::TOK * 4) + (wave & 3) * (C::HCW * 4);
     if (lane < C::HCW)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(row + scal_off), (DLT_LDS void*)dst, 4, 0, 0);
+      dlt_copy4_to_lds(row, scal_off, dst);
   };
   swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF_KV, wave);
   issue_scalars(G.ch_first, smem + (G.ch_first & 1) * C::BUF_KV);

@@ -116,6 +116,21 @@ DLT_DEV bool swa2_visible(const Swa2Win& W, bool row_vis, int cg, int i, int ncg
   return row_vis & (cg < ncg) & ((unsigned)(4 * cg + i - W.clo) <= (unsigned)W.cspan);
 }
 
+// One copy instruction as the hardware sees it: 64 lanes x 16 (or 4) bytes from `base + voff` (base wave-uniform)
+// to the LDS address `lds` + 16 (4) lane.  It is issued from inline assembly on purpose: the compiler models the
+// instruction as a flat access that may touch LDS, and while one is in flight it turns every wait for an LDS read into
+// a wait for ALL outstanding LDS reads (lgkmcnt(0)) and for all outstanding copies (vmcnt(0)), which serialises the
+// operand read-ahead of the loops that overlap copies with products.  Hidden from its counters, the waits for operand
+// reads are exact again; the waits for the copies themselves are explicit (swa2_wait_copies).
+DLT_DEV void dlt_copy16_to_lds(const char* base, uint32_t voff, char* lds) {
+  const uint32_t m = (uint32_t)(uintptr_t)(DLT_LDS char*)lds;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(base), "v"(voff), "s"(m) : "memory");
+}
+DLT_DEV void dlt_copy4_to_lds(const char* base, uint32_t voff, char* lds) {
+  const uint32_t m = (uint32_t)(uintptr_t)(DLT_LDS char*)lds;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, %0" ::"s"(base), "v"(voff), "s"(m) : "memory");
+}
+
 // ---- asynchronous staging -------------------------------------------------------------------------------
 // Wave w copies halo row (w & 3) of tensor (w >> 2) of every chunk in NI instructions of 64 lanes; instruction i,
 // lane l writes LDS slot 64 i + l of the row = physical piece l % PIECES of halo column TPI i + l / PIECES, and
@@ -145,8 +160,7 @@ template <typename C, int I>
 DLT_DEV void swa2_issue_one(const Swa2Stage<C>& st, const char* row, char* dst) {
   if constexpr (I < C::NI) {
     if (I + 1 < C::NI || C::HCW % C::TPI == 0 || st.last_on)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(row + st.off[I]), (DLT_LDS void*)(dst + 1024 * I),
-                                       16, 0, 0);
+      dlt_copy16_to_lds(row, st.off[I], dst + 1024 * I);
   }
 }
 DLT_DEV const char* swa2_issue_row(const Swa2Geom& G, int ch, const char* base, uint32_t rowstride, int wave) {
