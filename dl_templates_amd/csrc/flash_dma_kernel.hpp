@@ -56,18 +56,19 @@ DLT_DEV u32x4 flashd_read_tr(Swa2Lds tile, const FlashDLane<D>& L, int d) {
   return r;
 }
 
-// Copy of one chunk of CK tokens of a [token][D] tensor by the 4 waves of a workgroup: wave w copies tokens
-// w CK / 4 .. + CK / 4 - 1 in NI instructions; instruction i, lane l writes LDS slot l of its 1 KB = physical piece
-// l % PIECES of token w CK / 4 + TPI i + l / PIECES, and therefore fetches the logical piece (l % PIECES) ^ (SWZ (token & 7)).
-template <int D, int CK>
+// Copy of one chunk of CK tokens of a [token][D] tensor by the NW waves of a workgroup: wave w copies tokens
+// w CK / NW .. + CK / NW - 1 in NI instructions; instruction i, lane l writes LDS slot l of its 1 KB = physical piece
+// l % PIECES of token w CK / NW + TPI i + l / PIECES, and therefore fetches the logical piece (l % PIECES) ^ (SWZ (token & 7)).
+template <int D, int CK, int NW = 4>
 struct FlashDStage {
   typedef FlashDRow<D> R;
-  static constexpr int NI = CK / 4 / R::TPI;
+  static constexpr int NI = CK / NW / R::TPI;
+  static_assert(NI >= 1 && NI * R::TPI * NW == CK, "chunk must split evenly over the waves' copy instructions");
   int tok0;   // token of the lane in instruction 0
   int lp;     // physical piece the lane writes
 
   DLT_DEV void init(int wave, int lane) {
-    tok0 = wave * (CK / 4) + lane / R::PIECES;
+    tok0 = wave * (CK / NW) + lane / R::PIECES;
     lp = lane % R::PIECES;
   }
   // tokens past the end of the chunk are clamped onto its last token (the caller masks them)
@@ -77,7 +78,7 @@ struct FlashDStage {
     for (int i = 0; i < NI; i++) {
       const int t = tok0 + R::TPI * i;
       const uint32_t off = ad(c, dlt_imin(t, c.nvalid - 1)) + 16u * (uint32_t)(lp ^ (R::SWZ * (t & 7)));
-      char* dst = region + (wave * (CK / 4) + R::TPI * i) * R::ROW;   // wave-uniform
+      char* dst = region + (wave * (CK / NW) + R::TPI * i) * R::ROW;   // wave-uniform
       dlt_copy16_to_lds(base, off, dst);
     }
   }
@@ -94,6 +95,11 @@ DLT_DEV void flashd_issue_scalars(const float* base, int stride, const FlashChun
   }
 }
 
+// operands the LDS reads of a chunk loop run ahead of their products
+#ifndef FLASHD_RD
+#define FLASHD_RD 3
+#endif
+
 // at most N of this wave's copies (the youngest ones) are still in flight
 template <int N>
 DLT_DEV void flashd_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -104,6 +110,10 @@ DLT_DEV void flashd_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) 
 #define FLASHD_NBUF(dk, dv) ((dk) + (dv) > 192 ? 2 : 3)
 #endif
 constexpr int flashd_nbuf(int dk, int dv) { return FLASHD_NBUF(dk, dv); }
+// 8-wave workgroups of the backward kernels (one per CU, 64-token chunks)
+#ifndef FLASHD_NBUF8
+#define FLASHD_NBUF8 3
+#endif
 
 template <int DK, int DV, int CK>
 struct FlashDBuf {
@@ -115,14 +125,14 @@ struct FlashDBuf {
 };
 
 // ---- dK / dV: own = keys; Q, dO, lse2 and delta stream.  Replaces _attn_bwd_dkdv (src/flash_attn.py:204-307).
-template <typename TIO, int DK, int DV, int NP, int CK, int MODE>
-__global__ __launch_bounds__(256, NP >= 4 ? 1 : 2) void flashd_bwd_kv_kernel(const FlashBwdArgs a) {
+template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef FlashDBuf<DK, DV, CK> B;
   extern __shared__ __align__(16) char smem[];
   constexpr bool CAUSAL = MODE == 1, TILE = MODE >= 2, IMG = MODE == 3;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16, NQB = CK / 32;
-  constexpr int OWN = 64 * NP;
+  constexpr int OWN = 16 * NP * NW;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -147,8 +157,8 @@ __global__ __launch_bounds__(256, NP >= 4 ? 1 : 2) void flashd_bwd_kv_kernel(con
   else W.init_seq(CAUSAL ? (x0 / CK) * CK : 0, a.Lq);
   const int wk0 = x0 + wave * 16 * NP;  // first own key of this wave
 
-  FlashDStage<DK, CK> stq;
-  FlashDStage<DV, CK> std_;
+  FlashDStage<DK, CK, NW> stq;
+  FlashDStage<DV, CK, NW> std_;
   stq.init(wave, lane);
   std_.init(wave, lane);
   // waves 0 and 1 also copy the chunk's lse2 / delta
@@ -158,8 +168,8 @@ __global__ __launch_bounds__(256, NP >= 4 ? 1 : 2) void flashd_bwd_kv_kernel(con
     std_.issue(dob, ad, c, buf + B::REG_A, wave);
     if (wave < 2) flashd_issue_scalars<CK>(scal_base, (int)a.ls[2], c, buf + B::REG_A + B::REG_B + wave * (CK * 4), lane);
   };
-  constexpr int NBUF = flashd_nbuf(DK, DV), AHEAD = NBUF - 1;
-  constexpr int PER_CHUNK = FlashDStage<DK, CK>::NI + FlashDStage<DV, CK>::NI;   // copies per wave and chunk (waves 0, 1: more)
+  constexpr int NBUF = NW == 4 ? flashd_nbuf(DK, DV) : FLASHD_NBUF8, AHEAD = NBUF - 1;
+  constexpr int PER_CHUNK = FlashDStage<DK, CK, NW>::NI + FlashDStage<DV, CK, NW>::NI;   // copies per wave and chunk (waves 0, 1: more)
 #pragma unroll
   for (int i = 0; i < AHEAD; i++)
     if (i < W.nchunks) issue(W.at(i), smem + i * B::BUF_KV);
@@ -219,9 +229,6 @@ __global__ __launch_bounds__(256, NP >= 4 ? 1 : 2) void flashd_bwd_kv_kernel(con
     // causal: every query of the chunk lies below every own key of this wave
     if (CAUSAL && q0 + CK - 1 < wk0) return;
     constexpr int N1H = KC + VC, N1 = 2 * N1H, NB = N1 + VB + KB, NT = NQB * NB;
-#ifndef FLASHD_RD
-#define FLASHD_RD 3
-#endif
     constexpr int RD = FLASHD_RD;
     u32x4 ring[RD + 1];
     auto rd = [&](auto kc) __attribute__((always_inline)) {
@@ -328,6 +335,400 @@ __global__ __launch_bounds__(256, NP >= 4 ? 1 : 2) void flashd_bwd_kv_kernel(con
   __syncthreads();
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
-  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, flash_tok<IMG>(a.dks, a.tm), a.dks[3], a.dk_, a.dk_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
-  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, flash_tok<IMG>(a.dvs, a.tm), a.dvs[3], a.dv_, a.dv_vec != 0, own_base, x0, a.Lk, wave, n, g, tid);
+  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, flash_tok<IMG>(a.dks, a.tm), a.dks[3], a.dk_, a.dk_vec != 0, own_base, x0, a.Lk, wave, n, g, tid, OWN);
+  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, flash_tok<IMG>(a.dvs, a.tm), a.dvs[3], a.dv_, a.dv_vec != 0, own_base, x0, a.Lk, wave, n, g, tid, OWN);
+}
+
+// ---- forward: own = queries; K and V stream.  Replaces _attn_fwd (src/flash_attn.py:81-172).
+// Per chunk: S^T = K Q^T for every 32-key block (a stream of NKB 2 KC operand reads, NP products each), one softmax
+// update per query block, then O^T += V^T P^T (NKB VB transposed operands) with the row sums from a ones-row product.
+// The reads of the second stream are already in flight while the softmax runs.
+template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(const FlashArgs a) {
+  typedef typename ComputeOf<TIO>::type CT;
+  typedef typename TileOf<TIO>::type TL;
+  typedef FlashDBuf<DK, DV, CK> B;
+  extern __shared__ __align__(16) char smem[];
+  constexpr bool CAUSAL = MODE == 1;
+  static_assert(MODE < 2, "asynchronous staging: dense and causal only");
+  constexpr int PO = DV * (int)sizeof(TL) + 16;
+  constexpr int KC = DK / 32, VB = DV / 16, NKB = CK / 32;
+  constexpr int OWN = 16 * NP * NW;
+  constexpr int NBUF = NW == 4 ? flashd_nbuf(DK, DV) : 2, AHEAD = NBUF - 1;   // forward: 128-key chunks
+  constexpr int PER_CHUNK = FlashDStage<DK, CK, NW>::NI + FlashDStage<DV, CK, NW>::NI;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int lin = xcd_remap(blockIdx.x, gridDim.x);
+  int bh, r_own, x0;
+  flash_block(lin, a.nblk, 1, OWN, CAUSAL, bh, r_own, x0);
+  const int wq0 = x0 + wave * 16 * NP;
+  const int b = bh / a.H, h = bh - b * a.H;
+  const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
+  const char* kb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1]);
+  const char* vb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1]);
+  TIO* ob = reinterpret_cast<TIO*>(a.o) + b * a.os[0] + h * a.os[1];
+  const FlashAddr<false> ak = flash_addr<false>(a.ks, a.tm), av = flash_addr<false>(a.vs, a.tm);
+  RopeDev no_rope = RopeDev{};
+
+  FlashWalk<MODE, CK> W;
+  W.init_seq(0, CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk);
+
+  FlashDStage<DK, CK, NW> stk;
+  FlashDStage<DV, CK, NW> stv;
+  stk.init(wave, lane);
+  stv.init(wave, lane);
+  auto issue = [&](const FlashChunk& c, char* buf) {
+    stk.issue(kb_, ak, c, buf, wave);
+    stv.issue(vb_, av, c, buf + B::REG_A, wave);
+  };
+#pragma unroll
+  for (int i = 0; i < AHEAD; i++)
+    if (i < W.nchunks) issue(W.at(i), smem + i * B::BUF);
+
+  u32x4 qf[NP][KC];
+  int64_t tq[NP];
+  int klim[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int xq = wq0 + 16 * p + n;
+    tq[p] = xq < a.Lq ? (int64_t)xq : (int64_t)-1;
+    klim[p] = CAUSAL ? dlt_imin(xq, a.Lk - 1) : a.Lk - 1;
+    swa1_load_own<TIO, CT, DK>(qf[p], qb, 1, a.dk, flash_own_off<false>(a.qs, a.tm, tq[p]), g, no_rope, false);
+  }
+  float m_run[NP];
+  f32x4 acc[NP][VB], acc_l[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    m_run[p] = -INFINITY;
+    acc_l[p] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int d = 0; d < VB; d++) acc[p][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float scale = a.scale_log2;
+  const unsigned one2 = pack2<CT>(1.f, 1.f);
+  const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
+  FlashDLane<DK> LK;
+  FlashDLane<DV> LV;
+  flashd_lane_init(LK, n, g);
+  flashd_lane_init(LV, n, g);
+
+  swa2_wait_copies();   // also: the own fragments have arrived
+  __syncthreads();
+
+  auto chunk_tail = [&](const int ci) {
+    const FlashChunk c = W.at(ci);
+    return c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0);
+  };
+  auto consume_t = [&](const int ci, Swa2Lds __restrict__ cur, char* __restrict__ nxt, auto tail_tag, auto more_tag) __attribute__((always_inline)) {
+    bool tail;
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    else tail = decltype(tail_tag)::value;
+    if constexpr (decltype(more_tag)::value) issue(W.at(ci + AHEAD), nxt);
+    Swa2Lds sK = cur, sV = cur + B::REG_A;
+    const FlashChunk c = W.at(ci);
+    const int k0 = c.x;
+    // causal: every key of the chunk lies above every query of this wave
+    if (CAUSAL && k0 > wq0 + 16 * NP - 1) return;
+    constexpr int N1 = NKB * 2 * KC, NT = N1 + NKB * VB;
+    constexpr int RD = FLASHD_RD;
+    u32x4 ring[RD + 1];
+    auto rd = [&](auto kc) __attribute__((always_inline)) {
+      constexpr int k = decltype(kc)::value;
+      if constexpr (k < N1) {
+        constexpr int kb = k / (2 * KC), mb = (k / KC) % 2, r = k % KC;
+        ring[k % (RD + 1)] = swa2_lds16(sK + (32 * kb + 16 * mb) * FlashDRow<DK>::ROW + LK.a[r]);
+      } else {
+        constexpr int kb = (k - N1) / VB, d = (k - N1) % VB;
+        ring[k % (RD + 1)] = flashd_read_tr<DV, 32 * kb>(sV, LV, d);
+      }
+    };
+    swa2_for<0, RD>([&](auto kc) __attribute__((always_inline)) { rd(kc); });
+    float t[NP][NKB][8];
+    u32x4 pb[NP][NKB];
+    f32x4 s[NP];
+    swa2_for<0, NT>([&](auto kc) __attribute__((always_inline)) {
+      constexpr int k = decltype(kc)::value;
+      if constexpr (k + RD < NT) rd(std::integral_constant<int, k + RD>{});
+      __builtin_amdgcn_sched_barrier(0);
+      const u32x4 x = ring[k % (RD + 1)];
+      if constexpr (k < N1) {
+        constexpr int kb = k / (2 * KC), mb = (k / KC) % 2, r = k % KC;
+#pragma unroll
+        for (int p = 0; p < NP; p++) s[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[p]);
+        if constexpr (r == KC - 1) {
+#pragma unroll
+          for (int p = 0; p < NP; p++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+              float v = s[p][i];
+              if (tail) v = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? v : -INFINITY;
+              t[p][kb][4 * mb + i] = v;
+            }
+        }
+        if constexpr (k == N1 - 1) {
+          // one softmax update per query block on the raw scores of the chunk
+#pragma unroll
+          for (int p = 0; p < NP; p++) {
+            float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+#pragma unroll
+            for (int kb2 = 0; kb2 < NKB; kb2++)
+#pragma unroll
+              for (int i = 0; i < 4; i++) mx[i] = fmaxf(fmaxf(mx[i], t[p][kb2][2 * i]), t[p][kb2][2 * i + 1]);
+            const float mloc = wave_max4(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])));
+            // the reference maximum only moves when a score exceeds it by more than 2^8 after scaling (see flash_kernel.hpp)
+            if (__builtin_amdgcn_ballot_w64((mloc - m_run[p]) * scale > 8.f)) {
+              keep_branch();
+              const float m_new = fmaxf(m_run[p], mloc);
+              const float alpha = fast_exp2((m_run[p] - m_new) * scale);
+              m_run[p] = m_new;
+#pragma unroll
+              for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
+              acc_l[p] *= alpha;
+            }
+            const float neg_m2 = m_run[p] == -INFINITY ? 0.f : -m_run[p] * scale;
+#pragma unroll
+            for (int kb2 = 0; kb2 < NKB; kb2++) {
+#pragma unroll
+              for (int i = 0; i < 8; i++) t[p][kb2][i] = fast_exp2(fmaf(t[p][kb2][i], scale, neg_m2));
+              pb[p][kb2] = pack8<CT>(t[p][kb2]);
+            }
+          }
+        }
+      } else {
+        constexpr int kb = (k - N1) / VB, d = (k - N1) % VB;
+#pragma unroll
+        for (int p = 0; p < NP; p++) acc[p][d] = Mma<CT>::mfma(x, pb[p][kb], acc[p][d]);
+        if constexpr (d == VB - 1) {
+#pragma unroll
+          for (int p = 0; p < NP; p++) acc_l[p] = Mma<CT>::mfma(ones, pb[p][kb], acc_l[p]);
+        }
+      }
+    });
+  };
+  int ci = 0, bi = 0;
+  auto buf_of = [&](int i) { return smem + (i >= NBUF ? i - NBUF : i) * B::BUF; };
+  for (; ci + AHEAD < W.nchunks; ci++) {
+    if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
+    flashd_wait_copies<PER_CHUNK>();
+    __syncthreads();
+    bi = bi + 1 == NBUF ? 0 : bi + 1;
+  }
+  for (; ci + 1 < W.nchunks; ci++) {
+    if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
+    swa2_wait_copies();
+    __syncthreads();
+    bi = bi + 1 == NBUF ? 0 : bi + 1;
+  }
+  if (W.nchunks > 0) {
+    if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
+    else if (chunk_tail(ci)) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
+  }
+  __syncthreads();
+
+  // ---- epilogue: normalise, O^T fragments -> LDS tile -> coalesced rows
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const float lt = wave_sum4(acc_l[p][0]);
+    const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
+    TL* orow = reinterpret_cast<TL*>(smem + (wave * 16 * NP + 16 * p + n) * PO);
+#pragma unroll
+    for (int d = 0; d < VB; d++)
+#pragma unroll
+      for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * inv);
+    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
+  }
+  __syncthreads();
+  if (tid < 256)   // the tile writer walks the rows with 256 threads
+    store_tile<TIO, TL, DV>(smem, PO, ob, flash_tok<false>(a.os, a.tm), a.os[3], a.dv, a.o_vec != 0, OWN,
+                            [&](int row) { return x0 + row < a.Lq ? (int64_t)(x0 + row) : (int64_t)-1; }, no_rope, tid);
+}
+
+// ---- dQ: own = queries; K and V stream.  Replaces _attn_bwd_dq (src/flash_attn.py:310-449) and, with fuse_delta, the
+// delta pre-pass (:186-202).  Per 32-key block: per 16-key half KC pieces of K (S = K Q^T) and VC pieces of V
+// (dP = V dO^T), then KB transposed pieces of K (dQ^T += K^T dS).
+template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE>
+__global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(const FlashBwdArgs a) {
+  typedef typename ComputeOf<TIO>::type CT;
+  typedef FlashDBuf<DK, DV, CK> B;
+  extern __shared__ __align__(16) char smem[];
+  constexpr bool CAUSAL = MODE == 1;
+  static_assert(MODE < 2, "asynchronous staging: dense and causal only");
+  constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, NKB = CK / 32;
+  constexpr int OWN = 16 * NP * NW;
+  constexpr int NBUF = NW == 4 ? flashd_nbuf(DK, DV) : FLASHD_NBUF8, AHEAD = NBUF - 1;
+  constexpr int PER_CHUNK = FlashDStage<DK, CK, NW>::NI + FlashDStage<DV, CK, NW>::NI;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, n = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+  const int lin = xcd_remap(blockIdx.x, gridDim.x);
+  int bh, r_own, x0;
+  flash_block(lin, a.nblk_q, 1, OWN, CAUSAL, bh, r_own, x0);
+  const int wq0 = x0 + wave * 16 * NP;
+  const int b = bh / a.H, h = bh - b * a.H;
+  const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
+  const TIO* dob = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1];
+  const char* kb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1]);
+  const char* vb_ = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1]);
+  const FlashAddr<false> ak = flash_addr<false>(a.ks, a.tm), av = flash_addr<false>(a.vs, a.tm);
+  RopeDev no_rope = RopeDev{};
+
+  FlashWalk<MODE, CK> W;
+  W.init_seq(0, CAUSAL ? dlt_imin(a.Lk, x0 + OWN) : a.Lk);
+
+  FlashDStage<DK, CK, NW> stk;
+  FlashDStage<DV, CK, NW> stv;
+  stk.init(wave, lane);
+  stv.init(wave, lane);
+  auto issue = [&](const FlashChunk& c, char* buf) {
+    stk.issue(kb_, ak, c, buf, wave);
+    stv.issue(vb_, av, c, buf + B::REG_A, wave);
+  };
+#pragma unroll
+  for (int i = 0; i < AHEAD; i++)
+    if (i < W.nchunks) issue(W.at(i), smem + i * B::BUF);
+
+  u32x4 qf[NP][KC], dof[NP][VC];
+  float nlse[NP], del_n[NP];
+  int klim[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    const int xq = wq0 + 16 * p + n;
+    const int64_t tq = xq < a.Lq ? (int64_t)xq : (int64_t)-1;
+    klim[p] = CAUSAL ? dlt_imin(xq, a.Lk - 1) : a.Lk - 1;
+    swa1_load_own<TIO, CT, DK>(qf[p], qb, 1, a.dk_, flash_own_off<false>(a.qs, a.tm, tq), g, no_rope, false);
+    swa1_load_own<TIO, CT, DV>(dof[p], dob, 1, a.dv_, flash_own_off<false>(a.dos, a.tm, tq), g, no_rope, false);
+    const int64_t off = b * a.ls[0] + h * a.ls[1] + (tq >= 0 ? tq : 0) * a.ls[2];
+    nlse[p] = tq >= 0 ? -a.lse[off] : 0.f;
+    if (a.fuse_delta != 0) {
+      const TIO* ob = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1];
+      u32x4 of[VC];
+      swa1_load_own<TIO, CT, DV>(of, ob, 1, a.dv_, flash_own_off<false>(a.os, a.tm, tq), g, no_rope, false);
+      float part = 0.f;
+#pragma unroll
+      for (int c_ = 0; c_ < VC; c_++) {
+        float fo[8], fd[8];
+        unpack8<CT>(of[c_], fo);
+        unpack8<CT>(dof[p][c_], fd);
+#pragma unroll
+        for (int j = 0; j < 8; j++) part += fo[j] * fd[j];
+      }
+      del_n[p] = wave_sum4(part);
+      if (g == 0 && tq >= 0) a.delta_out[off] = del_n[p];
+    } else {
+      del_n[p] = tq >= 0 ? a.delta[off] : 0.f;
+    }
+  }
+  f32x4 dq_acc[NP][KB];
+#pragma unroll
+  for (int p = 0; p < NP; p++)
+#pragma unroll
+    for (int d = 0; d < KB; d++) dq_acc[p][d] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const float scale = a.scale_log2;
+  FlashDLane<DK> LK;
+  FlashDLane<DV> LV;
+  flashd_lane_init(LK, n, g);
+  flashd_lane_init(LV, n, g);
+
+  swa2_wait_copies();   // also: the own fragments and scalars have arrived
+  __syncthreads();
+
+  auto chunk_tail = [&](const int ci) {
+    const FlashChunk c = W.at(ci);
+    return c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0);
+  };
+  auto consume_t = [&](const int ci, Swa2Lds __restrict__ cur, char* __restrict__ nxt, auto tail_tag, auto more_tag) __attribute__((always_inline)) {
+    bool tail;
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    else tail = decltype(tail_tag)::value;
+    if constexpr (decltype(more_tag)::value) issue(W.at(ci + AHEAD), nxt);
+    Swa2Lds sK = cur, sV = cur + B::REG_A;
+    const FlashChunk c = W.at(ci);
+    const int k0 = c.x;
+    if (CAUSAL && k0 > wq0 + 16 * NP - 1) return;
+    constexpr int N1H = KC + VC, N1 = 2 * N1H, NB = N1 + KB, NT = NKB * NB;
+    constexpr int RD = FLASHD_RD;
+    u32x4 ring[RD + 1];
+    auto rd = [&](auto kc) __attribute__((always_inline)) {
+      constexpr int k = decltype(kc)::value;
+      constexpr int kb = k / NB, j = k % NB;
+      if constexpr (j < N1) {
+        constexpr int mb = j / N1H, r = j % N1H, T0 = 32 * kb + 16 * mb;
+        if constexpr (r < KC) ring[k % (RD + 1)] = swa2_lds16(sK + T0 * FlashDRow<DK>::ROW + LK.a[r]);
+        else ring[k % (RD + 1)] = swa2_lds16(sV + T0 * FlashDRow<DV>::ROW + LV.a[r - KC]);
+      } else {
+        ring[k % (RD + 1)] = flashd_read_tr<DK, 32 * kb>(sK, LK, j - N1);
+      }
+    };
+    swa2_for<0, RD>([&](auto kc) __attribute__((always_inline)) { rd(kc); });
+    swa2_for<0, NKB>([&](auto kbc) __attribute__((always_inline)) {
+      constexpr int kb = decltype(kbc)::value;
+      float ds[NP][8];
+      f32x4 sv[NP], dp[NP];
+      u32x4 dsb[NP];
+      swa2_for<0, NB>([&](auto jc) __attribute__((always_inline)) {
+        constexpr int j = decltype(jc)::value, k = kb * NB + j;
+        if constexpr (k + RD < NT) rd(std::integral_constant<int, k + RD>{});
+        __builtin_amdgcn_sched_barrier(0);
+        const u32x4 x = ring[k % (RD + 1)];
+        if constexpr (j < N1) {
+          constexpr int mb = j / N1H, r = j % N1H;
+#pragma unroll
+          for (int p = 0; p < NP; p++) {
+            if constexpr (r < KC) sv[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sv[p]);
+            else dp[p] = Mma<CT>::mfma(x, dof[p][r - KC], r == KC ? f32x4{0.f, 0.f, 0.f, 0.f} : dp[p]);
+          }
+          if constexpr (r == N1H - 1) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+#pragma unroll
+              for (int i = 0; i < 4; i++) {
+                float pv = fast_exp2(fmaf(sv[p][i], scale, nlse[p]));
+                if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? pv : 0.f;
+                ds[p][4 * mb + i] = pv * (dp[p][i] - del_n[p]);
+              }
+            }
+            if constexpr (mb == 1) {
+#pragma unroll
+              for (int p = 0; p < NP; p++) dsb[p] = pack8<CT>(ds[p]);
+            }
+          }
+        } else {
+#pragma unroll
+          for (int p = 0; p < NP; p++) dq_acc[p][j - N1] = Mma<CT>::mfma(x, dsb[p], dq_acc[p][j - N1]);
+        }
+      });
+    });
+  };
+  int ci = 0, bi = 0;
+  auto buf_of = [&](int i) { return smem + (i >= NBUF ? i - NBUF : i) * B::BUF; };
+  for (; ci + AHEAD < W.nchunks; ci++) {
+    if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
+    flashd_wait_copies<PER_CHUNK>();
+    __syncthreads();
+    bi = bi + 1 == NBUF ? 0 : bi + 1;
+  }
+  for (; ci + 1 < W.nchunks; ci++) {
+    if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
+    swa2_wait_copies();
+    __syncthreads();
+    bi = bi + 1 == NBUF ? 0 : bi + 1;
+  }
+  if (W.nchunks > 0) {
+    if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
+    else if (chunk_tail(ci)) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
+  }
+  __syncthreads();
+  TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
+  flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, flash_tok<false>(a.dqs, a.tm), a.dqs[3], a.dk_, a.dq_vec != 0, 0, x0, a.Lq, wave, n, g, tid, OWN);
 }

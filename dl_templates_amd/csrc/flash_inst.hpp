@@ -7,8 +7,49 @@
 #define DLT_FCAT3(a, b, c) DLT_FCAT3_(a, b, c)
 
 namespace {
+// shape of the asynchronously staged forward kernel: keys per chunk, waves per workgroup (16 NP queries per wave)
+#ifndef FLASHD_FWD_CK
+#define FLASHD_FWD_CK 128
+#endif
+#ifndef FLASHD_FWD_NW
+#define FLASHD_FWD_NW 8
+#endif
+// waves per workgroup of the asynchronously staged backward kernels (64-token chunks)
+#ifndef FLASHD_BWD_NW
+#define FLASHD_BWD_NW 4
+#endif
+
+// DLT_FLASH_SYNC_STAGING=1 keeps the register-staged kernels for every class (A/B timing)
+inline bool flash_async_staging() {
+  static const bool on = [] { const char* e = std::getenv("DLT_FLASH_SYNC_STAGING"); return !(e != nullptr && e[0] == '1'); }();
+  return on;
+}
+
+template <typename KernT>
+int flash_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cast<const void*>(kern), bytes); }
+
 template <typename TIO, int MODE>
 int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
+  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
+    // dense / causal with exact head dims: chunks are copied HBM -> LDS asynchronously (a copy cannot zero-fill padded dims)
+    if (a.dk == DLT_DK && a.dv == DLT_DV && flash_async_staging()) {
+      constexpr int NP = FLASH_NP, CK = FLASHD_FWD_CK, NW = FLASHD_FWD_NW;
+      auto kern = flashd_fwd_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
+      constexpr int own = 16 * NP * NW;
+      constexpr int tile = own * (DLT_DV * 2 + 16);
+      constexpr int bufs = (NW == 4 ? flashd_nbuf(DLT_DK, DLT_DV) : 2) * FlashDBuf<DLT_DK, DLT_DV, CK>::BUF;
+      constexpr int lds = bufs > tile ? bufs : tile;
+      const int rc = flash_set_lds(kern, lds);
+      if (rc != DLT_OK) return rc;
+      FlashArgs ad = a;
+      ad.nblk = (a.Lq + own - 1) / own;
+      dlt_timing_before(DLT_K_FWD, stream);
+      hipLaunchKernelGGL(kern, dim3(a.B * a.H * ad.nblk), dim3(64 * NW), lds, stream, ad);
+      dlt_timing_after(stream);
+      DLT_CHECK_LAUNCH("flash forward launch");
+      return DLT_OK;
+    }
+  }
   auto kern = flash_fwd_kernel<TIO, DLT_DK, DLT_DV, FLASH_NP, flash_ck_fwd(DLT_DK, DLT_DV), MODE>;
   {
     const int rc = dlt_ensure_lds(reinterpret_cast<const void*>(kern), a.lds_bytes);
@@ -27,19 +68,30 @@ int flash_launch_fwd_t(const FlashArgs& a, int grid, hipStream_t stream) {
   return a.causal ? flash_launch_fwd_c<TIO, 1>(a, grid, stream) : flash_launch_fwd_c<TIO, 0>(a, grid, stream);
 }
 
-// DLT_FLASH_SYNC_STAGING=1 keeps the register-staged kernels for every class (A/B timing)
-inline bool flash_async_staging() {
-  static const bool on = [] { const char* e = std::getenv("DLT_FLASH_SYNC_STAGING"); return !(e != nullptr && e[0] == '1'); }();
-  return on;
-}
-
-template <typename KernT>
-int flash_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cast<const void*>(kern), bytes); }
-
 template <typename TIO, int MODE>
 int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream_t stream) {
   // dQ first: with fuse_delta it produces the delta vector the dK/dV kernel consumes
-  {
+  bool dq_done = false;
+  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
+    if (a.dk_ == DLT_DK && a.dv_ == DLT_DV && flash_async_staging()) {
+      constexpr int NP = flash_np_q(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
+      auto kern = flashd_bwd_q_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
+      constexpr int own = 16 * NP * NW;
+      constexpr int tile = own * (DLT_DK * 2 + 16);
+      constexpr int bufs = (NW == 4 ? flashd_nbuf(DLT_DK, DLT_DV) : FLASHD_NBUF8) * FlashDBuf<DLT_DK, DLT_DV, CK>::BUF;
+      constexpr int lds = bufs > tile ? bufs : tile;
+      int rc = flash_set_lds(kern, lds);
+      if (rc != DLT_OK) return rc;
+      FlashBwdArgs ad = a;
+      ad.nblk_q = (a.Lq + own - 1) / own;
+      dlt_timing_before(DLT_K_BWD_Q, stream);
+      hipLaunchKernelGGL(kern, dim3(a.B * a.H * ad.nblk_q), dim3(64 * NW), lds, stream, ad);
+      dlt_timing_after(stream);
+      DLT_CHECK_LAUNCH("flash dQ launch");
+      dq_done = true;
+    }
+  }
+  if (!dq_done) {
     auto kern = flash_bwd_q_kernel<TIO, DLT_DK, DLT_DV, flash_np_q(DLT_DK, DLT_DV), flash_ck_q(DLT_DK, DLT_DV), MODE>;
     int rc = flash_set_lds(kern, a.lds_q);
     if (rc != DLT_OK) return rc;
@@ -53,15 +105,18 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
     // dims; in tile mode, where whole blocks are skipped, the register-staged kernel measured 1.5 % faster)
     const bool scalars_fit = a.ls[2] >= 0 && ((int64_t)a.Lq - 1) * a.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1);   // 32-bit offsets of the lse2 / delta copies
     if (a.dk_ == DLT_DK && a.dv_ == DLT_DV && scalars_fit && flash_async_staging()) {
-      constexpr int NP = flash_np_kv(DLT_DK, DLT_DV), CK = 64;
-      auto kern = flashd_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP, CK, MODE>;
-      constexpr int tile_k = 64 * NP * (DLT_DK * 2 + 16), tile_v = 64 * NP * (DLT_DV * 2 + 16);
-      constexpr int bufs = flashd_nbuf(DLT_DK, DLT_DV) * FlashDBuf<DLT_DK, DLT_DV, CK>::BUF_KV;
+      constexpr int NP = flash_np_kv(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
+      auto kern = flashd_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
+      constexpr int own = 16 * NP * NW;
+      constexpr int tile_k = own * (DLT_DK * 2 + 16), tile_v = own * (DLT_DV * 2 + 16);
+      constexpr int bufs = (NW == 4 ? flashd_nbuf(DLT_DK, DLT_DV) : FLASHD_NBUF8) * FlashDBuf<DLT_DK, DLT_DV, CK>::BUF_KV;
       constexpr int lds = bufs > tile_v ? (bufs > tile_k ? bufs : tile_k) : (tile_v > tile_k ? tile_v : tile_k);
       int rc = flash_set_lds(kern, lds);
       if (rc != DLT_OK) return rc;
+      FlashBwdArgs ad = a;
+      ad.nblk_k = (a.Lk + own - 1) / own;
       dlt_timing_before(DLT_K_BWD_KV, stream);
-      hipLaunchKernelGGL(kern, dim3(grid_kv), dim3(256), lds, stream, a);
+      hipLaunchKernelGGL(kern, dim3(a.B * a.H * ad.nblk_k), dim3(64 * NW), lds, stream, ad);
       dlt_timing_after(stream);
       DLT_CHECK_LAUNCH("flash dK/dV launch");
       return DLT_OK;

@@ -521,7 +521,7 @@ struct PairStage {
 // accumulators (C layout, [dim][own token]) of NP blocks -> LDS tile -> HBM rows
 template <typename TIO, int D, int NP, typename SN>
 DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO* base, const SN& sn, int64_t sd, int dact,
-                              bool vec, int own_base, int x0, int len, int wave, int n, int g, int tid) {
+                              bool vec, int own_base, int x0, int len, int wave, int n, int g, int tid, int nrows = 64 * NP) {
   typedef typename TileOf<TIO>::type TL;
   constexpr int PT = D * (int)sizeof(TL) + 16;
   RopeDev no_rope = RopeDev{};
@@ -534,8 +534,9 @@ DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO
       for (int i = 0; i < 4; i++) row[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * mul);
   }
   __syncthreads();
-  store_tile<TIO, TL, D>(sT, PT, base, sn, sd, dact, vec, 64 * NP,
-                         [&](int r) { return x0 + r < len ? (int64_t)(own_base + x0 + r) : (int64_t)-1; }, no_rope, tid);
+  if (tid < 256)   // the tile writer walks the rows with 256 threads
+    store_tile<TIO, TL, D>(sT, PT, base, sn, sd, dact, vec, nrows,
+                           [&](int r) { return x0 + r < len ? (int64_t)(own_base + x0 + r) : (int64_t)-1; }, no_rope, tid);
   __syncthreads();
 }
 
