@@ -152,6 +152,29 @@ def test_causal_lengths_and_dims(N, dk, dv, dtype):
     assert max(errs) <= 5e-2, errs
 
 
+@pytest.mark.parametrize("causal,dk,dv,dtype", [
+    (False, 64, 128, torch.bfloat16), (False, 64, 64, torch.float16), (False, 128, 128, torch.bfloat16),
+    (True, 64, 128, torch.float16), (True, 128, 128, torch.bfloat16)])
+def test_chunk_boundaries_of_the_async_staged_kernels(causal, dk, dv, dtype):
+    """Head dims of exactly 64 / 128 run on the kernels that copy chunks HBM -> LDS asynchronously into two or three
+    buffers: lengths of one, two, three and four chunks (64 keys in the backward kernels, 128 in the forward kernel),
+    one token more and one less, and query counts around the 128- and 256-query workgroups."""
+    pairs = [(1, 1), (63, 64), (200, 65), (128, 127), (129, 128), (256, 129), (257, 191), (130, 192), (70, 193), (255, 256),
+             (33, 257), (300, 320)]
+    scale = 1 / math.sqrt(dk)
+    for Lq, Lk in pairs:
+        if causal:
+            Lq = Lk
+        q, k, v, do = orc.make_qkv(Lq * 5 + Lk + dk, 1, 2, Lq, Lk, dk, dv, dtype)
+        o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), causal, scale)
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        o = _fa().attention(qg, kg, vg, causal, scale)
+        o.backward(do.cuda())
+        assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2, (Lq, Lk)
+        errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+        assert max(errs) <= 5e-2, (Lq, Lk, errs)
+
+
 def test_bad_arguments_raise():
     from dl_templates_amd._lib import DltError
     q = torch.randn(1, 1, 64, 64, dtype=torch.bfloat16).cuda()
