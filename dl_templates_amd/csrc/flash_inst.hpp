@@ -8,6 +8,9 @@
 
 namespace {
 // shape of the asynchronously staged forward kernel: keys per chunk, waves per workgroup (16 NP queries per wave)
+#ifndef FLASHD_FWD_NP
+#define FLASHD_FWD_NP FLASH_NP
+#endif
 #ifndef FLASHD_FWD_CK
 #define FLASHD_FWD_CK 128
 #endif
@@ -30,10 +33,13 @@ int flash_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cas
 
 template <typename TIO, int MODE>
 int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
-  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
-    // dense / causal with exact head dims: chunks are copied HBM -> LDS asynchronously (a copy cannot zero-fill padded dims)
+  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && DLT_DK + DLT_DV > 128 && MODE == 0) {
+    // dense with exact head dims 64/128 or 128/128: chunks are copied HBM -> LDS asynchronously (a copy cannot zero-fill
+    // padded dims).  Measured per class and mode against the register-staged kernel: -4 % and -7 % here; at 64/64 the
+    // 8-wave workgroups lose (+14 %), and with a causal mask they lose in every class (+30 % and more: the waves of a
+    // 256-query workgroup see very different numbers of keys and the workgroup keeps its CU until the last one is done).
     if (a.dk == DLT_DK && a.dv == DLT_DV && flash_async_staging()) {
-      constexpr int NP = FLASH_NP, CK = FLASHD_FWD_CK, NW = FLASHD_FWD_NW;
+      constexpr int NP = FLASHD_FWD_NP, CK = FLASHD_FWD_CK, NW = FLASHD_FWD_NW;
       auto kern = flashd_fwd_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
       constexpr int own = 16 * NP * NW;
       constexpr int tile = own * (DLT_DV * 2 + 16);
@@ -100,9 +106,10 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
     dlt_timing_after(stream);
     DLT_CHECK_LAUNCH("flash dQ launch");
   }
-  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
+  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2 && !(DLT_DK + DLT_DV <= 128 && MODE == 0)) {
     // dense / causal with exact head dims: chunks are copied HBM -> LDS asynchronously (a copy cannot zero-fill padded
-    // dims; in tile mode, where whole blocks are skipped, the register-staged kernel measured 1.5 % faster)
+    // dims; in tile mode, where whole blocks are skipped, the register-staged kernel measured 1.5 % faster, and so it
+    // did dense at 64/64 (3 %))
     const bool scalars_fit = a.ls[2] >= 0 && ((int64_t)a.Lq - 1) * a.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1);   // 32-bit offsets of the lse2 / delta copies
     if (a.dk_ == DLT_DK && a.dv_ == DLT_DV && scalars_fit && flash_async_staging()) {
       constexpr int NP = flash_np_kv(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
