@@ -17,6 +17,11 @@ namespace {
 #ifndef FLASHD_FWD_NW
 #define FLASHD_FWD_NW 8
 #endif
+// query blocks per wave of the asynchronously staged dQ kernel: two in every class (without staging registers two blocks
+// fit at 128/128 as well: -18 % there; three blocks measured 8 % slower at 64/64 and 64/128)
+#ifndef FLASHD_DQ_NP
+#define FLASHD_DQ_NP(dk, dv) 2
+#endif
 // waves per workgroup of the asynchronously staged backward kernels (64-token chunks)
 #ifndef FLASHD_BWD_NW
 #define FLASHD_BWD_NW 4
@@ -80,7 +85,7 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
   bool dq_done = false;
   if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
     if (a.dk_ == DLT_DK && a.dv_ == DLT_DV && flash_async_staging()) {
-      constexpr int NP = flash_np_q(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
+      constexpr int NP = FLASHD_DQ_NP(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
       auto kern = flashd_bwd_q_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
       constexpr int own = 16 * NP * NW;
       constexpr int tile = own * (DLT_DK * 2 + 16);
