@@ -252,7 +252,6 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
       bool bv[NP];
 #pragma unroll
       for (int p = 0; p < NP; p++) bv[p] = !TILE || (q0 + 32 * qb_ + 32 > vlo[p] && q0 + 32 * qb_ < vhi[p]);
-      float pr[NP][8], ds[NP][8];
       f32x4 sv[NP], dp[NP], lq, dl;
       u32x4 pb[NP], dsb[NP];
       swa2_for<0, NB>([&](auto jc) __attribute__((always_inline)) {
@@ -278,6 +277,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 #pragma unroll
             for (int p = 0; p < NP; p++) {
               const bool hv = !TILE || (q0 + 32 * qb_ + 16 * mb >= vlo[p] && q0 + 32 * qb_ + 16 * mb < vhi[p]);
+              float pr[4], ds[4];
 #pragma unroll
               for (int i = 0; i < 4; i++) {
                 float pv = bv[p] ? fast_exp2(fmaf(sv[p][i], scale, -lq[i])) : 0.f;
@@ -286,15 +286,16 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
                   pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
                 }
                 if (TILE) pv = hv ? pv : 0.f;
-                pr[p][4 * mb + i] = pv;
-                ds[p][4 * mb + i] = bv[p] ? pv * (dp[p][i] - dl[i]) : 0.f;
+                pr[i] = pv;
+                ds[i] = bv[p] ? pv * (dp[p][i] - dl[i]) : 0.f;
               }
-            }
-            if constexpr (mb == 1) {
-#pragma unroll
-              for (int p = 0; p < NP; p++) {
-                pb[p] = pack8<CT>(pr[p]);
-                dsb[p] = pack8<CT>(ds[p]);
+              // packed at once: elements 4 mb .. 4 mb + 3 of the block's 8 per lane
+              if constexpr (mb == 0) {
+                pb[p].x = pack2<CT>(pr[0], pr[1]); pb[p].y = pack2<CT>(pr[2], pr[3]);
+                dsb[p].x = pack2<CT>(ds[0], ds[1]); dsb[p].y = pack2<CT>(ds[2], ds[3]);
+              } else {
+                pb[p].z = pack2<CT>(pr[0], pr[1]); pb[p].w = pack2<CT>(pr[2], pr[3]);
+                dsb[p].z = pack2<CT>(ds[0], ds[1]); dsb[p].w = pack2<CT>(ds[2], ds[3]);
               }
             }
           }
