@@ -175,6 +175,30 @@ def test_chunk_boundaries_of_the_async_staged_kernels(causal, dk, dv, dtype):
         assert max(errs) <= 5e-2, (Lq, Lk, errs)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_views_of_a_packed_projection(causal):
+    """q, k, v as strided views of one packed [B, L, H, dk + dk + dv] projection output (token stride H (2 dk + dv), head
+    stride 2 dk + dv) and a transposed upstream gradient: the asynchronously staged kernels address tokens by stride."""
+    B, H, L, dk, dv = 2, 3, 200, 64, 128
+    g = torch.Generator().manual_seed(11)
+    packed = torch.randn(B, L, H, 2 * dk + dv, generator=g).to(torch.bfloat16)
+    do = torch.randn(B, L, H, dv, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(dk)
+    views = lambda t: (t[..., :dk].permute(0, 2, 1, 3), t[..., dk:2 * dk].permute(0, 2, 1, 3), t[..., 2 * dk:].permute(0, 2, 1, 3))
+    q, k, v = views(packed)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float().contiguous(), k.float().contiguous(), v.float().contiguous(),
+                                            do.permute(0, 2, 1, 3).float().contiguous(), causal, scale)
+    pg = packed.cuda().requires_grad_(True)
+    qg, kg, vg = views(pg)
+    assert not qg.is_contiguous()
+    o = _fa().attention(qg, kg, vg, causal, scale)
+    o.backward(do.cuda().permute(0, 2, 1, 3))
+    assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
+    got = views(pg.grad)
+    errs = (_rel(got[0], dq_w), _rel(got[1], dk_w), _rel(got[2], dv_w))
+    assert max(errs) <= 5e-2, errs
+
+
 def test_bad_arguments_raise():
     from dl_templates_amd._lib import DltError
     q = torch.randn(1, 1, 64, 64, dtype=torch.bfloat16).cuda()
