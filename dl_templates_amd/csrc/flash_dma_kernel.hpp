@@ -102,6 +102,11 @@ DLT_DEV void flashd_issue_scalars(const float* base, int stride, const FlashChun
 #define FLASHD_RD 1
 #endif
 
+// how the scheduler is asked to place an element-wise piece behind the NP products of its operand
+#ifndef FLASHD_EW_MIX
+#define FLASHD_EW_MIX SWA2_MIX(NP, 12 / NP)
+#endif
+
 // at most N of this wave's copies (the youngest ones) are still in flight
 template <int N>
 DLT_DEV void flashd_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
@@ -132,7 +137,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   typedef typename ComputeOf<TIO>::type CT;
   typedef FlashDBuf<DK, DV, CK> B;
   extern __shared__ __align__(16) char smem[];
-  constexpr bool CAUSAL = MODE == 1, TILE = MODE >= 2, IMG = MODE == 3;
+  constexpr bool CAUSAL = MODE == 1, TILE = false, IMG = false;
+  static_assert(MODE < 2, "asynchronous staging: dense and causal only");
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16, NQB = CK / 32;
   constexpr int OWN = 16 * NP * NW;
 
@@ -178,17 +184,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 
   u32x4 kf[NP][KC], vf[NP][VC];
   int qmin[NP];           // causal: first query that sees this lane's key
-  int vlo[NP], vhi[NP];   // tile mode: x interval of the queries that see this key block
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int xk = wk0 + 16 * p + n;
     const int64_t tk = xk < a.Lk ? (int64_t)(own_base + xk) : (int64_t)-1;
     qmin[p] = CAUSAL ? xk : 0;
-    vlo[p] = vhi[p] = 0;
-    if (TILE && wk0 + 16 * p < a.Lk) {
-      int rl, rh;
-      dlt_query_range(a.g, r_own, wk0 + 16 * p, rl, rh, vlo[p], vhi[p]);
-    }
     swa1_load_own<TIO, CT, DK>(kf[p], kb_, 1, a.dk_, flash_own_off<IMG>(a.ks, a.tm, tk), g, no_rope, false);
     swa1_load_own<TIO, CT, DV>(vf[p], vb_, 1, a.dv_, flash_own_off<IMG>(a.vs, a.tm, tk), g, no_rope, false);
   }
@@ -230,85 +230,87 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     const int q0 = c.x;
     // causal: every query of the chunk lies below every own key of this wave
     if (CAUSAL && q0 + CK - 1 < wk0) return;
-    constexpr int N1H = KC + VC, N1 = 2 * N1H, NB = N1 + VB + KB, NT = NQB * NB;
+    // Order of a chunk's operands: the first products (S, dP) of every 16-query half of every block, then the second
+    // products (dV, dK) block by block.  The element-wise work of a half (P, dS: vector instructions that depend on its
+    // first products) is issued in pieces behind the matrix instructions of the FOLLOWING segment, which do not depend on
+    // it: a wave issues in order, and with the element-wise work directly behind the products it waits for, matrix pipe
+    // and vector ALU take turns instead of running side by side.
+    constexpr int N1H = KC + VC, NH = 2 * NQB, N1 = NH * N1H, NP2 = VB + KB, NT = N1 + NQB * NP2;
+    constexpr int NU = 2 * NP;   // element-wise pieces of a half: (own block p, pair of queries)
+    static_assert(N1H >= NU && NP2 >= NU, "a segment must have room for the element-wise pieces of a half");
     constexpr int RD = FLASHD_RD;
     u32x4 ring[RD + 1];
     auto rd = [&](auto kc) __attribute__((always_inline)) {
       constexpr int k = decltype(kc)::value;
-      constexpr int qb_ = k / NB, j = k % NB;
-      if constexpr (j < N1) {
-        constexpr int mb = j / N1H, r = j % N1H, T0 = 32 * qb_ + 16 * mb;
+      if constexpr (k < N1) {
+        constexpr int hh = k / N1H, r = k % N1H, T0 = 16 * hh;
         if constexpr (r < KC) ring[k % (RD + 1)] = swa2_lds16(sQ + T0 * FlashDRow<DK>::ROW + LQ.a[r]);
         else ring[k % (RD + 1)] = swa2_lds16(sDO + T0 * FlashDRow<DV>::ROW + LD.a[r - KC]);
       } else {
-        constexpr int d = j - N1;
+        constexpr int qb_ = (k - N1) / NP2, d = (k - N1) % NP2;
         if constexpr (d < VB) ring[k % (RD + 1)] = flashd_read_tr<DV, 32 * qb_>(sDO, LD, d);
         else ring[k % (RD + 1)] = flashd_read_tr<DK, 32 * qb_>(sQ, LQ, d - VB);
       }
     };
     swa2_for<0, RD>([&](auto kc) __attribute__((always_inline)) { rd(kc); });
-    swa2_for<0, NQB>([&](auto qbc) __attribute__((always_inline)) {
-      constexpr int qb_ = decltype(qbc)::value;
-      bool bv[NP];
+    f32x4 sv[2][NP], dp[2][NP], lq[2], dl[2];   // indexed by the parity of the half
+    u32x4 pb[NQB][NP], dsb[NQB][NP];
+    // piece u of the element-wise work of half hh: p = exp2(s scale - lse2), dS = p (dP - delta) for own block u / 2,
+    // queries 2 (u % 2), 2 (u % 2) + 1 of the lane's four
+    auto ew = [&](auto hhc, auto uc) __attribute__((always_inline)) {
+      constexpr int hh = decltype(hhc)::value, u = decltype(uc)::value;
+      constexpr int qb_ = hh / 2, mb = hh % 2, p = u / 2, i0_ = 2 * (u % 2);
+      float pr[2], ds[2];
 #pragma unroll
-      for (int p = 0; p < NP; p++) bv[p] = !TILE || (q0 + 32 * qb_ + 32 > vlo[p] && q0 + 32 * qb_ < vhi[p]);
-      f32x4 sv[NP], dp[NP], lq, dl;
-      u32x4 pb[NP], dsb[NP];
-      swa2_for<0, NB>([&](auto jc) __attribute__((always_inline)) {
-        constexpr int j = decltype(jc)::value, k = qb_ * NB + j;
-        if constexpr (k + RD < NT) rd(std::integral_constant<int, k + RD>{});
-        if constexpr (j < N1 && j % N1H == 0) {
-          constexpr int mb = j / N1H;
-          lq = __builtin_bit_cast(f32x4, swa2_lds16(sLse + (32 * qb_ + 16 * mb) * 4));
-          dl = __builtin_bit_cast(f32x4, swa2_lds16(sDel + (32 * qb_ + 16 * mb) * 4));
+      for (int t = 0; t < 2; t++) {
+        const int i = i0_ + t;
+        float pv = fast_exp2(fmaf(sv[hh & 1][p][i], scale, -lq[hh & 1][i]));
+        if (tail) {
+          const int qi = q0 + 16 * hh + 4 * g + i;
+          pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
         }
-        __builtin_amdgcn_sched_barrier(0);
-        const u32x4 x = ring[k % (RD + 1)];
-        if constexpr (j < N1) {
-          constexpr int mb = j / N1H, r = j % N1H;
+        pr[t] = pv;
+        ds[t] = pv * (dp[hh & 1][p][i] - dl[hh & 1][i]);
+      }
+      const unsigned pw = pack2<CT>(pr[0], pr[1]), dw = pack2<CT>(ds[0], ds[1]);
+      if constexpr (mb == 0 && i0_ == 0) { pb[qb_][p].x = pw; dsb[qb_][p].x = dw; }
+      if constexpr (mb == 0 && i0_ == 2) { pb[qb_][p].y = pw; dsb[qb_][p].y = dw; }
+      if constexpr (mb == 1 && i0_ == 0) { pb[qb_][p].z = pw; dsb[qb_][p].z = dw; }
+      if constexpr (mb == 1 && i0_ == 2) { pb[qb_][p].w = pw; dsb[qb_][p].w = dw; }
+    };
+    swa2_for<0, NT>([&](auto kc) __attribute__((always_inline)) {
+      constexpr int k = decltype(kc)::value;
+      if constexpr (k + RD < NT) rd(std::integral_constant<int, k + RD>{});
+      if constexpr (k < N1 && k % N1H == 0) {
+        constexpr int hh = k / N1H;
+        lq[hh & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 16 * hh * 4));
+        dl[hh & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sDel + 16 * hh * 4));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const u32x4 x = ring[k % (RD + 1)];
+      if constexpr (k < N1) {
+        constexpr int hh = k / N1H, r = k % N1H;
 #pragma unroll
-          for (int p = 0; p < NP; p++) {
-            if (!bv[p]) continue;
-            if constexpr (r < KC) sv[p] = Mma<CT>::mfma(x, kf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sv[p]);
-            else dp[p] = Mma<CT>::mfma(x, vf[p][r - KC], r == KC ? f32x4{0.f, 0.f, 0.f, 0.f} : dp[p]);
-          }
-          if constexpr (r == N1H - 1) {
-            // P and dS of the half: p = exp2(s scale - lse2), dS = p (dP - delta)
-#pragma unroll
-            for (int p = 0; p < NP; p++) {
-              const bool hv = !TILE || (q0 + 32 * qb_ + 16 * mb >= vlo[p] && q0 + 32 * qb_ + 16 * mb < vhi[p]);
-              float pr[4], ds[4];
-#pragma unroll
-              for (int i = 0; i < 4; i++) {
-                float pv = bv[p] ? fast_exp2(fmaf(sv[p][i], scale, -lq[i])) : 0.f;
-                if (tail) {
-                  const int qi = q0 + 32 * qb_ + 16 * mb + 4 * g + i;
-                  pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
-                }
-                if (TILE) pv = hv ? pv : 0.f;
-                pr[i] = pv;
-                ds[i] = bv[p] ? pv * (dp[p][i] - dl[i]) : 0.f;
-              }
-              // packed at once: elements 4 mb .. 4 mb + 3 of the block's 8 per lane
-              if constexpr (mb == 0) {
-                pb[p].x = pack2<CT>(pr[0], pr[1]); pb[p].y = pack2<CT>(pr[2], pr[3]);
-                dsb[p].x = pack2<CT>(ds[0], ds[1]); dsb[p].y = pack2<CT>(ds[2], ds[3]);
-              } else {
-                pb[p].z = pack2<CT>(pr[0], pr[1]); pb[p].w = pack2<CT>(pr[2], pr[3]);
-                dsb[p].z = pack2<CT>(ds[0], ds[1]); dsb[p].w = pack2<CT>(ds[2], ds[3]);
-              }
-            }
-          }
-        } else {
-          constexpr int d = j - N1;
-#pragma unroll
-          for (int p = 0; p < NP; p++) {
-            if (!bv[p]) continue;
-            if constexpr (d < VB) dv_acc[p][d] = Mma<CT>::mfma(x, pb[p], dv_acc[p][d]);
-            else dk_acc[p][d - VB] = Mma<CT>::mfma(x, dsb[p], dk_acc[p][d - VB]);
-          }
+        for (int p = 0; p < NP; p++) {
+          if constexpr (r < KC) sv[hh & 1][p] = Mma<CT>::mfma(x, kf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sv[hh & 1][p]);
+          else dp[hh & 1][p] = Mma<CT>::mfma(x, vf[p][r - KC], r == KC ? f32x4{0.f, 0.f, 0.f, 0.f} : dp[hh & 1][p]);
         }
-      });
+        if constexpr (hh >= 1 && r < NU) {
+          ew(std::integral_constant<int, hh - 1>{}, std::integral_constant<int, r>{});
+          FLASHD_EW_MIX
+        }
+      } else {
+        constexpr int qb_ = (k - N1) / NP2, d = (k - N1) % NP2;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+          if constexpr (d < VB) dv_acc[p][d] = Mma<CT>::mfma(x, pb[qb_][p], dv_acc[p][d]);
+          else dk_acc[p][d - VB] = Mma<CT>::mfma(x, dsb[qb_][p], dk_acc[p][d - VB]);
+        }
+        if constexpr (qb_ == 0 && d < NU) {
+          ew(std::integral_constant<int, NH - 1>{}, std::integral_constant<int, d>{});
+          FLASHD_EW_MIX
+        }
+      }
     });
   };
   // Chunk ci lives in buffer ci % NBUF; its copy is started AHEAD chunks before it is consumed (the latency of a copy
