@@ -1,7 +1,7 @@
 // Flash kernels with asynchronous staging: the variants of flash_kernel.hpp for head dims that are exactly 64 or
 // 128 (no padded dims: a copy cannot zero-fill).  Streamed chunks travel HBM -> LDS by the DMA path of the vector
-// memory unit (16 bytes per lane, no staging registers, no LDS write instructions) into one of two chunk buffers
-// while the other one is consumed: one workgroup barrier per chunk instead of two.  LDS rows are 2 D bytes without
+// memory unit (16 bytes per lane, no staging registers, no LDS write instructions) into a ring of two or three chunk
+// buffers while an earlier chunk is consumed: one workgroup barrier per chunk instead of two.  LDS rows are 2 D bytes without
 // padding; the 16-byte piece c of token t is stored at piece c ^ (m (t & 7)), m = D / 64, which keeps the operand
 // reads (16 lanes x 16 bytes), the transposing reads (32 lanes x 8 bytes) and the 64 x 16 bytes a copy instruction
 // writes on distinct banks.  The arithmetic, the masks and the chunk walk are those of flash_kernel.hpp.
@@ -117,7 +117,8 @@ DLT_DEV void flashd_wait_copies() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) 
 #define FLASHD_NBUF(dk, dv) ((dk) + (dv) > 192 ? 2 : 3)
 #endif
 constexpr int flashd_nbuf(int dk, int dv) { return FLASHD_NBUF(dk, dv); }
-// 8-wave workgroups of the backward kernels (one per CU, 64-token chunks)
+// the same for 8-wave workgroups of the backward kernels (one per CU, 64-token chunks; measured slower than 4-wave
+// workgroups and not instantiated by default: FLASHD_BWD_NW in flash_inst.hpp)
 #ifndef FLASHD_NBUF8
 #define FLASHD_NBUF8 3
 #endif
