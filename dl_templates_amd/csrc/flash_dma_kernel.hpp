@@ -138,7 +138,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   typedef typename ComputeOf<TIO>::type CT;
   typedef FlashDBuf<DK, DV, CK> B;
   extern __shared__ __align__(16) char smem[];
-  constexpr bool CAUSAL = MODE == 1, TILE = false, IMG = false;
+  constexpr bool CAUSAL = MODE == 1;
   static_assert(MODE < 2, "asynchronous staging: dense and causal only");
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16, NQB = CK / 32;
   constexpr int OWN = 16 * NP * NW;
@@ -149,7 +149,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
   int bh, r_own, x0;
-  flash_block(lin, a.nblk_k, TILE ? a.g.TR : 1, OWN, false, bh, r_own, x0);
+  flash_block(lin, a.nblk_k, 1, OWN, false, bh, r_own, x0);
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* kb_ = reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1];
   const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
@@ -157,13 +157,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   const char* dob = reinterpret_cast<const char*>(reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1]);
   const float* lseb = a.lse + b * a.ls[0] + h * a.ls[1];
   const float* delb = a.delta + b * a.ls[0] + h * a.ls[1];
-  const FlashAddr<IMG> aq = flash_addr<IMG>(a.qs, a.tm), ad = flash_addr<IMG>(a.dos, a.tm);
+  const FlashAddr<false> aq = flash_addr<false>(a.qs, a.tm), ad = flash_addr<false>(a.dos, a.tm);
   RopeDev no_rope = RopeDev{};
-  const int own_base = TILE ? r_own * a.Lk : 0;
 
   FlashWalk<MODE, CK> W;
-  if (TILE) W.init_tile(a.g, r_own, x0, OWN, true);
-  else W.init_seq(CAUSAL ? (x0 / CK) * CK : 0, a.Lq);
+  W.init_seq(CAUSAL ? (x0 / CK) * CK : 0, a.Lq);
   const int wk0 = x0 + wave * 16 * NP;  // first own key of this wave
 
   FlashDStage<DK, CK, NW> stq;
@@ -188,10 +186,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int xk = wk0 + 16 * p + n;
-    const int64_t tk = xk < a.Lk ? (int64_t)(own_base + xk) : (int64_t)-1;
+    const int64_t tk = xk < a.Lk ? (int64_t)xk : (int64_t)-1;
     qmin[p] = CAUSAL ? xk : 0;
-    swa1_load_own<TIO, CT, DK>(kf[p], kb_, 1, a.dk_, flash_own_off<IMG>(a.ks, a.tm, tk), g, no_rope, false);
-    swa1_load_own<TIO, CT, DV>(vf[p], vb_, 1, a.dv_, flash_own_off<IMG>(a.vs, a.tm, tk), g, no_rope, false);
+    swa1_load_own<TIO, CT, DK>(kf[p], kb_, 1, a.dk_, flash_own_off<false>(a.ks, a.tm, tk), g, no_rope, false);
+    swa1_load_own<TIO, CT, DV>(vf[p], vb_, 1, a.dv_, flash_own_off<false>(a.vs, a.tm, tk), g, no_rope, false);
   }
   f32x4 dk_acc[NP][KB], dv_acc[NP][VB];
 #pragma unroll
@@ -212,7 +210,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 
   auto chunk_tail = [&](const int ci) {
     const FlashChunk c = W.at(ci);
-    return !TILE && (c.nvalid < CK || (CAUSAL && c.x < wk0 + 16 * NP - 1));
+    return c.nvalid < CK || (CAUSAL && c.x < wk0 + 16 * NP - 1);
   };
   // Products of the chunk resident in `cur`; with `more` the copy of the next chunk into `nxt` is started first.
   // A block of 32 queries is a stream of NB operand reads, each feeding NP matrix instructions: per 16-query half KC
@@ -341,8 +339,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   __syncthreads();
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
-  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, flash_tok<IMG>(a.dks, a.tm), a.dks[3], a.dk_, a.dk_vec != 0, own_base, x0, a.Lk, wave, n, g, tid, OWN);
-  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, flash_tok<IMG>(a.dvs, a.tm), a.dvs[3], a.dv_, a.dv_vec != 0, own_base, x0, a.Lk, wave, n, g, tid, OWN);
+  flash_write_grad<TIO, DK, NP>(smem, dk_acc, a.sm_scale, dkb, flash_tok<false>(a.dks, a.tm), a.dks[3], a.dk_, a.dk_vec != 0, 0, x0, a.Lk, wave, n, g, tid, OWN);
+  flash_write_grad<TIO, DV, NP>(smem, dv_acc, 1.0f, dvb, flash_tok<false>(a.dvs, a.tm), a.dvs[3], a.dv_, a.dv_vec != 0, 0, x0, a.Lk, wave, n, g, tid, OWN);
 }
 
 // ---- forward: own = queries; K and V stream.  Replaces _attn_fwd (src/flash_attn.py:81-172).
