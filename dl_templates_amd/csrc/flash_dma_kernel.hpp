@@ -206,6 +206,10 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   flashd_lane_init(LD, n, g);
 
   swa2_wait_copies();   // also: the own fragments have arrived
+  // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
+  // for every copy in flight) at their first use inside every round of the chunk loop
+  pin_loaded(kf);
+  pin_loaded(vf);
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -420,6 +424,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
   flashd_lane_init(LV, n, g);
 
   swa2_wait_copies();   // also: the own fragments have arrived
+  // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
+  // for every copy in flight) at their first use inside every round of the chunk loop
+  pin_loaded(qf);
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -642,6 +649,12 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
   flashd_lane_init(LV, n, g);
 
   swa2_wait_copies();   // also: the own fragments and scalars have arrived
+  // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
+  // for every copy in flight) at their first use inside every round of the chunk loop
+  pin_loaded(qf);
+  pin_loaded(dof);
+#pragma unroll
+  for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {

@@ -67,6 +67,9 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
   const int ncg = (4 + 2 * G.WC + 3) >> 2;   // column groups of the wave window that can hold a visible token
 
   swa2_wait_copies();   // also: the own fragments have arrived
+  // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
+  // for every copy in flight) at their first use inside every round of the chunk loop
+  pin_loaded(qf);
   __syncthreads();
 
   // `cur` (the chunk being read) and `nxt` (the buffer the next chunk is copied into) are distinct buffers: the restrict
