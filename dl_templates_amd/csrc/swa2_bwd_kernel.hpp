@@ -91,6 +91,11 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
   const int ncg = (4 + 2 * G.WC + 3) >> 2;
 
   swa2_wait_copies();   // also: the own fragments have arrived
+  // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
+  // for every copy in flight) at their first use inside every round of the chunk loop
+  pin_loaded(qf);
+  pin_loaded(dof);
+  pin_loaded(neg_lse);
   __syncthreads();
 
   // `cur` and `nxt` are distinct chunk buffers (see the forward kernel)
@@ -255,6 +260,10 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
   const int ncg = (4 + 2 * G.WC + 3) >> 2;
 
   swa2_wait_copies();
+  // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
+  // for every copy in flight) at their first use inside every round of the chunk loop
+  pin_loaded(kf);
+  pin_loaded(vf);
   __syncthreads();
 
   auto consume = [&](const int ch, Swa2Lds __restrict__ cur, char* __restrict__ nxt, auto more_tag) {
