@@ -394,6 +394,7 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
   const int own = 64 * FLASH_NP;
   a.nblk = (a.Lq + own - 1) / own;
   a.causal = p.g.mode == DLT_GEOM_CAUSAL;
+  a.causal_group = flash_causal_group(a.Lk, p.dk, p.dv);
   a.tile = p.g.mode == DLT_GEOM_SWA;
   a.g = p.g;
   a.o_vec = tvec_ok(t.out_o, t.os, p.dv, 2);
@@ -443,6 +444,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
   a.nblk_q = (a.Lq + own - 1) / own;
   a.nblk_k = (a.Lk + own_kv - 1) / own_kv;
   a.causal = p.g.mode == DLT_GEOM_CAUSAL;
+  a.causal_group = flash_causal_group(a.Lk, p.dk, p.dv);
   a.tile = p.g.mode == DLT_GEOM_SWA;
   a.g = p.g;
   a.dq_vec = tvec_ok(t.dq, t.dqs, p.dk, 2);

@@ -149,7 +149,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
   int bh, r_own, x0;
-  flash_block(lin, a.nblk_k, 1, OWN, false, bh, r_own, x0);
+  if constexpr (CAUSAL) flash_block_causal(lin, a.nblk_k, a.B * a.H, a.causal_group, OWN, false, bh, r_own, x0);
+  else flash_block(lin, a.nblk_k, 1, OWN, bh, r_own, x0);
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* kb_ = reinterpret_cast<const TIO*>(a.k) + b * a.ks[0] + h * a.ks[1];
   const TIO* vb_ = reinterpret_cast<const TIO*>(a.v) + b * a.vs[0] + h * a.vs[1];
@@ -232,7 +233,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     const FlashChunk c = W.at(ci);
     const int q0 = c.x;
     // causal: every query of the chunk lies below every own key of this wave
-    if (CAUSAL && q0 + CK - 1 < wk0) return;
+    if (CAUSAL && !std::is_same<decltype(tail_tag), std::false_type>::value && q0 + CK - 1 < wk0) return;
     // Order of a chunk's operands: the first products (S, dP) of every 16-query half of every block, then the second
     // products (dV, dK) block by block.  The element-wise work of a half (P, dS: vector instructions that depend on its
     // first products) is issued in pieces behind the matrix instructions of the FOLLOWING segment, which do not depend on
@@ -321,9 +322,18 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   // bodies then hold no per-pair test.
   int ci = 0, bi = 0;   // bi = ci % NBUF
   auto buf_of = [&](int i) { return smem + (i >= NBUF ? i - NBUF : i) * B::BUF_KV; };
+  if constexpr (CAUSAL) {
+    // the chunks on the diagonal come first: per-chunk and per-pair tests; every later chunk but the last is full and
+    // lies below every own key, its body holds no test (as without a mask)
+    for (; ci + AHEAD < W.nchunks && W.at(ci).x < x0 + OWN - 1; ci++) {
+      consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
+      flashd_wait_copies<PER_CHUNK>();
+      __syncthreads();
+      bi = bi + 1 == NBUF ? 0 : bi + 1;
+    }
+  }
   for (; ci + AHEAD < W.nchunks; ci++) {
-    if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
-    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
+    consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
     flashd_wait_copies<PER_CHUNK>();   // all but the copies just issued: chunk ci + 1 has landed
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
@@ -371,7 +381,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
   int bh, r_own, x0;
-  flash_block(lin, a.nblk, 1, OWN, CAUSAL, bh, r_own, x0);
+  if constexpr (CAUSAL) flash_block_causal(lin, a.nblk, a.B * a.H, a.causal_group, OWN, true, bh, r_own, x0);
+  else flash_block(lin, a.nblk, 1, OWN, bh, r_own, x0);
   const int wq0 = x0 + wave * 16 * NP;
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
@@ -442,7 +453,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
     // causal: every key of the chunk lies above every query of this wave
-    if (CAUSAL && k0 > wq0 + 16 * NP - 1) return;
+    if (CAUSAL && !std::is_same<decltype(tail_tag), std::false_type>::value && k0 > wq0 + 16 * NP - 1) return;
     constexpr int N1 = NKB * 2 * KC, NT = N1 + NKB * VB;
     constexpr int RD = FLASHD_RD;
     u32x4 ring[RD + 1];
@@ -521,6 +532,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
   };
   int ci = 0, bi = 0;
   auto buf_of = [&](int i) { return smem + (i >= NBUF ? i - NBUF : i) * B::BUF; };
+  if constexpr (CAUSAL) {
+    // the chunks below the first query of the workgroup: every wave sees every pair, the body holds no test (as without
+    // a mask); the chunks on the diagonal follow with the per-chunk and per-pair tests
+    const int nfull = dlt_imin(x0, W.len) / CK;
+    for (; ci + AHEAD < W.nchunks && ci < nfull; ci++) {
+      consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
+      flashd_wait_copies<PER_CHUNK>();
+      __syncthreads();
+      bi = bi + 1 == NBUF ? 0 : bi + 1;
+    }
+  }
   for (; ci + AHEAD < W.nchunks; ci++) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
     else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
@@ -581,7 +603,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
 
   const int lin = xcd_remap(blockIdx.x, gridDim.x);
   int bh, r_own, x0;
-  flash_block(lin, a.nblk_q, 1, OWN, CAUSAL, bh, r_own, x0);
+  if constexpr (CAUSAL) flash_block_causal(lin, a.nblk_q, a.B * a.H, a.causal_group, OWN, true, bh, r_own, x0);
+  else flash_block(lin, a.nblk_q, 1, OWN, bh, r_own, x0);
   const int wq0 = x0 + wave * 16 * NP;
   const int b = bh / a.H, h = bh - b * a.H;
   const TIO* qb = reinterpret_cast<const TIO*>(a.q) + b * a.qs[0] + h * a.qs[1];
@@ -669,7 +692,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
     Swa2Lds sK = cur, sV = cur + B::REG_A;
     const FlashChunk c = W.at(ci);
     const int k0 = c.x;
-    if (CAUSAL && k0 > wq0 + 16 * NP - 1) return;
+    if (CAUSAL && !std::is_same<decltype(tail_tag), std::false_type>::value && k0 > wq0 + 16 * NP - 1) return;
     constexpr int N1H = KC + VC, N1 = 2 * N1H, NB = N1 + KB, NT = NKB * NB;
     constexpr int RD = FLASHD_RD;
     u32x4 ring[RD + 1];
@@ -726,6 +749,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
   };
   int ci = 0, bi = 0;
   auto buf_of = [&](int i) { return smem + (i >= NBUF ? i - NBUF : i) * B::BUF; };
+  if constexpr (CAUSAL) {
+    // the chunks below the first query of the workgroup: every wave sees every pair, the body holds no test (as without
+    // a mask); the chunks on the diagonal follow with the per-chunk and per-pair tests
+    const int nfull = dlt_imin(x0, W.len) / CK;
+    for (; ci + AHEAD < W.nchunks && ci < nfull; ci++) {
+      consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
+      flashd_wait_copies<PER_CHUNK>();
+      __syncthreads();
+      bi = bi + 1 == NBUF ? 0 : bi + 1;
+    }
+  }
   for (; ci + AHEAD < W.nchunks; ci++) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
     else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});

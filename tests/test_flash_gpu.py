@@ -152,6 +152,30 @@ def test_causal_lengths_and_dims(N, dk, dv, dtype):
     assert max(errs) <= 5e-2, errs
 
 
+@pytest.mark.parametrize("B,H,N,dk,dv", [(1, 7, 4096, 128, 128), (3, 3, 2048, 64, 64), (1, 5, 1536, 64, 128)])
+def test_causal_block_order_over_heads(B, H, N, dk, dv):
+    """Under a causal mask the workgroups of several (batch, head) slabs are interleaved, heaviest blocks first, in groups
+    sized by their K / V footprint (groups of 2, 8 and 7 heads here, the last one partial).  The order must not change any
+    result: every slab run on its own (one head per call) gives the same bits, and slab 0 matches the oracle."""
+    q, k, v, do = orc.make_qkv(N + H, B, H, N, N, dk, dv, torch.bfloat16)
+    scale = 1 / math.sqrt(dk)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = _fa().attention(qg, kg, vg, True, scale)
+    o.backward(do.cuda())
+    for b in range(B):
+        for h in range(H):
+            q1, k1, v1 = (t[b:b + 1, h:h + 1].contiguous().cuda().requires_grad_(True) for t in (q, k, v))
+            o1 = _fa().attention(q1, k1, v1, True, scale)
+            o1.backward(do[b:b + 1, h:h + 1].contiguous().cuda())
+            assert torch.equal(o1[0, 0], o[b, h]), (b, h)
+            assert torch.equal(q1.grad[0, 0], qg.grad[b, h]) and torch.equal(k1.grad[0, 0], kg.grad[b, h]) \
+                and torch.equal(v1.grad[0, 0], vg.grad[b, h]), (b, h)
+    sl = (slice(0, 1), slice(0, 1))
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q[sl].float(), k[sl].float(), v[sl].float(), do[sl].float(), True, scale)
+    assert (o[sl].float().cpu() - o_w).abs().max().item() <= 2e-2
+    assert max(_rel(qg.grad[sl], dq_w), _rel(kg.grad[sl], dk_w), _rel(vg.grad[sl], dv_w)) <= 5e-2
+
+
 @pytest.mark.parametrize("causal,dk,dv,dtype", [
     (False, 64, 128, torch.bfloat16), (False, 64, 64, torch.float16), (False, 128, 128, torch.bfloat16),
     (True, 64, 128, torch.float16), (True, 128, 128, torch.bfloat16)])
