@@ -7,15 +7,17 @@
 #define DLT_FCAT3(a, b, c) DLT_FCAT3_(a, b, c)
 
 namespace {
-// shape of the asynchronously staged forward kernel: keys per chunk, waves per workgroup (16 NP queries per wave)
+// shape of the asynchronously staged forward kernel: keys per chunk, waves per workgroup (16 NP queries per wave).
+// 8 waves on 128-key chunks at 64/128 and 128/128 (K / V copied once per 256 queries), 4 waves on 64-key chunks at 64/64
+// (there the 8-wave shape only ties with the register-staged kernel)
 #ifndef FLASHD_FWD_NP
 #define FLASHD_FWD_NP FLASH_NP
 #endif
 #ifndef FLASHD_FWD_CK
-#define FLASHD_FWD_CK 128
+#define FLASHD_FWD_CK(dk, dv) ((dk) + (dv) > 128 ? 128 : 64)
 #endif
 #ifndef FLASHD_FWD_NW
-#define FLASHD_FWD_NW 8
+#define FLASHD_FWD_NW(dk, dv) ((dk) + (dv) > 128 ? 8 : 4)
 #endif
 // query blocks per wave of the asynchronously staged dQ kernel: two in every class (without staging registers two blocks
 // fit at 128/128 as well: -18 % there; three blocks measured 8 % slower at 64/64 and 64/128)
@@ -38,13 +40,12 @@ int flash_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cas
 
 template <typename TIO, int MODE>
 int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
-  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && DLT_DK + DLT_DV > 128 && MODE == 0) {
-    // dense with exact head dims 64/128 or 128/128: chunks are copied HBM -> LDS asynchronously (a copy cannot zero-fill
-    // padded dims).  Measured per class and mode against the register-staged kernel: -4 % and -7 % here; at 64/64 the
-    // 8-wave workgroups lose (+14 %), and with a causal mask they lose in every class (+30 % and more: the waves of a
-    // 256-query workgroup see very different numbers of keys and the workgroup keeps its CU until the last one is done).
+  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
+    // dense / causal with exact head dims of 64 / 128: chunks are copied HBM -> LDS asynchronously (a copy cannot
+    // zero-fill padded dims).  Measured per class and mode against the register-staged kernel: dense -2 % (64/64), -4 %
+    // (64/128), -7 % (128/128); causal -4 % (64/64), -18 % (128/128).
     if (a.dk == DLT_DK && a.dv == DLT_DV && flash_async_staging()) {
-      constexpr int NP = FLASHD_FWD_NP, CK = FLASHD_FWD_CK, NW = FLASHD_FWD_NW;
+      constexpr int NP = FLASHD_FWD_NP, CK = FLASHD_FWD_CK(DLT_DK, DLT_DV), NW = FLASHD_FWD_NW(DLT_DK, DLT_DV);
       auto kern = flashd_fwd_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
       constexpr int own = 16 * NP * NW;
       constexpr int tile = own * (DLT_DV * 2 + 16);

@@ -178,7 +178,7 @@ def test_causal_block_order_over_heads(B, H, N, dk, dv):
 
 @pytest.mark.parametrize("causal,dk,dv,dtype", [
     (False, 64, 128, torch.bfloat16), (False, 64, 64, torch.float16), (False, 128, 128, torch.bfloat16),
-    (True, 64, 128, torch.float16), (True, 128, 128, torch.bfloat16)])
+    (True, 64, 128, torch.float16), (True, 128, 128, torch.bfloat16), (True, 64, 64, torch.bfloat16)])
 def test_chunk_boundaries_of_the_async_staged_kernels(causal, dk, dv, dtype):
     """Head dims of exactly 64 / 128 run on the kernels that copy chunks HBM -> LDS asynchronously into two or three
     buffers: lengths of one, two, three and four chunks (64 keys in the backward kernels, 128 in the forward kernel),
