@@ -112,10 +112,9 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
     dlt_timing_after(stream);
     DLT_CHECK_LAUNCH("flash dQ launch");
   }
-  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2 && !(DLT_DK + DLT_DV <= 128 && MODE == 0)) {
+  if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
     // dense / causal with exact head dims: chunks are copied HBM -> LDS asynchronously (a copy cannot zero-fill padded
-    // dims; in tile mode, where whole blocks are skipped, the register-staged kernel measured 1.5 % faster, and so it
-    // did dense at 64/64 (3 %))
+    // dims; in tile mode, where whole blocks are skipped, the register-staged kernel measured 1.5 % faster)
     const bool scalars_fit = a.ls[2] >= 0 && ((int64_t)a.Lq - 1) * a.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1);   // 32-bit offsets of the lse2 / delta copies
     if (a.dk_ == DLT_DK && a.dv_ == DLT_DV && scalars_fit && flash_async_staging()) {
       constexpr int NP = flash_np_kv(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
