@@ -301,18 +301,24 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
   };
   // o of step s: accumulators -> 16-byte row pieces (through the wave's LDS scratch), then the stores
   struct OutRows { u32x4 v[2]; int tok[2]; };
+  // The lane-derived addresses of the epilogue are computed from an opaque copy of the lane id: computed from `lane`
+  // itself they are hoisted out of the step loop and then live (spilled to scratch) across the products.
   auto transpose_o = [&](const SwamFwdOut& r, int s) {
     OutRows w;
     const int r_p = G.r0 + 8 * s + 4 * rg;
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
 #pragma unroll
-    for (int it = 0; it < 2; it++) w.tok[it] = swam_own_tok(G, r_p, c_p, (lane >> 3) + 8 * it);
+    for (int it = 0; it < 2; it++) w.tok[it] = swam_own_tok(G, r_p, c_p, (ln >> 3) + 8 * it);
     u32x4 unused[2];
-    swam_tile_transpose<CT, false>(scratch_of(s), r.acc, r.inv, lane, w.v, unused);
+    swam_tile_transpose<CT, false>(scratch_of(s), r.acc, r.inv, ln, w.v, unused);
     return w;
   };
   auto store_o = [&](const OutRows& w, const SwamFwdOut& r) {
     if (g == 0 && qo.tok >= 0) lseb[(int64_t)qo.tok * ls2] = r.lse2;
-    swam_store_rows<TIO>(ob, os2, w.tok, lane, w.v);
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    swam_store_rows<TIO>(ob, os2, w.tok, ln, w.v);
   };
 
   // The last step is peeled off so that inside the loop prefetch and commit are unconditional (a conditional
