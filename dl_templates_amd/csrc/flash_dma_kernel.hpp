@@ -577,9 +577,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
     if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
   }
   __syncthreads();
-  if (tid < 256)   // the tile writer walks the rows with 256 threads
+  int tw = tid;   // opaque copy: keeps the tile writer's addresses out of the registers that live across the chunk loop
+  asm volatile("" : "+v"(tw));
+  if (tw < 256)   // the tile writer walks the rows with 256 threads
     store_tile<TIO, TL, DV>(smem, PO, ob, flash_tok<false>(a.os, a.tm), a.os[3], a.dv, a.o_vec != 0, OWN,
-                            [&](int row) { return x0 + row < a.Lq ? (int64_t)(x0 + row) : (int64_t)-1; }, no_rope, tid);
+                            [&](int row) { return x0 + row < a.Lq ? (int64_t)(x0 + row) : (int64_t)-1; }, no_rope, tw);
 }
 
 // ---- dQ: own = queries; K and V stream.  Replaces _attn_bwd_dq (src/flash_attn.py:310-449) and, with fuse_delta, the

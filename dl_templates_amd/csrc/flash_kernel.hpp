@@ -468,8 +468,10 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
     if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
   }
   __syncthreads();
+  int tw = tid;   // opaque copy: keeps the tile writer's addresses out of the registers that live across the chunk loop
+  asm volatile("" : "+v"(tw));
   store_tile<TIO, TL, DV>(smem, PO, ob, flash_tok<IMG>(a.os, a.tm), a.os[3], a.dv, a.o_vec != 0, OWN,
-                          [&](int row) { return x0 + row < a.Lq ? (int64_t)(own_base + x0 + row) : (int64_t)-1; }, no_rope, tid);
+                          [&](int row) { return x0 + row < a.Lq ? (int64_t)(own_base + x0 + row) : (int64_t)-1; }, no_rope, tw);
 }
 
 // =============================================================================================
@@ -556,9 +558,13 @@ DLT_DEV void flash_write_grad(char* sT, f32x4 (&acc)[NP][D / 16], float mul, TIO
       for (int i = 0; i < 4; i++) row[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * mul);
   }
   __syncthreads();
-  if (tid < 256)   // the tile writer walks the rows with 256 threads
+  // the tile writer's addresses are computed from an opaque copy of the thread id: computed from `tid` itself they are
+  // hoisted above the chunk loop and occupy (or spill) registers across it
+  int tw = tid;
+  asm volatile("" : "+v"(tw));
+  if (tw < 256)   // the tile writer walks the rows with 256 threads
     store_tile<TIO, TL, D>(sT, PT, base, sn, sd, dact, vec, nrows,
-                           [&](int r) { return x0 + r < len ? (int64_t)(own_base + x0 + r) : (int64_t)-1; }, no_rope, tid);
+                           [&](int r) { return x0 + r < len ? (int64_t)(own_base + x0 + r) : (int64_t)-1; }, no_rope, tw);
   __syncthreads();
 }
 
