@@ -438,6 +438,23 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
   // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
   // for every copy in flight) at their first use inside every round of the chunk loop
   pin_loaded(qf);
+  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
+  // src/flash_attn.py:509-510), and the score products start from minus the running reference maximum (the C operand of
+  // the first product of a chain): the matrix pipe then delivers t = s2 - m2 directly and p = exp2(t) is the only vector
+  // instruction left per score.
+#pragma unroll
+  for (int p = 0; p < NP; p++)
+#pragma unroll
+    for (int c = 0; c < KC; c++) {
+      float e[8];
+      unpack8<CT>(qf[p][c], e);
+#pragma unroll
+      for (int i = 0; i < 8; i++) e[i] *= scale;
+      qf[p][c] = pack8<CT>(e);
+    }
+  f32x4 cinit[NP];   // -m2 in all four elements (0 while the block has seen no key)
+#pragma unroll
+  for (int p = 0; p < NP; p++) cinit[p] = f32x4{0.f, 0.f, 0.f, 0.f};
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -479,7 +496,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
       if constexpr (k < N1) {
         constexpr int kb = k / (2 * KC), mb = (k / KC) % 2, r = k % KC;
 #pragma unroll
-        for (int p = 0; p < NP; p++) s[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[p]);
+        for (int p = 0; p < NP; p++) s[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? cinit[p] : s[p]);
         if constexpr (r == KC - 1) {
 #pragma unroll
           for (int p = 0; p < NP; p++)
@@ -491,7 +508,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
             }
         }
         if constexpr (k == N1 - 1) {
-          // one softmax update per query block on the raw scores of the chunk
+          // one softmax update per query block; t holds the scaled scores relative to the reference maximum m2
 #pragma unroll
           for (int p = 0; p < NP; p++) {
             float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
@@ -500,21 +517,29 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
 #pragma unroll
               for (int i = 0; i < 4; i++) mx[i] = fmaxf(fmaxf(mx[i], t[p][kb2][2 * i]), t[p][kb2][2 * i + 1]);
             const float mloc = wave_max4(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])));
-            // the reference maximum only moves when a score exceeds it by more than 2^8 after scaling (see flash_kernel.hpp)
-            if (__builtin_amdgcn_ballot_w64((mloc - m_run[p]) * scale > 8.f)) {
+            // the reference maximum only moves when a score exceeds it by more than 2^8 (see flash_kernel.hpp), or when
+            // the block meets its first visible key
+            const bool first = m_run[p] == -INFINITY;
+            const bool move = first ? mloc != -INFINITY : mloc > 8.f;
+            if (__builtin_amdgcn_ballot_w64(move)) {
               keep_branch();
-              const float m_new = fmaxf(m_run[p], mloc);
-              const float alpha = fast_exp2((m_run[p] - m_new) * scale);
-              m_run[p] = m_new;
+              const float shift = move ? mloc : 0.f;
+              const float alpha = fast_exp2(-shift);
+              m_run[p] = move ? (first ? 0.f : m_run[p]) + mloc : m_run[p];
+              const float c0 = m_run[p] == -INFINITY ? 0.f : -m_run[p];
+              cinit[p] = f32x4{c0, c0, c0, c0};
 #pragma unroll
               for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
               acc_l[p] *= alpha;
+#pragma unroll
+              for (int kb2 = 0; kb2 < NKB; kb2++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) t[p][kb2][i] -= shift;
             }
-            const float neg_m2 = m_run[p] == -INFINITY ? 0.f : -m_run[p] * scale;
 #pragma unroll
             for (int kb2 = 0; kb2 < NKB; kb2++) {
 #pragma unroll
-              for (int i = 0; i < 8; i++) t[p][kb2][i] = fast_exp2(fmaf(t[p][kb2][i], scale, neg_m2));
+              for (int i = 0; i < 8; i++) t[p][kb2][i] = fast_exp2(t[p][kb2][i]);
               pb[p][kb2] = pack8<CT>(t[p][kb2]);
             }
           }
@@ -574,7 +599,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
     for (int d = 0; d < VB; d++)
 #pragma unroll
       for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * inv);
-    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
+    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] + fast_log2(lt);
   }
   __syncthreads();
   int tw = tid;   // opaque copy: keeps the tile writer's addresses out of the registers that live across the chunk loop
