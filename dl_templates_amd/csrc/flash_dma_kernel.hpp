@@ -211,6 +211,26 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   // for every copy in flight) at their first use inside every round of the chunk loop
   pin_loaded(kf);
   pin_loaded(vf);
+  // The own keys are multiplied by -sm_scale log2(e) once and the own values negated (the reference scales k on the host,
+  // src/flash_attn.py:509-510); the products start from the staged lse2 / delta of the lane's four queries, read from
+  // LDS straight into the C operand of the first product of a chain: the matrix pipe delivers -(s2 - lse2) and
+  // -(dP - delta), and p = exp2(-.), dS = -p (.) are the only vector instructions left per score (the signs are operand
+  // modifiers).
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+#pragma unroll
+    for (int c = 0; c < KC; c++) {
+      float e[8];
+      unpack8<CT>(kf[p][c], e);
+#pragma unroll
+      for (int i = 0; i < 8; i++) e[i] *= -scale;
+      kf[p][c] = pack8<CT>(e);
+    }
+#pragma unroll
+    for (int c = 0; c < VC; c++) {
+      vf[p][c].x ^= 0x80008000u; vf[p][c].y ^= 0x80008000u; vf[p][c].z ^= 0x80008000u; vf[p][c].w ^= 0x80008000u;
+    }
+  }
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -258,6 +278,9 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     };
     swa2_for<0, RD>([&](auto kc) __attribute__((always_inline)) { rd(kc); });
     f32x4 sv[2][NP], dp[2][NP], lq[2], dl[2];   // indexed by the parity of the half
+    // lse2 / delta of the lane's four queries of a half: read one half ahead, they are the C operands of its first products
+    lq[0] = __builtin_bit_cast(f32x4, swa2_lds16(sLse));
+    dl[0] = __builtin_bit_cast(f32x4, swa2_lds16(sDel));
     u32x4 pb[NQB][NP], dsb[NQB][NP];
     // piece u of the element-wise work of half hh: p = exp2(s scale - lse2), dS = p (dP - delta) for own block u / 2,
     // queries 2 (u % 2), 2 (u % 2) + 1 of the lane's four
@@ -268,13 +291,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const int i = i0_ + t;
-        float pv = fast_exp2(fmaf(sv[hh & 1][p][i], scale, -lq[hh & 1][i]));
+        float pv = fast_exp2(-sv[hh & 1][p][i]);
         if (tail) {
           const int qi = q0 + 16 * hh + 4 * g + i;
           pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
         }
         pr[t] = pv;
-        ds[t] = pv * (dp[hh & 1][p][i] - dl[hh & 1][i]);
+        ds[t] = -pv * dp[hh & 1][p][i];
       }
       const unsigned pw = pack2<CT>(pr[0], pr[1]), dw = pack2<CT>(ds[0], ds[1]);
       if constexpr (mb == 0 && i0_ == 0) { pb[qb_][p].x = pw; dsb[qb_][p].x = dw; }
@@ -285,10 +308,11 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     swa2_for<0, NT>([&](auto kc) __attribute__((always_inline)) {
       constexpr int k = decltype(kc)::value;
       if constexpr (k + RD < NT) rd(std::integral_constant<int, k + RD>{});
-      if constexpr (k < N1 && k % N1H == 0) {
-        constexpr int hh = k / N1H;
-        lq[hh & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 16 * hh * 4));
-        dl[hh & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sDel + 16 * hh * 4));
+      if constexpr (k < N1 && k % N1H == KC && k / N1H + 1 < NH) {
+        // (behind the first products of half hh, which consumed the registers this overwrites two halves ago)
+        constexpr int hn = k / N1H + 1;
+        lq[hn & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 16 * hn * 4));
+        dl[hn & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sDel + 16 * hn * 4));
       }
       __builtin_amdgcn_sched_barrier(0);
       const u32x4 x = ring[k % (RD + 1)];
@@ -296,8 +320,8 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
         constexpr int hh = k / N1H, r = k % N1H;
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-          if constexpr (r < KC) sv[hh & 1][p] = Mma<CT>::mfma(x, kf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sv[hh & 1][p]);
-          else dp[hh & 1][p] = Mma<CT>::mfma(x, vf[p][r - KC], r == KC ? f32x4{0.f, 0.f, 0.f, 0.f} : dp[hh & 1][p]);
+          if constexpr (r < KC) sv[hh & 1][p] = Mma<CT>::mfma(x, kf[p][r], r == 0 ? lq[hh & 1] : sv[hh & 1][p]);
+          else dp[hh & 1][p] = Mma<CT>::mfma(x, vf[p][r - KC], r == KC ? dl[hh & 1] : dp[hh & 1][p]);
         }
         if constexpr (hh >= 1 && r < NU) {
           ew(std::integral_constant<int, hh - 1>{}, std::integral_constant<int, r>{});
@@ -705,6 +729,24 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
   pin_loaded(dof);
 #pragma unroll
   for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
+  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
+  // src/flash_attn.py:509-510) and the products start from -lse2 and -delta of the lane's query (the C operand of the
+  // first product of a chain): the matrix pipe delivers s2 - lse2 and dP - delta, and p = exp2(.), dS = p (.) are the
+  // only vector instructions left per score.
+  f32x4 sinit[NP], dinit[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+#pragma unroll
+    for (int c = 0; c < KC; c++) {
+      float e[8];
+      unpack8<CT>(qf[p][c], e);
+#pragma unroll
+      for (int i = 0; i < 8; i++) e[i] *= scale;
+      qf[p][c] = pack8<CT>(e);
+    }
+    sinit[p] = f32x4{nlse[p], nlse[p], nlse[p], nlse[p]};
+    dinit[p] = f32x4{-del_n[p], -del_n[p], -del_n[p], -del_n[p]};
+  }
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -749,17 +791,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
           constexpr int mb = j / N1H, r = j % N1H;
 #pragma unroll
           for (int p = 0; p < NP; p++) {
-            if constexpr (r < KC) sv[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sv[p]);
-            else dp[p] = Mma<CT>::mfma(x, dof[p][r - KC], r == KC ? f32x4{0.f, 0.f, 0.f, 0.f} : dp[p]);
+            if constexpr (r < KC) sv[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? sinit[p] : sv[p]);
+            else dp[p] = Mma<CT>::mfma(x, dof[p][r - KC], r == KC ? dinit[p] : dp[p]);
           }
           if constexpr (r == N1H - 1) {
 #pragma unroll
             for (int p = 0; p < NP; p++) {
 #pragma unroll
               for (int i = 0; i < 4; i++) {
-                float pv = fast_exp2(fmaf(sv[p][i], scale, nlse[p]));
+                float pv = fast_exp2(sv[p][i]);
                 if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? pv : 0.f;
-                ds[p][4 * mb + i] = pv * (dp[p][i] - del_n[p]);
+                ds[p][4 * mb + i] = pv * dp[p][i];
               }
             }
             if constexpr (mb == 1) {
