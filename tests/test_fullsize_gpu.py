@@ -147,7 +147,8 @@ def test_c3_one_batch_fused_rope_against_cpu_oracle(save_rotated, monkeypatch):
 @pytest.mark.parametrize("save_rotated", [True, False])
 def test_c3_full_batch_fused_rope_equals_composition(save_rotated, monkeypatch):
     """Both fused variants (rotated q, k kept for the backward pass / rotated again in every tile load) at the
-    full size of config 3, bit-equal to the composition of the standalone rotation and the plain operator."""
+    full size of config 3 against the composition of the standalone rotation and the plain operator: bit-equal where
+    both run on the marching kernels (forward; backward from the kept rotated q, k)."""
     sw, _, fr = _mods()
     monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save_rotated)
     B, H, th, tw, d, W = 2, 8, 64, 64, 64, 6
@@ -164,7 +165,14 @@ def test_c3_full_batch_fused_rope_equals_composition(save_rotated, monkeypatch):
     o2 = sw.TiledSwa.apply(qr, kr, v2, 1, th, tw, W, W, 0.125)
     o2.backward(do)
     assert torch.equal(o, o2)
-    assert torch.equal(qg.grad, q2.grad) and torch.equal(kg.grad, k2.grad) and torch.equal(vg.grad, v2.grad)
+    if save_rotated:
+        assert torch.equal(qg.grad, q2.grad) and torch.equal(kg.grad, k2.grad) and torch.equal(vg.grad, v2.grad)
+    else:
+        # the backward pass that rotates in every tile load runs on the tile kernels, which scale the scores after the
+        # products; the marching kernels of the composition scale the own q / k fragments before them (one more
+        # rounding to bf16): equal within that rounding
+        rel = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
+        assert max(rel(qg.grad, q2.grad), rel(kg.grad, k2.grad), rel(vg.grad, v2.grad)) <= 1e-2
     assert torch.isfinite(o.float()).all() and torch.isfinite(qg.grad.float()).all()
 
 
