@@ -656,6 +656,24 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
   pin_loaded(dof);
 #pragma unroll
   for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
+  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
+  // src/flash_attn.py:509-510) and the first products start from -lse2 and -delta of the lane's query (the C operand):
+  // the matrix pipe delivers s2 - lse2 and dP - delta, and p = exp2(.), dS = p (.) are the only vector instructions left
+  // per score besides the masks.
+  f32x4 sinit[NP], dinit[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+#pragma unroll
+    for (int c_ = 0; c_ < KC; c_++) {
+      float e[8];
+      unpack8<CT>(qf[p][c_], e);
+#pragma unroll
+      for (int i = 0; i < 8; i++) e[i] *= scale;
+      qf[p][c_] = pack8<CT>(e);
+    }
+    sinit[p] = f32x4{nlse[p], nlse[p], nlse[p], nlse[p]};
+    dinit[p] = f32x4{-del_n[p], -del_n[p], -del_n[p], -del_n[p]};
+  }
 
   // `tail`: some keys of the chunk lie past the end or (causal) above the wave's first query, and every pair is tested.
   // It is a compile-time tag: as a run-time flag the test was folded into a select per element of every chunk.
@@ -696,8 +714,8 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
         f32x4 s[2], dp[2];
 #pragma unroll
         for (int mb = 0; mb < 2; mb++) {
-          s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
-          dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+          s[mb] = sinit[p];
+          dp[mb] = dinit[p];
 #pragma unroll
           for (int c_ = 0; c_ < KC; c_++) s[mb] = Mma<CT>::mfma(ka[mb][c_], qf[p][c_], s[mb]);
 #pragma unroll
@@ -709,10 +727,10 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
           const bool hv = !TILE || (k0 + 32 * kb + 16 * mb >= vlo[p] && k0 + 32 * kb + 16 * mb < vhi[p]);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            float pv = fast_exp2(fmaf(s[mb][i], scale, nlse[p]));
+            float pv = fast_exp2(s[mb][i]);
             if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? pv : 0.f;
             if (TILE) pv = hv ? pv : 0.f;
-            ds[4 * mb + i] = pv * (dp[mb][i] - del_n[p]);
+            ds[4 * mb + i] = pv * dp[mb][i];
           }
         }
         dsb[p] = pack8<CT>(ds);
@@ -832,6 +850,25 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
   __syncthreads();
   pin_loaded(kf);
   pin_loaded(vf);
+  // The own keys are multiplied by -sm_scale log2(e) once and the own values negated; the first products start from the
+  // staged lse2 / delta of the lane's four queries (the C operand): the matrix pipe delivers -(s2 - lse2) and
+  // -(dP - delta), and p = exp2(-.), dS = -p (.) are the only vector instructions left per score besides the masks (the
+  // signs are operand modifiers).
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+#pragma unroll
+    for (int c_ = 0; c_ < KC; c_++) {
+      float e[8];
+      unpack8<CT>(kf[p][c_], e);
+#pragma unroll
+      for (int i = 0; i < 8; i++) e[i] *= -scale;
+      kf[p][c_] = pack8<CT>(e);
+    }
+#pragma unroll
+    for (int c_ = 0; c_ < VC; c_++) {
+      vf[p][c_].x ^= 0x80008000u; vf[p][c_].y ^= 0x80008000u; vf[p][c_].z ^= 0x80008000u; vf[p][c_].w ^= 0x80008000u;
+    }
+  }
 
   // `tail`: some queries of the chunk lie past the end or (causal) below the wave's last own key (a compile-time tag, as
   // in the dQ kernel)
@@ -873,7 +910,7 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
 #pragma unroll
         for (int p = 0; p < NP; p++) {
           if (!bv[p]) continue;
-          f32x4 sv = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+          f32x4 sv = lq, dp = dl;
 #pragma unroll
           for (int c_ = 0; c_ < KC; c_++) sv = Mma<CT>::mfma(qa[c_], kf[p][c_], sv);
 #pragma unroll
@@ -881,14 +918,14 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
           const bool hv = !TILE || (q0 + 32 * qb_ + 16 * mb >= vlo[p] && q0 + 32 * qb_ + 16 * mb < vhi[p]);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            float pv = fast_exp2(fmaf(sv[i], scale, -lq[i]));
+            float pv = fast_exp2(-sv[i]);
             if (tail) {
               const int qi = q0 + 32 * qb_ + 16 * mb + 4 * g + i;
               pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
             }
             if (TILE) pv = hv ? pv : 0.f;
             pr[p][4 * mb + i] = pv;
-            ds[p][4 * mb + i] = pv * (dp[i] - dl[i]);
+            ds[p][4 * mb + i] = -pv * dp[i];
           }
         }
       }
