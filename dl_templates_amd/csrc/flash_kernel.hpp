@@ -311,6 +311,23 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   if (W.nchunks > 0) commit();
   __syncthreads();
   pin_loaded(qf);
+  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
+  // src/flash_attn.py:509-510), and the score products start from minus the running reference maximum (the C operand of
+  // the first product of a chain): the matrix pipe then delivers t = s2 - m2 directly and p = exp2(t) is the only vector
+  // instruction left per score besides the masks.  m_run is kept in log2 units.
+#pragma unroll
+  for (int p = 0; p < NP; p++)
+#pragma unroll
+    for (int c_ = 0; c_ < KC; c_++) {
+      float e[8];
+      unpack8<CT>(qf[p][c_], e);
+#pragma unroll
+      for (int i = 0; i < 8; i++) e[i] *= scale;
+      qf[p][c_] = pack8<CT>(e);
+    }
+  f32x4 cinit[NP];   // -m2 in all four elements (0 while the block has seen no key)
+#pragma unroll
+  for (int p = 0; p < NP; p++) cinit[p] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // products and softmax update of the chunk resident in LDS
   // `tail` (dense / causal): some keys of the chunk lie past the end or (causal) above the wave's first query, and every
@@ -359,7 +376,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
 #pragma unroll
         for (int p = 0; p < NP; p++) {
           if (bv[p][kb]) {
-            f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+            f32x4 s0 = cinit[p], s1 = cinit[p];
 #pragma unroll
             for (int c_ = 0; c_ < KC; c_++) {
               s0 = Mma<CT>::mfma(ka[0][c_], qf[p][c_], s0);
@@ -398,20 +415,27 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
         // The reference maximum only moves when a score exceeds it by more than 2^8 after scaling: p stays below 2^8,
         // well inside the range of the 16-bit operand and of the fp32 sums, and most chunks skip the rescaling of the
         // accumulators.  o and lse do not depend on which reference was used.
-        if (__builtin_amdgcn_ballot_w64((mloc - m_run[p]) * scale > 8.f)) {
+        const bool first = m_run[p] == -INFINITY;
+        const bool move = first ? mloc != -INFINITY : mloc > 8.f;   // t is relative to the reference already
+        if (__builtin_amdgcn_ballot_w64(move)) {
           keep_branch();
-          const float m_new = fmaxf(m_run[p], mloc);   // finite here
-          const float alpha = fast_exp2((m_run[p] - m_new) * scale);
-          m_run[p] = m_new;
+          const float shift = move ? mloc : 0.f;
+          const float alpha = fast_exp2(-shift);
+          m_run[p] = move ? (first ? 0.f : m_run[p]) + mloc : m_run[p];
+          const float c0 = m_run[p] == -INFINITY ? 0.f : -m_run[p];
+          cinit[p] = f32x4{c0, c0, c0, c0};
 #pragma unroll
           for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
           acc_l[p] *= alpha;
+#pragma unroll
+          for (int kb = 0; kb < NKB; kb++)
+#pragma unroll
+            for (int i = 0; i < 8; i++) t[p][kb][i] -= shift;
         }
-        const float neg_m2 = m_run[p] == -INFINITY ? 0.f : -m_run[p] * scale;   // -inf: a block that has seen no key yet
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
-          for (int i = 0; i < 8; i++) t[p][kb][i] = fast_exp2(fmaf(t[p][kb][i], scale, neg_m2));
+          for (int i = 0; i < 8; i++) t[p][kb][i] = fast_exp2(t[p][kb][i]);
           pb[p][kb] = pack8<CT>(t[p][kb]);
         }
       }
@@ -465,7 +489,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
     for (int d = 0; d < VB; d++)
 #pragma unroll
       for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * inv);
-    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
+    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] + fast_log2(lt);
   }
   __syncthreads();
   int tw = tid;   // opaque copy: keeps the tile writer's addresses out of the registers that live across the chunk loop
