@@ -211,26 +211,15 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
   // for every copy in flight) at their first use inside every round of the chunk loop
   pin_loaded(kf);
   pin_loaded(vf);
-  // The own keys are multiplied by -sm_scale log2(e) once and the own values negated (the reference scales k on the host,
-  // src/flash_attn.py:509-510); the products start from the staged lse2 / delta of the lane's four queries, read from
-  // LDS straight into the C operand of the first product of a chain: the matrix pipe delivers -(s2 - lse2) and
-  // -(dP - delta), and p = exp2(-.), dS = -p (.) are the only vector instructions left per score (the signs are operand
-  // modifiers).
+  // The own values are negated and the dP products start from the staged delta of the lane's four queries, read from LDS
+  // straight into the C operand of the first product of a chain: the matrix pipe delivers -(dP - delta), and dS = -p (.)
+  // (the sign is an operand modifier).
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-#pragma unroll
-    for (int c = 0; c < KC; c++) {
-      float e[8];
-      unpack8<CT>(kf[p][c], e);
-#pragma unroll
-      for (int i = 0; i < 8; i++) e[i] *= -scale;
-      kf[p][c] = pack8<CT>(e);
-    }
+  for (int p = 0; p < NP; p++)
 #pragma unroll
     for (int c = 0; c < VC; c++) {
       vf[p][c].x ^= 0x80008000u; vf[p][c].y ^= 0x80008000u; vf[p][c].z ^= 0x80008000u; vf[p][c].w ^= 0x80008000u;
     }
-  }
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -278,8 +267,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     };
     swa2_for<0, RD>([&](auto kc) __attribute__((always_inline)) { rd(kc); });
     f32x4 sv[2][NP], dp[2][NP], lq[2], dl[2];   // indexed by the parity of the half
-    // lse2 / delta of the lane's four queries of a half: read one half ahead, they are the C operands of its first products
-    lq[0] = __builtin_bit_cast(f32x4, swa2_lds16(sLse));
+    // delta of the lane's four queries of a half is the C operand of its first dP product: read one half ahead
     dl[0] = __builtin_bit_cast(f32x4, swa2_lds16(sDel));
     u32x4 pb[NQB][NP], dsb[NQB][NP];
     // piece u of the element-wise work of half hh: p = exp2(s scale - lse2), dS = p (dP - delta) for own block u / 2,
@@ -291,7 +279,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 #pragma unroll
       for (int t = 0; t < 2; t++) {
         const int i = i0_ + t;
-        float pv = fast_exp2(-sv[hh & 1][p][i]);
+        float pv = fast_exp2(fmaf(sv[hh & 1][p][i], scale, -lq[hh & 1][i]));
         if (tail) {
           const int qi = q0 + 16 * hh + 4 * g + i;
           pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;
@@ -308,10 +296,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     swa2_for<0, NT>([&](auto kc) __attribute__((always_inline)) {
       constexpr int k = decltype(kc)::value;
       if constexpr (k + RD < NT) rd(std::integral_constant<int, k + RD>{});
+      if constexpr (k < N1 && k % N1H == 0) {
+        constexpr int hh = k / N1H;
+        lq[hh & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 16 * hh * 4));
+      }
       if constexpr (k < N1 && k % N1H == KC && k / N1H + 1 < NH) {
-        // (behind the first products of half hh, which consumed the registers this overwrites two halves ago)
+        // (the dP products of half hh - 1 consumed the registers this overwrites)
         constexpr int hn = k / N1H + 1;
-        lq[hn & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 16 * hn * 4));
         dl[hn & 1] = __builtin_bit_cast(f32x4, swa2_lds16(sDel + 16 * hn * 4));
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -320,7 +311,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
         constexpr int hh = k / N1H, r = k % N1H;
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-          if constexpr (r < KC) sv[hh & 1][p] = Mma<CT>::mfma(x, kf[p][r], r == 0 ? lq[hh & 1] : sv[hh & 1][p]);
+          if constexpr (r < KC) sv[hh & 1][p] = Mma<CT>::mfma(x, kf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sv[hh & 1][p]);
           else dp[hh & 1][p] = Mma<CT>::mfma(x, vf[p][r - KC], r == KC ? dl[hh & 1] : dp[hh & 1][p]);
         }
         if constexpr (hh >= 1 && r < NU) {
@@ -462,23 +453,6 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
   // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
   // for every copy in flight) at their first use inside every round of the chunk loop
   pin_loaded(qf);
-  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
-  // src/flash_attn.py:509-510), and the score products start from minus the running reference maximum (the C operand of
-  // the first product of a chain): the matrix pipe then delivers t = s2 - m2 directly and p = exp2(t) is the only vector
-  // instruction left per score.
-#pragma unroll
-  for (int p = 0; p < NP; p++)
-#pragma unroll
-    for (int c = 0; c < KC; c++) {
-      float e[8];
-      unpack8<CT>(qf[p][c], e);
-#pragma unroll
-      for (int i = 0; i < 8; i++) e[i] *= scale;
-      qf[p][c] = pack8<CT>(e);
-    }
-  f32x4 cinit[NP];   // -m2 in all four elements (0 while the block has seen no key)
-#pragma unroll
-  for (int p = 0; p < NP; p++) cinit[p] = f32x4{0.f, 0.f, 0.f, 0.f};
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -520,7 +494,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
       if constexpr (k < N1) {
         constexpr int kb = k / (2 * KC), mb = (k / KC) % 2, r = k % KC;
 #pragma unroll
-        for (int p = 0; p < NP; p++) s[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? cinit[p] : s[p]);
+        for (int p = 0; p < NP; p++) s[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : s[p]);
         if constexpr (r == KC - 1) {
 #pragma unroll
           for (int p = 0; p < NP; p++)
@@ -532,7 +506,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
             }
         }
         if constexpr (k == N1 - 1) {
-          // one softmax update per query block; t holds the scaled scores relative to the reference maximum m2
+          // one softmax update per query block on the raw scores of the chunk
 #pragma unroll
           for (int p = 0; p < NP; p++) {
             float mx[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
@@ -541,29 +515,21 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
 #pragma unroll
               for (int i = 0; i < 4; i++) mx[i] = fmaxf(fmaxf(mx[i], t[p][kb2][2 * i]), t[p][kb2][2 * i + 1]);
             const float mloc = wave_max4(fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3])));
-            // the reference maximum only moves when a score exceeds it by more than 2^8 (see flash_kernel.hpp), or when
-            // the block meets its first visible key
-            const bool first = m_run[p] == -INFINITY;
-            const bool move = first ? mloc != -INFINITY : mloc > 8.f;
-            if (__builtin_amdgcn_ballot_w64(move)) {
+            // the reference maximum only moves when a score exceeds it by more than 2^8 after scaling (see flash_kernel.hpp)
+            if (__builtin_amdgcn_ballot_w64((mloc - m_run[p]) * scale > 8.f)) {
               keep_branch();
-              const float shift = move ? mloc : 0.f;
-              const float alpha = fast_exp2(-shift);
-              m_run[p] = move ? (first ? 0.f : m_run[p]) + mloc : m_run[p];
-              const float c0 = m_run[p] == -INFINITY ? 0.f : -m_run[p];
-              cinit[p] = f32x4{c0, c0, c0, c0};
+              const float m_new = fmaxf(m_run[p], mloc);
+              const float alpha = fast_exp2((m_run[p] - m_new) * scale);
+              m_run[p] = m_new;
 #pragma unroll
               for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
               acc_l[p] *= alpha;
-#pragma unroll
-              for (int kb2 = 0; kb2 < NKB; kb2++)
-#pragma unroll
-                for (int i = 0; i < 8; i++) t[p][kb2][i] -= shift;
             }
+            const float neg_m2 = m_run[p] == -INFINITY ? 0.f : -m_run[p] * scale;
 #pragma unroll
             for (int kb2 = 0; kb2 < NKB; kb2++) {
 #pragma unroll
-              for (int i = 0; i < 8; i++) t[p][kb2][i] = fast_exp2(t[p][kb2][i]);
+              for (int i = 0; i < 8; i++) t[p][kb2][i] = fast_exp2(fmaf(t[p][kb2][i], scale, neg_m2));
               pb[p][kb2] = pack8<CT>(t[p][kb2]);
             }
           }
@@ -623,7 +589,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
     for (int d = 0; d < VB; d++)
 #pragma unroll
       for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * inv);
-    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] + fast_log2(lt);
+    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
   }
   __syncthreads();
   int tw = tid;   // opaque copy: keeps the tile writer's addresses out of the registers that live across the chunk loop
@@ -729,24 +695,13 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
   pin_loaded(dof);
 #pragma unroll
   for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
-  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
-  // src/flash_attn.py:509-510) and the products start from -lse2 and -delta of the lane's query (the C operand of the
-  // first product of a chain): the matrix pipe delivers s2 - lse2 and dP - delta, and p = exp2(.), dS = p (.) are the
-  // only vector instructions left per score.
-  f32x4 sinit[NP], dinit[NP];
+  // The dP products start from -delta of the lane's query (the C operand of the first product of a chain): the matrix
+  // pipe delivers dP - delta.  (Folding the scale into the own queries and -lse2 into the score products the same way
+  // would save two more vector instructions per score, but rounds q sm_scale to 16 bits: at bf16 the forward error grew
+  // from 1.0e-2 to 2.6e-2 at sm_scale sqrt(d) = 4.)
+  f32x4 dinit[NP];
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-#pragma unroll
-    for (int c = 0; c < KC; c++) {
-      float e[8];
-      unpack8<CT>(qf[p][c], e);
-#pragma unroll
-      for (int i = 0; i < 8; i++) e[i] *= scale;
-      qf[p][c] = pack8<CT>(e);
-    }
-    sinit[p] = f32x4{nlse[p], nlse[p], nlse[p], nlse[p]};
-    dinit[p] = f32x4{-del_n[p], -del_n[p], -del_n[p], -del_n[p]};
-  }
+  for (int p = 0; p < NP; p++) dinit[p] = f32x4{-del_n[p], -del_n[p], -del_n[p], -del_n[p]};
   __syncthreads();
 
   auto chunk_tail = [&](const int ci) {
@@ -791,7 +746,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
           constexpr int mb = j / N1H, r = j % N1H;
 #pragma unroll
           for (int p = 0; p < NP; p++) {
-            if constexpr (r < KC) sv[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? sinit[p] : sv[p]);
+            if constexpr (r < KC) sv[p] = Mma<CT>::mfma(x, qf[p][r], r == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : sv[p]);
             else dp[p] = Mma<CT>::mfma(x, dof[p][r - KC], r == KC ? dinit[p] : dp[p]);
           }
           if constexpr (r == N1H - 1) {
@@ -799,7 +754,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
             for (int p = 0; p < NP; p++) {
 #pragma unroll
               for (int i = 0; i < 4; i++) {
-                float pv = fast_exp2(sv[p][i]);
+                float pv = fast_exp2(fmaf(sv[p][i], scale, nlse[p]));
                 if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? pv : 0.f;
                 ds[p][4 * mb + i] = pv * dp[p][i];
               }

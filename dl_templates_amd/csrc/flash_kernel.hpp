@@ -311,23 +311,6 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   if (W.nchunks > 0) commit();
   __syncthreads();
   pin_loaded(qf);
-  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
-  // src/flash_attn.py:509-510), and the score products start from minus the running reference maximum (the C operand of
-  // the first product of a chain): the matrix pipe then delivers t = s2 - m2 directly and p = exp2(t) is the only vector
-  // instruction left per score besides the masks.  m_run is kept in log2 units.
-#pragma unroll
-  for (int p = 0; p < NP; p++)
-#pragma unroll
-    for (int c_ = 0; c_ < KC; c_++) {
-      float e[8];
-      unpack8<CT>(qf[p][c_], e);
-#pragma unroll
-      for (int i = 0; i < 8; i++) e[i] *= scale;
-      qf[p][c_] = pack8<CT>(e);
-    }
-  f32x4 cinit[NP];   // -m2 in all four elements (0 while the block has seen no key)
-#pragma unroll
-  for (int p = 0; p < NP; p++) cinit[p] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // products and softmax update of the chunk resident in LDS
   // `tail` (dense / causal): some keys of the chunk lie past the end or (causal) above the wave's first query, and every
@@ -376,7 +359,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
 #pragma unroll
         for (int p = 0; p < NP; p++) {
           if (bv[p][kb]) {
-            f32x4 s0 = cinit[p], s1 = cinit[p];
+            f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c_ = 0; c_ < KC; c_++) {
               s0 = Mma<CT>::mfma(ka[0][c_], qf[p][c_], s0);
@@ -415,27 +398,20 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
         // The reference maximum only moves when a score exceeds it by more than 2^8 after scaling: p stays below 2^8,
         // well inside the range of the 16-bit operand and of the fp32 sums, and most chunks skip the rescaling of the
         // accumulators.  o and lse do not depend on which reference was used.
-        const bool first = m_run[p] == -INFINITY;
-        const bool move = first ? mloc != -INFINITY : mloc > 8.f;   // t is relative to the reference already
-        if (__builtin_amdgcn_ballot_w64(move)) {
+        if (__builtin_amdgcn_ballot_w64((mloc - m_run[p]) * scale > 8.f)) {
           keep_branch();
-          const float shift = move ? mloc : 0.f;
-          const float alpha = fast_exp2(-shift);
-          m_run[p] = move ? (first ? 0.f : m_run[p]) + mloc : m_run[p];
-          const float c0 = m_run[p] == -INFINITY ? 0.f : -m_run[p];
-          cinit[p] = f32x4{c0, c0, c0, c0};
+          const float m_new = fmaxf(m_run[p], mloc);   // finite here
+          const float alpha = fast_exp2((m_run[p] - m_new) * scale);
+          m_run[p] = m_new;
 #pragma unroll
           for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
           acc_l[p] *= alpha;
-#pragma unroll
-          for (int kb = 0; kb < NKB; kb++)
-#pragma unroll
-            for (int i = 0; i < 8; i++) t[p][kb][i] -= shift;
         }
+        const float neg_m2 = m_run[p] == -INFINITY ? 0.f : -m_run[p] * scale;   // -inf: a block that has seen no key yet
 #pragma unroll
         for (int kb = 0; kb < NKB; kb++) {
 #pragma unroll
-          for (int i = 0; i < 8; i++) t[p][kb][i] = fast_exp2(t[p][kb][i]);
+          for (int i = 0; i < 8; i++) t[p][kb][i] = fast_exp2(fmaf(t[p][kb][i], scale, neg_m2));
           pb[p][kb] = pack8<CT>(t[p][kb]);
         }
       }
@@ -489,7 +465,7 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
     for (int d = 0; d < VB; d++)
 #pragma unroll
       for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * inv);
-    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] + fast_log2(lt);
+    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
   }
   __syncthreads();
   int tw = tid;   // opaque copy: keeps the tile writer's addresses out of the registers that live across the chunk loop
@@ -680,24 +656,11 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
   pin_loaded(dof);
 #pragma unroll
   for (int p = 0; p < NP; p++) { pin_loaded(nlse[p]); pin_loaded(del_n[p]); }
-  // The own queries are multiplied by sm_scale log2(e) once (the reference does the same to k on the host,
-  // src/flash_attn.py:509-510) and the first products start from -lse2 and -delta of the lane's query (the C operand):
-  // the matrix pipe delivers s2 - lse2 and dP - delta, and p = exp2(.), dS = p (.) are the only vector instructions left
-  // per score besides the masks.
-  f32x4 sinit[NP], dinit[NP];
+  // The dP products start from -delta of the lane's query (the C operand of the first product of a chain): the matrix
+  // pipe delivers dP - delta.
+  f32x4 dinit[NP];
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-#pragma unroll
-    for (int c_ = 0; c_ < KC; c_++) {
-      float e[8];
-      unpack8<CT>(qf[p][c_], e);
-#pragma unroll
-      for (int i = 0; i < 8; i++) e[i] *= scale;
-      qf[p][c_] = pack8<CT>(e);
-    }
-    sinit[p] = f32x4{nlse[p], nlse[p], nlse[p], nlse[p]};
-    dinit[p] = f32x4{-del_n[p], -del_n[p], -del_n[p], -del_n[p]};
-  }
+  for (int p = 0; p < NP; p++) dinit[p] = f32x4{-del_n[p], -del_n[p], -del_n[p], -del_n[p]};
 
   // `tail`: some keys of the chunk lie past the end or (causal) above the wave's first query, and every pair is tested.
   // It is a compile-time tag: as a run-time flag the test was folded into a select per element of every chunk.
@@ -738,7 +701,7 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
         f32x4 s[2], dp[2];
 #pragma unroll
         for (int mb = 0; mb < 2; mb++) {
-          s[mb] = sinit[p];
+          s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
           dp[mb] = dinit[p];
 #pragma unroll
           for (int c_ = 0; c_ < KC; c_++) s[mb] = Mma<CT>::mfma(ka[mb][c_], qf[p][c_], s[mb]);
@@ -751,7 +714,7 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
           const bool hv = !TILE || (k0 + 32 * kb + 16 * mb >= vlo[p] && k0 + 32 * kb + 16 * mb < vhi[p]);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            float pv = fast_exp2(s[mb][i]);
+            float pv = fast_exp2(fmaf(s[mb][i], scale, nlse[p]));
             if (tail) pv = (k0 + 32 * kb + 16 * mb + 4 * g + i) <= klim[p] ? pv : 0.f;
             if (TILE) pv = hv ? pv : 0.f;
             ds[4 * mb + i] = pv * dp[mb][i];
@@ -874,25 +837,15 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
   __syncthreads();
   pin_loaded(kf);
   pin_loaded(vf);
-  // The own keys are multiplied by -sm_scale log2(e) once and the own values negated; the first products start from the
-  // staged lse2 / delta of the lane's four queries (the C operand): the matrix pipe delivers -(s2 - lse2) and
-  // -(dP - delta), and p = exp2(-.), dS = -p (.) are the only vector instructions left per score besides the masks (the
-  // signs are operand modifiers).
+  // The own values are negated and the dP products start from the staged delta of the lane's four queries (the C operand
+  // of the first product of a chain): the matrix pipe delivers -(dP - delta), and dS = -p (.) (the sign is an operand
+  // modifier).
 #pragma unroll
-  for (int p = 0; p < NP; p++) {
-#pragma unroll
-    for (int c_ = 0; c_ < KC; c_++) {
-      float e[8];
-      unpack8<CT>(kf[p][c_], e);
-#pragma unroll
-      for (int i = 0; i < 8; i++) e[i] *= -scale;
-      kf[p][c_] = pack8<CT>(e);
-    }
+  for (int p = 0; p < NP; p++)
 #pragma unroll
     for (int c_ = 0; c_ < VC; c_++) {
       vf[p][c_].x ^= 0x80008000u; vf[p][c_].y ^= 0x80008000u; vf[p][c_].z ^= 0x80008000u; vf[p][c_].w ^= 0x80008000u;
     }
-  }
 
   // `tail`: some queries of the chunk lie past the end or (causal) below the wave's last own key (a compile-time tag, as
   // in the dQ kernel)
@@ -934,7 +887,7 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
 #pragma unroll
         for (int p = 0; p < NP; p++) {
           if (!bv[p]) continue;
-          f32x4 sv = lq, dp = dl;
+          f32x4 sv = {0.f, 0.f, 0.f, 0.f}, dp = dl;
 #pragma unroll
           for (int c_ = 0; c_ < KC; c_++) sv = Mma<CT>::mfma(qa[c_], kf[p][c_], sv);
 #pragma unroll
@@ -942,7 +895,7 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
           const bool hv = !TILE || (q0 + 32 * qb_ + 16 * mb >= vlo[p] && q0 + 32 * qb_ + 16 * mb < vhi[p]);
 #pragma unroll
           for (int i = 0; i < 4; i++) {
-            float pv = fast_exp2(-sv[i]);
+            float pv = fast_exp2(fmaf(sv[i], scale, -lq[i]));
             if (tail) {
               const int qi = q0 + 32 * qb_ + 16 * mb + 4 * g + i;
               pv = (qi >= qmin[p] && qi < a.Lq) ? pv : 0.f;

@@ -96,18 +96,8 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
   pin_loaded(qf);
   pin_loaded(dof);
   pin_loaded(neg_lse);
-  // The own queries are multiplied by sm_scale log2(e) once and the first products start from -lse2 and -delta of the
-  // lane's query (the C operand): the matrix pipe delivers s2 - lse2 and dP - delta, and p = exp2(.), dS = p (.) are the
-  // only vector instructions left per score besides the window mask.
-#pragma unroll
-  for (int c = 0; c < KC; c++) {
-    float e[8];
-    unpack8<CT>(qf[c], e);
-#pragma unroll
-    for (int i = 0; i < 8; i++) e[i] *= scale;
-    qf[c] = pack8<CT>(e);
-  }
-  const f32x4 sinit = {neg_lse, neg_lse, neg_lse, neg_lse}, dinit = {-del_n, -del_n, -del_n, -del_n};
+  // the dP products start from -delta of the lane's query (the C operand): the matrix pipe delivers dP - delta
+  const f32x4 dinit = {-del_n, -del_n, -del_n, -del_n};
   __syncthreads();
 
   // `cur` and `nxt` are distinct chunk buffers (see the forward kernel)
@@ -130,7 +120,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
         const int cg = 2 * kb + half;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const float p = fast_exp2(s[half][i]);
+          const float p = fast_exp2(fmaf(s[half][i], scale, neg_lse));
           const float ds = p * dp[half][i];
           t[4 * half + i] = swa2_visible(W, row_vis, cg, i, ncg) ? ds : 0.f;
         }
@@ -139,7 +129,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
       if constexpr (more) swa2_issue_one<C, 4 * kb>(st, nrow, ndst);
       swa2_read_a<C, 2 * kb>(sV, L, xv[0]);
       __builtin_amdgcn_sched_barrier(0);
-      s[0] = sinit;
+      s[0] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KC; c++) s[0] = Mma<CT>::mfma(xk[0][c], qf[c], s[0]);
       __builtin_amdgcn_sched_barrier(0);
@@ -155,7 +145,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
       if constexpr (more) swa2_issue_one<C, 4 * kb + 2>(st, nrow, ndst);
       swa2_read_a<C, 2 * kb + 1>(sV, L, xv[1]);
       __builtin_amdgcn_sched_barrier(0);
-      s[1] = sinit;
+      s[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KC; c++) s[1] = Mma<CT>::mfma(xk[1][c], qf[c], s[1]);
       __builtin_amdgcn_sched_barrier(0);
@@ -276,17 +266,11 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
   // for every copy in flight) at their first use inside every round of the chunk loop
   pin_loaded(kf);
   pin_loaded(vf);
-  // The own keys are multiplied by -sm_scale log2(e) once and the own values negated; the first products start from the
-  // staged lse2 / delta of the lane's four queries (read from LDS straight into the C operand, one stage or more ahead):
-  // the matrix pipe delivers -(s2 - lse2) and -(dP - delta), and p = exp2(-.), dS = -p (.) are the only vector
-  // instructions left per score besides the window mask (the signs are operand modifiers).
+  // The own values are negated and the dP products start from the staged delta of the lane's four queries (read from LDS
+  // straight into the C operand, a stage or more ahead): the matrix pipe delivers -(dP - delta), and dS = -p (.) (the sign
+  // is an operand modifier).
 #pragma unroll
   for (int c = 0; c < KC; c++) {
-    float e[8];
-    unpack8<CT>(kf[c], e);
-#pragma unroll
-    for (int i = 0; i < 8; i++) e[i] *= -scale;
-    kf[c] = pack8<CT>(e);
     vf[c].x ^= 0x80008000u; vf[c].y ^= 0x80008000u; vf[c].z ^= 0x80008000u; vf[c].w ^= 0x80008000u;
   }
   __syncthreads();
@@ -311,12 +295,12 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
       constexpr int kb = decltype(kbc)::value;
       u32x4 pp, pd;
       // P and dS of one column group, packed: p = exp2(s scale - lse2) where visible, dS = p (dP - delta)
-      auto elementwise = [&](const int half, const f32x4& sv, const f32x4& dpv) {
+      auto elementwise = [&](const int half, const f32x4& sv, const f32x4& dpv, const f32x4& lse4) {
         const int cg = 2 * kb + half;
         float tp[4], td[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-          const float p = fast_exp2(-sv[i]);
+          const float p = fast_exp2(fmaf(sv[i], scale, -lse4[i]));
           const bool vis = swa2_visible(W, row_vis, cg, i, ncg);
           tp[i] = vis ? p : 0.f;
           td[i] = vis ? -p * dpv[i] : 0.f;
@@ -335,7 +319,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
       const f32x4 lse_o = __builtin_bit_cast(f32x4, swa2_lds16(sLse + 32 * kb + 16));
       const f32x4 del_o = __builtin_bit_cast(f32x4, swa2_lds16(sDel + 32 * kb + 16));
       __builtin_amdgcn_sched_barrier(0);
-      f32x4 s0 = lse_e;
+      f32x4 s0 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KC; c++) s0 = Mma<CT>::mfma(x[0][c], kf[c], s0);
       __builtin_amdgcn_sched_barrier(0);
@@ -351,10 +335,10 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
       if constexpr (more) swa2_issue_one<C, 4 * kb + 2>(st, nrow, ndst);
       swa2_read_a<C, 2 * kb + 1>(sD, L, x[1]);
       __builtin_amdgcn_sched_barrier(0);
-      f32x4 s1 = lse_o;
+      f32x4 s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KC; c++) s1 = Mma<CT>::mfma(x[0][c], kf[c], s1);
-      elementwise(0, s0, dp0);
+      elementwise(0, s0, dp0, lse_e);
       SWA2_MIX(KC, 20 / KC)
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 4: dP of the odd column group
@@ -367,7 +351,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
       // ---- stage 5: elementwise work of the odd column group
       if constexpr (more) swa2_issue_one<C, 4 * kb + 3>(st, nrow, ndst);
       swa2_read_tr<C, kb, 2, 2>(sD, L, tr[1]);
-      elementwise(1, s1, dp1);
+      elementwise(1, s1, dp1, lse_o);
       __builtin_amdgcn_sched_barrier(0);
       // ---- stage 6: dV^T += dO^T P over NP2 pairs of 16-dim blocks, then dK^T += Q^T dS over NP2 pairs.  Pair j of the
       //      sequence sits in tr[j & 1]; pair j + 2 is requested once the products of pair j are issued, and the first

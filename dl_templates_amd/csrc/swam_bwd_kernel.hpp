@@ -97,20 +97,6 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
     w.lse = lseb[(int64_t)(w.tok >= 0 ? w.tok : 0) * ls2];
   };
   auto own_pin = [&](const Own& w) { swam_frag_pin(w.q); swam_frag_pin(w.d_o); swam_frag_pin(w.o); pin_loaded(w.lse); };
-  // The own queries are multiplied by sm_scale log2(e) once per step (the reference scales k on the host,
-  // src/flash_attn.py:509-510; src/tiled_swa.py applies the scale to the scores) and the first products start from -lse2
-  // and -delta of the lane's query (the C operand): the matrix pipe delivers s2 - lse2 and dP - delta, and p = exp2(.),
-  // dS = p (.) are the only vector instructions left per score besides the window mask.
-  auto own_scale = [&](Own& w) {
-#pragma unroll
-    for (int c = 0; c < 2; c++) {
-      float e[8];
-      unpack8<CT>(w.q.f[c], e);
-#pragma unroll
-      for (int j = 0; j < 8; j++) e[j] *= scale;
-      w.q.f[c] = pack8<CT>(e);
-    }
-  };
   // delta = rowsum(o * dO) of the own tokens, published for the dK/dV kernel
   auto own_delta = [&](const Own& w) {
     float part = 0.f;
@@ -152,7 +138,6 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
     }
     own_pin(cur);
     del_n = own_delta(cur);
-    own_scale(cur);
   }
   __syncthreads();
 
@@ -167,8 +152,9 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
     const bool q_ok = (r_p + qr_l < G.TR) && (c_p + qc_l < G.TC);
     const int rlo = dlt_imax(qr_l, G.WR - r_p), rhi = dlt_imin(qr_l + 2 * G.WR, G.TR - 1 - r_p + G.WR);
     const int cspan = q_ok ? chi - clo : -1;
+    // the dP products start from -delta of the lane's query (the C operand): the matrix pipe delivers dP - delta
     const float neg_lse = -cur.lse, neg_del = -del_n;
-    const f32x4 sinit = {neg_lse, neg_lse, neg_lse, neg_lse}, dinit = {neg_del, neg_del, neg_del, neg_del};
+    const f32x4 dinit = {neg_del, neg_del, neg_del, neg_del};
     int sb[4];
     {
       const int s5 = (2 * s + rg) % SWAM_NSLOT;
@@ -205,15 +191,15 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
         __builtin_amdgcn_sched_barrier(0);
         const u32x4(&kc)[2] = ka[hb & 1];
         const u32x4(&vc)[2] = va[hb & 1];
-        f32x4 sv, pv;
-        sv = Mma<CT>::mfma(kc[0], qf0, sinit);
+        f32x4 sv = {0.f, 0.f, 0.f, 0.f}, pv;
+        sv = Mma<CT>::mfma(kc[0], qf0, sv);
         pv = Mma<CT>::mfma(vc[0], df0, dinit);
         sv = Mma<CT>::mfma(kc[1], qf1, sv);
         pv = Mma<CT>::mfma(vc[1], df1, pv);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const bool vis = row_vis & ((unsigned)(8 * kb + 4 * mb + i - clo) <= (unsigned)cspan);
-          const float e = fast_exp2(vis ? sv[i] : -INFINITY);
+          const float e = fast_exp2(fmaf(sv[i], scale, vis ? neg_lse : -INFINITY));
           ds[4 * mb + i] = e * pv[i];
         }
       }
@@ -263,7 +249,6 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
     commit_chunk(ib, 2 * s + 6);
     cur = nxt;
     del_n = own_delta(cur);
-    own_scale(cur);
     __syncthreads();
   }
   {
@@ -342,18 +327,11 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
     swam_frag_issue(w.v, vb_, sn2v, w.tok, g);
   };
   auto own_pin = [&](const Own& w) { swam_frag_pin(w.k); swam_frag_pin(w.v); };
-  // The own keys are multiplied by -sm_scale log2(e) once per step and the own values negated; the first products start
-  // from the staged lse2 / delta of the lane's four queries (read from LDS straight into the C operand): the matrix pipe
-  // delivers -(s2 - lse2) and -(dP - delta), and p = exp2(-.), dS = -p (.) are the only vector instructions left per
-  // score besides the window mask (the signs are operand modifiers).
-  auto own_scale = [&](Own& w) {
+  // The own values are negated and the dP products start from the staged delta of the lane's four queries (read from LDS
+  // straight into the C operand): the matrix pipe delivers -(dP - delta), and dS = -p (.) (the sign is an operand modifier).
+  auto own_negate_v = [&](Own& w) {
 #pragma unroll
     for (int c = 0; c < 2; c++) {
-      float e[8];
-      unpack8<CT>(w.k.f[c], e);
-#pragma unroll
-      for (int j = 0; j < 8; j++) e[j] *= -scale;
-      w.k.f[c] = pack8<CT>(e);
       w.v.f[c].x ^= 0x80008000u; w.v.f[c].y ^= 0x80008000u; w.v.f[c].z ^= 0x80008000u; w.v.f[c].w ^= 0x80008000u;
     }
   };
@@ -385,7 +363,7 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
 #pragma unroll
     for (int i = 0; i < 3; i++) pin_loaded(sc[i]);
     own_pin(cur);
-    own_scale(cur);
+    own_negate_v(cur);
 #pragma unroll
     for (int i = 0; i < 3; i++)
       if (kpar + 2 * i < SWAM_NSLOT) scalar_commit(sc[i], kpar + 2 * i);
@@ -445,15 +423,15 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
         __builtin_amdgcn_sched_barrier(0);
         const u32x4(&qc)[2] = qa[hb & 1];
         const u32x4(&dc)[2] = da[hb & 1];
-        f32x4 sv, pv;
-        sv = Mma<CT>::mfma(qc[0], kf0, lq);
+        f32x4 sv = {0.f, 0.f, 0.f, 0.f}, pv;
+        sv = Mma<CT>::mfma(qc[0], kf0, sv);
         pv = Mma<CT>::mfma(dc[0], vf0, dq_);
         sv = Mma<CT>::mfma(qc[1], kf1, sv);
         pv = Mma<CT>::mfma(dc[1], vf1, pv);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const bool vis = row_vis & ((unsigned)(8 * kb + 4 * mb + i - clo) <= (unsigned)cspan);
-          pr[4 * mb + i] = fast_exp2(vis ? -sv[i] : -INFINITY);
+          pr[4 * mb + i] = fast_exp2(fmaf(sv[i], scale, vis ? -lq[i] : -INFINITY));
           ds[4 * mb + i] = -pr[4 * mb + i] * pv[i];
         }
       }
@@ -513,7 +491,7 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
     commit_chunk(ib, 2 * s + 6);
     scalar_commit(sc, 2 * s + 6 - kpar);
     cur = nxt;
-    own_scale(cur);
+    own_negate_v(cur);
     __syncthreads();
   }
   {

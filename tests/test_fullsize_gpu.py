@@ -168,9 +168,9 @@ def test_c3_full_batch_fused_rope_equals_composition(save_rotated, monkeypatch):
     if save_rotated:
         assert torch.equal(qg.grad, q2.grad) and torch.equal(kg.grad, k2.grad) and torch.equal(vg.grad, v2.grad)
     else:
-        # the backward pass that rotates in every tile load runs on the tile kernels, which scale the scores after the
-        # products; the marching kernels of the composition scale the own q / k fragments before them (one more
-        # rounding to bf16): equal within that rounding
+        # the backward pass that rotates in every tile load runs on the tile kernels, which subtract delta from the
+        # finished dP products; the marching kernels of the composition start those products from -delta (another fp32
+        # summation order): equal within that rounding
         rel = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
         assert max(rel(qg.grad, q2.grad), rel(kg.grad, k2.grad), rel(vg.grad, v2.grad)) <= 1e-2
     assert torch.isfinite(o.float()).all() and torch.isfinite(qg.grad.float()).all()

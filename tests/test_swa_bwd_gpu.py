@@ -151,8 +151,8 @@ def test_fused_rope_backward(d, R, save_rotated, monkeypatch):
         if save_rotated:
             assert torch.equal(q2.grad, qg.grad) and torch.equal(k2.grad, kg.grad) and torch.equal(v2.grad, vg.grad)
         else:
-            # the backward pass that rotates in every tile load runs on the tile kernels, which scale the scores after
-            # the products; the marching kernels scale the own q / k fragments before them (one more rounding to bf16)
+            # the backward pass that rotates in every tile load runs on the tile kernels, which subtract delta from the
+            # finished dP products; the marching kernels start those products from -delta (another fp32 summation order)
             assert torch.equal(v2.grad, vg.grad) or _rel(v2.grad, vg.grad.float().cpu()) <= 1e-2
             assert max(_rel(q2.grad, qg.grad.float().cpu()), _rel(k2.grad, kg.grad.float().cpu())) <= 1e-2
 
