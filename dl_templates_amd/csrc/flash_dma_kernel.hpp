@@ -342,14 +342,14 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     // lies below every own key, its body holds no test (as without a mask)
     for (; ci + AHEAD < W.nchunks && W.at(ci).x < x0 + OWN - 1; ci++) {
       consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
-      flashd_wait_copies<PER_CHUNK>();
+      flashd_wait_copies<(AHEAD - 1) * PER_CHUNK>();
       __syncthreads();
       bi = bi + 1 == NBUF ? 0 : bi + 1;
     }
   }
   for (; ci + AHEAD < W.nchunks; ci++) {
     consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
-    flashd_wait_copies<PER_CHUNK>();   // all but the copies just issued: chunk ci + 1 has landed
+    flashd_wait_copies<(AHEAD - 1) * PER_CHUNK>();   // chunk ci + 1 has landed: all copies but those of the AHEAD - 1 chunks behind it
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
@@ -553,7 +553,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
     const int nfull = dlt_imin(x0, W.len) / CK;
     for (; ci + AHEAD < W.nchunks && ci < nfull; ci++) {
       consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
-      flashd_wait_copies<PER_CHUNK>();
+      flashd_wait_copies<(AHEAD - 1) * PER_CHUNK>();
       __syncthreads();
       bi = bi + 1 == NBUF ? 0 : bi + 1;
     }
@@ -561,7 +561,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
   for (; ci + AHEAD < W.nchunks; ci++) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
     else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
-    flashd_wait_copies<PER_CHUNK>();
+    flashd_wait_copies<(AHEAD - 1) * PER_CHUNK>();
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
@@ -779,7 +779,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
     const int nfull = dlt_imin(x0, W.len) / CK;
     for (; ci + AHEAD < W.nchunks && ci < nfull; ci++) {
       consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
-      flashd_wait_copies<PER_CHUNK>();
+      flashd_wait_copies<(AHEAD - 1) * PER_CHUNK>();
       __syncthreads();
       bi = bi + 1 == NBUF ? 0 : bi + 1;
     }
@@ -787,7 +787,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
   for (; ci + AHEAD < W.nchunks; ci++) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::true_type{});
     else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::true_type{});
-    flashd_wait_copies<PER_CHUNK>();
+    flashd_wait_copies<(AHEAD - 1) * PER_CHUNK>();
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
