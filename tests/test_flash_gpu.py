@@ -199,6 +199,28 @@ def test_chunk_boundaries_of_the_async_staged_kernels(causal, dk, dv, dtype):
         assert max(errs) <= 5e-2, (Lq, Lk, errs)
 
 
+@pytest.mark.parametrize("causal,dk,dv", [(False, 64, 128), (False, 128, 128), (True, 128, 128), (True, 64, 64)])
+def test_async_staged_kernels_repeat_bit_for_bit(causal, dk, dv):
+    """The kernels are deterministic, so a chunk read before its asynchronous copy has landed (or overwritten while it is
+    still being read) shows as a difference between repeats: 25 forward + backward passes over many chunks (two chunk
+    buffers at 64/128 forward and at 128/128, three elsewhere) must all equal the first, bit for bit."""
+    B, H, L = 2, 8, 4096
+    q, k, v, do = (t.cuda() for t in orc.make_qkv(77, B, H, L, L, dk, dv, torch.bfloat16))
+    scale = 1 / math.sqrt(dk)
+    first = None
+    for _ in range(25):
+        qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+        o, M = _fa()._forward(qg.detach(), kg.detach(), vg.detach(), causal, scale)
+        o2 = _fa().attention(qg, kg, vg, causal, scale)
+        o2.backward(do)
+        got = (o, M, o2.detach(), qg.grad, kg.grad, vg.grad)
+        if first is None:
+            first = got
+        else:
+            for a, b in zip(first, got):
+                assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_views_of_a_packed_projection(causal):
     """q, k, v as strided views of one packed [B, L, H, dk + dk + dv] projection output (token stride H (2 dk + dv), head
