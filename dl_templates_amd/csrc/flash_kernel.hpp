@@ -103,6 +103,21 @@ struct FlashWalk {
     nchunks = (rh - rl + 1) * nxc;
     first = 0; len = 0;
   }
+  // the chunk after c (the loops walk the chunks in order: no division per chunk)
+  DLT_DEV FlashChunk next(const FlashChunk& c) const {
+    FlashChunk n;
+    n.x = c.x + CK;
+    n.row = c.row;
+    if (MODE >= 2) {
+      if (n.x >= X1) { n.x = X0; n.row = c.row + 1; }
+      n.tok0 = n.row * XL + n.x;
+      n.nvalid = dlt_imin(CK, X1 - n.x);
+    } else {
+      n.tok0 = n.x;
+      n.nvalid = dlt_imin(CK, len - n.x);
+    }
+    return n;
+  }
   DLT_DEV FlashChunk at(int i) const {
     FlashChunk c;
     if (MODE >= 2) {
@@ -316,16 +331,14 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   // `tail` (dense / causal): some keys of the chunk lie past the end or (causal) above the wave's first query, and every
   // pair is tested.  A compile-time tag: without a causal mask only the last chunk can be short, and the loop body then
   // holds no test at all.
-  auto chunk_tail = [&](const int ci) {
-    const FlashChunk c = W.at(ci);
+  auto chunk_tail = [&](const FlashChunk& c) {
     return !TILE && (c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0));
   };
-  auto consume_t = [&](const int ci, auto tail_tag) __attribute__((always_inline)) {
+  auto consume_t = [&](const FlashChunk& c, auto tail_tag) __attribute__((always_inline)) {
     // the tag is true_type / false_type (dense: known per call site) or FlashTailDyn (causal: tested per chunk)
     bool tail;
-    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(c);
     else tail = decltype(tail_tag)::value;
-    const FlashChunk c = W.at(ci);
     const int k0 = c.x;
     // causal: every key of the chunk lies above every query of this wave (wave-uniform)
     bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
@@ -439,20 +452,23 @@ __global__ __launch_bounds__(256, flash_occ_fwd(DK, DV)) void flash_fwd_kernel(c
   // The last chunk is peeled off so that prefetch and commit are unconditional inside the loop:
   // with `if (has_next)` around each, the compiler sees a path on which loads stay pending across
   // the back edge and guards every later load with a full vmcnt(0) wait.
-  auto consume = [&](const int ci) __attribute__((always_inline)) {
-    if (CAUSAL) consume_t(ci, FlashTailDyn{});
-    else if (chunk_tail(ci)) consume_t(ci, std::true_type{});
-    else consume_t(ci, std::false_type{});
+  auto consume = [&](const FlashChunk& c) __attribute__((always_inline)) {
+    if (CAUSAL) consume_t(c, FlashTailDyn{});
+    else if (chunk_tail(c)) consume_t(c, std::true_type{});
+    else consume_t(c, std::false_type{});
   };
+  FlashChunk cc = W.at(0);
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
-    issue(W.at(ci + 1));
-    if (CAUSAL) consume(ci);
-    else consume_t(ci, std::false_type{});
+    const FlashChunk cn = W.next(cc);
+    issue(cn);
+    if (CAUSAL) consume(cc);
+    else consume_t(cc, std::false_type{});
     __syncthreads();
     commit();
     __syncthreads();
+    cc = cn;
   }
-  if (W.nchunks > 0) consume(W.nchunks - 1);
+  if (W.nchunks > 0) consume(cc);
   __syncthreads();
 
   // ---- epilogue: normalise, O^T fragments -> LDS tile -> coalesced rows
@@ -664,16 +680,14 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
 
   // `tail`: some keys of the chunk lie past the end or (causal) above the wave's first query, and every pair is tested.
   // It is a compile-time tag: as a run-time flag the test was folded into a select per element of every chunk.
-  auto chunk_tail = [&](const int ci) {
-    const FlashChunk c = W.at(ci);
+  auto chunk_tail = [&](const FlashChunk& c) {
     return !TILE && (c.nvalid < CK || (CAUSAL && c.x + CK - 1 > wq0));
   };
-  auto consume_t = [&](const int ci, auto tail_tag) __attribute__((always_inline)) {
+  auto consume_t = [&](const FlashChunk& c, auto tail_tag) __attribute__((always_inline)) {
     // the tag is true_type / false_type (dense: known per call site) or FlashTailDyn (causal: tested per chunk)
     bool tail;
-    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(c);
     else tail = decltype(tail_tag)::value;
-    const FlashChunk c = W.at(ci);
     const int k0 = c.x;
     const bool live = !CAUSAL || k0 <= wq0 + 16 * NP - 1;
 #pragma unroll
@@ -731,22 +745,25 @@ __global__ __launch_bounds__(256, flash_occ_q(DK, DV)) void flash_bwd_q_kernel(c
       }
     }
   };
-  auto consume = [&](const int ci) __attribute__((always_inline)) {
-    if (CAUSAL) consume_t(ci, FlashTailDyn{});
-    else if (chunk_tail(ci)) consume_t(ci, std::true_type{});
-    else consume_t(ci, std::false_type{});
+  auto consume = [&](const FlashChunk& c) __attribute__((always_inline)) {
+    if (CAUSAL) consume_t(c, FlashTailDyn{});
+    else if (chunk_tail(c)) consume_t(c, std::true_type{});
+    else consume_t(c, std::false_type{});
   };
   // last chunk peeled off: unconditional prefetch and commit inside the loop (see the forward kernel); without a causal
   // mask only the last chunk can be short
+  FlashChunk cc = W.at(0);
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
-    st.issue(kb_, ak, vb_, av, W.at(ci + 1));
-    if (CAUSAL) consume(ci);
-    else consume_t(ci, std::false_type{});
+    const FlashChunk cn = W.next(cc);
+    st.issue(kb_, ak, vb_, av, cn);
+    if (CAUSAL) consume(cc);
+    else consume_t(cc, std::false_type{});
     __syncthreads();
     st.commit(sK, PK, sV, PV);
     __syncthreads();
+    cc = cn;
   }
-  if (W.nchunks > 0) consume(W.nchunks - 1);
+  if (W.nchunks > 0) consume(cc);
   __syncthreads();
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
   flash_write_grad<TIO, DK, NP>(smem, dq_acc, a.sm_scale, dqb, flash_tok<IMG>(a.dqs, a.tm), a.dqs[3], a.dk_, a.dq_vec != 0, own_base, x0, a.Lq, wave, n, g, tid);
@@ -849,16 +866,14 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
 
   // `tail`: some queries of the chunk lie past the end or (causal) below the wave's last own key (a compile-time tag, as
   // in the dQ kernel)
-  auto chunk_tail = [&](const int ci) {
-    const FlashChunk c = W.at(ci);
+  auto chunk_tail = [&](const FlashChunk& c) {
     return !TILE && (c.nvalid < CK || (CAUSAL && c.x < wk0 + 16 * NP - 1));
   };
-  auto consume_t = [&](const int ci, auto tail_tag) __attribute__((always_inline)) {
+  auto consume_t = [&](const FlashChunk& c, auto tail_tag) __attribute__((always_inline)) {
     // the tag is true_type / false_type (dense: known per call site) or FlashTailDyn (causal: tested per chunk)
     bool tail;
-    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(ci);
+    if constexpr (std::is_same<decltype(tail_tag), FlashTailDyn>::value) tail = chunk_tail(c);
     else tail = decltype(tail_tag)::value;
-    const FlashChunk c = W.at(ci);
     const int q0 = c.x;
     // causal: every query of the chunk lies below every own key of this wave
     const bool live = !CAUSAL || q0 + CK - 1 >= wk0;
@@ -928,25 +943,27 @@ __global__ __launch_bounds__(256, flash_occ_kv(DK, DV, MODE)) void flash_bwd_kv_
       }
     }
   };
-  auto consume = [&](const int ci) __attribute__((always_inline)) {
-    if (CAUSAL) consume_t(ci, FlashTailDyn{});
-    else if (chunk_tail(ci)) consume_t(ci, std::true_type{});
-    else consume_t(ci, std::false_type{});
+  auto consume = [&](const FlashChunk& c) __attribute__((always_inline)) {
+    if (CAUSAL) consume_t(c, FlashTailDyn{});
+    else if (chunk_tail(c)) consume_t(c, std::true_type{});
+    else consume_t(c, std::false_type{});
   };
+  FlashChunk cc = W.at(0);
   for (int ci = 0; ci + 1 < W.nchunks; ci++) {
-    const FlashChunk cn = W.at(ci + 1);
+    const FlashChunk cn = W.next(cc);
     st.issue(qb, aq, dob, ad, cn);
     issue_scalars(cn);
-    if (CAUSAL) consume(ci);
-    else consume_t(ci, std::false_type{});   // without a causal mask only the last chunk can be short
+    if (CAUSAL) consume(cc);
+    else consume_t(cc, std::false_type{});   // without a causal mask only the last chunk can be short
     __syncthreads();
     st.commit(sQ, PQ, sDO, PD);
     pin_loaded(r_lse);
     pin_loaded(r_del);
     if (tid < CK) { sLse[tid] = r_lse; sDel[tid] = r_del; }
     __syncthreads();
+    cc = cn;
   }
-  if (W.nchunks > 0) consume(W.nchunks - 1);
+  if (W.nchunks > 0) consume(cc);
   __syncthreads();
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
   TIO* dvb = reinterpret_cast<TIO*>(a.dv) + b * a.dvs[0] + h * a.dvs[1];
