@@ -1,5 +1,6 @@
-// Flash kernels with asynchronous staging: the variants of flash_kernel.hpp for head dims that are exactly 64 or
-// 128 (no padded dims: a copy cannot zero-fill).  Streamed chunks travel HBM -> LDS by the DMA path of the vector
+// Flash kernels with asynchronous staging: the variants of flash_kernel.hpp for the classes of head dim 64 and 128
+// (head dims below the class in multiples of 8: template flag PAD, the copies skip the missing 16-byte pieces, whose
+// LDS slots are zeroed once).  Streamed chunks travel HBM -> LDS by the DMA path of the vector
 // memory unit (16 bytes per lane, no staging registers, no LDS write instructions) into a ring of two or three chunk
 // buffers while an earlier chunk is consumed: one workgroup barrier per chunk instead of two.  LDS rows are 2 D bytes without
 // padding; the 16-byte piece c of token t is stored at piece c ^ (m (t & 7)), m = D / 64, which keeps the operand
@@ -64,25 +65,42 @@ struct FlashDStage {
   typedef FlashDRow<D> R;
   static constexpr int NI = CK / NW / R::TPI;
   static_assert(NI >= 1 && NI * R::TPI * NW == CK, "chunk must split evenly over the waves' copy instructions");
-  int tok0;   // token of the lane in instruction 0
-  int lp;     // physical piece the lane writes
+  int tok0;      // token of the lane in instruction 0
+  int lp;        // physical piece the lane writes
+  int npieces;   // 16-byte pieces a row of the tensor really has (head dim / 8 <= PIECES)
 
-  DLT_DEV void init(int wave, int lane) {
+  DLT_DEV void init(int wave, int lane, int dact) {
     tok0 = wave * (CK / NW) + lane / R::PIECES;
     lp = lane % R::PIECES;
+    npieces = dact >> 3;
   }
-  // tokens past the end of the chunk are clamped onto its last token (the caller masks them)
-  template <typename AD>
+  // tokens past the end of the chunk are clamped onto its last token (the caller masks them).  With a head dim below
+  // the padded one the lanes of the missing pieces copy nothing: their LDS slots were zeroed once (flashd_zero_pads) and
+  // no copy ever writes them (PAD: a compile-time flag of the kernels, the test costs the exact-dim kernels 1.5 %).  Every
+  // instruction still has active lanes, so the count of copies in flight is the same.
+  template <bool PAD, typename AD>
   DLT_DEV void issue(const char* base, const AD& ad, const FlashChunk& c, char* region, int wave) const {
 #pragma unroll
     for (int i = 0; i < NI; i++) {
       const int t = tok0 + R::TPI * i;
-      const uint32_t off = ad(c, dlt_imin(t, c.nvalid - 1)) + 16u * (uint32_t)(lp ^ (R::SWZ * (t & 7)));
+      const int lgp = lp ^ (R::SWZ * (t & 7));
+      const uint32_t off = ad(c, dlt_imin(t, c.nvalid - 1)) + 16u * (uint32_t)lgp;
       char* dst = region + (wave * (CK / NW) + R::TPI * i) * R::ROW;   // wave-uniform
-      dlt_copy16_to_lds(base, off, dst);
+      if (!PAD || lgp < npieces) dlt_copy16_to_lds(base, off, dst);
     }
   }
 };
+
+// zeroes the 16-byte slots of a swizzled [ntok][D] region that hold head dims at or beyond 8 * npieces
+template <int D>
+DLT_DEV void flashd_zero_pads(char* region, int ntok, int npieces, int tid, int nthreads) {
+  typedef FlashDRow<D> R;
+  if (npieces == R::PIECES) return;
+  for (int s = tid; s < ntok * R::PIECES; s += nthreads) {
+    const int t = s / R::PIECES, pp = s % R::PIECES;
+    if ((pp ^ (R::SWZ * (t & 7))) >= npieces) *reinterpret_cast<u32x4*>(region + s * 16) = u32x4{0u, 0u, 0u, 0u};
+  }
+}
 
 // per-token fp32 scalars of a chunk: 64 tokens per instruction, 4 bytes per lane (32-bit byte offsets inside a
 // (batch, head) slab: checked by the host)
@@ -133,7 +151,7 @@ struct FlashDBuf {
 };
 
 // ---- dK / dV: own = keys; Q, dO, lse2 and delta stream.  Replaces _attn_bwd_dkdv (src/flash_attn.py:204-307).
-template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE>
+template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE, bool PAD>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef FlashDBuf<DK, DV, CK> B;
@@ -167,17 +185,23 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 
   FlashDStage<DK, CK, NW> stq;
   FlashDStage<DV, CK, NW> std_;
-  stq.init(wave, lane);
-  std_.init(wave, lane);
+  stq.init(wave, lane, a.dk_);
+  std_.init(wave, lane, a.dv_);
   // waves 0 and 1 also copy the chunk's lse2 / delta
   const float* scal_base = wave == 0 ? lseb : delb;
   auto issue = [&](const FlashChunk& c, char* buf) {
-    stq.issue(qb, aq, c, buf, wave);
-    std_.issue(dob, ad, c, buf + B::REG_A, wave);
+    stq.template issue<PAD>(qb, aq, c, buf, wave);
+    std_.template issue<PAD>(dob, ad, c, buf + B::REG_A, wave);
     if (wave < 2) flashd_issue_scalars<CK>(scal_base, (int)a.ls[2], c, buf + B::REG_A + B::REG_B + wave * (CK * 4), lane);
   };
   constexpr int NBUF = NW == 4 ? flashd_nbuf(DK, DV) : FLASHD_NBUF8, AHEAD = NBUF - 1;
   constexpr int PER_CHUNK = FlashDStage<DK, CK, NW>::NI + FlashDStage<DV, CK, NW>::NI;   // copies per wave and chunk (waves 0, 1: more)
+  // head dims below the padded ones: the slots of the missing pieces are zeroed once, no copy writes them
+#pragma unroll
+  for (int i = 0; PAD && i < NBUF; i++) {
+    flashd_zero_pads<DK>(smem + i * B::BUF_KV, CK, a.dk_ >> 3, tid, 64 * NW);
+    flashd_zero_pads<DV>(smem + i * B::BUF_KV + B::REG_A, CK, a.dv_ >> 3, tid, 64 * NW);
+  }
 #pragma unroll
   for (int i = 0; i < AHEAD; i++)
     if (i < W.nchunks) issue(W.at(i), smem + i * B::BUF_KV);
@@ -376,7 +400,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
 // Per chunk: S^T = K Q^T for every 32-key block (a stream of NKB 2 KC operand reads, NP products each), one softmax
 // update per query block, then O^T += V^T P^T (NKB VB transposed operands) with the row sums from a ones-row product.
 // The reads of the second stream are already in flight while the softmax runs.
-template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE>
+template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE, bool PAD>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(const FlashArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef typename TileOf<TIO>::type TL;
@@ -412,11 +436,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
 
   FlashDStage<DK, CK, NW> stk;
   FlashDStage<DV, CK, NW> stv;
-  stk.init(wave, lane);
-  stv.init(wave, lane);
+  stk.init(wave, lane, a.dk);
+  stv.init(wave, lane, a.dv);
+  // head dims below the padded ones: the slots of the missing pieces are zeroed once, no copy writes them
+#pragma unroll
+  for (int i = 0; PAD && i < NBUF; i++) {
+    flashd_zero_pads<DK>(smem + i * B::BUF, CK, a.dk >> 3, tid, 64 * NW);
+    flashd_zero_pads<DV>(smem + i * B::BUF + B::REG_A, CK, a.dv >> 3, tid, 64 * NW);
+  }
   auto issue = [&](const FlashChunk& c, char* buf) {
-    stk.issue(kb_, ak, c, buf, wave);
-    stv.issue(vb_, av, c, buf + B::REG_A, wave);
+    stk.template issue<PAD>(kb_, ak, c, buf, wave);
+    stv.template issue<PAD>(vb_, av, c, buf + B::REG_A, wave);
   };
 #pragma unroll
   for (int i = 0; i < AHEAD; i++)
@@ -602,7 +632,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
 // ---- dQ: own = queries; K and V stream.  Replaces _attn_bwd_dq (src/flash_attn.py:310-449) and, with fuse_delta, the
 // delta pre-pass (:186-202).  Per 32-key block: per 16-key half KC pieces of K (S = K Q^T) and VC pieces of V
 // (dP = V dO^T), then KB transposed pieces of K (dQ^T += K^T dS).
-template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE>
+template <typename TIO, int DK, int DV, int NP, int CK, int NW, int MODE, bool PAD>
 __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(const FlashBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef FlashDBuf<DK, DV, CK> B;
@@ -636,11 +666,17 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
 
   FlashDStage<DK, CK, NW> stk;
   FlashDStage<DV, CK, NW> stv;
-  stk.init(wave, lane);
-  stv.init(wave, lane);
+  stk.init(wave, lane, a.dk_);
+  stv.init(wave, lane, a.dv_);
+  // head dims below the padded ones: the slots of the missing pieces are zeroed once, no copy writes them
+#pragma unroll
+  for (int i = 0; PAD && i < NBUF; i++) {
+    flashd_zero_pads<DK>(smem + i * B::BUF, CK, a.dk_ >> 3, tid, 64 * NW);
+    flashd_zero_pads<DV>(smem + i * B::BUF + B::REG_A, CK, a.dv_ >> 3, tid, 64 * NW);
+  }
   auto issue = [&](const FlashChunk& c, char* buf) {
-    stk.issue(kb_, ak, c, buf, wave);
-    stv.issue(vb_, av, c, buf + B::REG_A, wave);
+    stk.template issue<PAD>(kb_, ak, c, buf, wave);
+    stv.template issue<PAD>(vb_, av, c, buf + B::REG_A, wave);
   };
 #pragma unroll
   for (int i = 0; i < AHEAD; i++)

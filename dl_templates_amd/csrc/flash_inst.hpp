@@ -41,12 +41,14 @@ int flash_set_lds(KernT kern, int bytes) { return dlt_ensure_lds(reinterpret_cas
 template <typename TIO, int MODE>
 int flash_launch_fwd_c(const FlashArgs& a, int grid, hipStream_t stream) {
   if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
-    // dense / causal with exact head dims of 64 / 128: chunks are copied HBM -> LDS asynchronously (a copy cannot
-    // zero-fill padded dims).  Measured per class and mode against the register-staged kernel: dense -2 % (64/64), -4 %
-    // (64/128), -7 % (128/128); causal -4 % (64/64), -18 % (128/128).
-    if (a.dk == DLT_DK && a.dv == DLT_DV && flash_async_staging()) {
+    // dense / causal, head dims that are multiples of 8: chunks are copied HBM -> LDS asynchronously.  Measured per
+    // class and mode against the register-staged kernel: dense -2 % (64/64), -4 % (64/128), -7 % (128/128); causal -4 %
+    // (64/64), -18 % (128/128); head dims below the class (80/80, 96/96): -18 % on the step.
+    if (a.dk % 8 == 0 && a.dv % 8 == 0 && flash_async_staging()) {
       constexpr int NP = FLASHD_FWD_NP, CK = FLASHD_FWD_CK(DLT_DK, DLT_DV), NW = FLASHD_FWD_NW(DLT_DK, DLT_DV);
-      auto kern = flashd_fwd_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
+      // head dims below the padded ones (multiples of 8): the kernel variant whose copies skip the missing pieces
+      auto kern = (a.dk != DLT_DK || a.dv != DLT_DV) ? flashd_fwd_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE, true>
+                                                     : flashd_fwd_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE, false>;
       constexpr int own = 16 * NP * NW;
       constexpr int tile = own * (DLT_DV * 2 + 16);
       constexpr int bufs = (NW == 4 ? flashd_nbuf(DLT_DK, DLT_DV) : 2) * FlashDBuf<DLT_DK, DLT_DV, CK>::BUF;
@@ -85,9 +87,10 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
   // dQ first: with fuse_delta it produces the delta vector the dK/dV kernel consumes
   bool dq_done = false;
   if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
-    if (a.dk_ == DLT_DK && a.dv_ == DLT_DV && flash_async_staging()) {
+    if (a.dk_ % 8 == 0 && a.dv_ % 8 == 0 && flash_async_staging()) {
       constexpr int NP = FLASHD_DQ_NP(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
-      auto kern = flashd_bwd_q_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
+      auto kern = (a.dk_ != DLT_DK || a.dv_ != DLT_DV) ? flashd_bwd_q_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE, true>
+                                                       : flashd_bwd_q_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE, false>;
       constexpr int own = 16 * NP * NW;
       constexpr int tile = own * (DLT_DK * 2 + 16);
       constexpr int bufs = (NW == 4 ? flashd_nbuf(DLT_DK, DLT_DV) : FLASHD_NBUF8) * FlashDBuf<DLT_DK, DLT_DV, CK>::BUF;
@@ -113,12 +116,13 @@ int flash_launch_bwd_c(const FlashBwdArgs& a, int grid_kv, int grid_q, hipStream
     DLT_CHECK_LAUNCH("flash dQ launch");
   }
   if constexpr (DLT_DK >= 64 && DLT_DV >= 64 && MODE < 2) {
-    // dense / causal with exact head dims: chunks are copied HBM -> LDS asynchronously (a copy cannot zero-fill padded
-    // dims; in tile mode, where whole blocks are skipped, the register-staged kernel measured 1.5 % faster)
+    // dense / causal, head dims that are multiples of 8: chunks are copied HBM -> LDS asynchronously (in tile mode,
+    // where whole blocks are skipped, the register-staged kernel measured 1.5 % faster)
     const bool scalars_fit = a.ls[2] >= 0 && ((int64_t)a.Lq - 1) * a.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1);   // 32-bit offsets of the lse2 / delta copies
-    if (a.dk_ == DLT_DK && a.dv_ == DLT_DV && scalars_fit && flash_async_staging()) {
+    if (a.dk_ % 8 == 0 && a.dv_ % 8 == 0 && scalars_fit && flash_async_staging()) {
       constexpr int NP = flash_np_kv(DLT_DK, DLT_DV), CK = 64, NW = FLASHD_BWD_NW;
-      auto kern = flashd_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE>;
+      auto kern = (a.dk_ != DLT_DK || a.dv_ != DLT_DV) ? flashd_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE, true>
+                                                       : flashd_bwd_kv_kernel<TIO, DLT_DK, DLT_DV, NP, CK, NW, MODE, false>;
       constexpr int own = 16 * NP * NW;
       constexpr int tile_k = own * (DLT_DK * 2 + 16), tile_v = own * (DLT_DV * 2 + 16);
       constexpr int bufs = (NW == 4 ? flashd_nbuf(DLT_DK, DLT_DV) : FLASHD_NBUF8) * FlashDBuf<DLT_DK, DLT_DV, CK>::BUF_KV;

@@ -199,6 +199,27 @@ def test_chunk_boundaries_of_the_async_staged_kernels(causal, dk, dv, dtype):
         assert max(errs) <= 5e-2, (Lq, Lk, errs)
 
 
+@pytest.mark.parametrize("causal,dk,dv,dtype", [
+    (False, 40, 40, torch.bfloat16), (True, 48, 80, torch.float16), (False, 80, 80, torch.bfloat16), (True, 96, 96, torch.bfloat16),
+    (False, 72, 120, torch.float16), (False, 56, 128, torch.bfloat16), (True, 128, 104, torch.bfloat16), (False, 64, 8, torch.float16)])
+def test_async_staged_kernels_with_head_dims_below_the_padded_class(causal, dk, dv, dtype):
+    """Head dims that are multiples of 8 below their class (64 or 128) also run on the asynchronously staged kernels: the
+    lanes of the missing 16-byte pieces copy nothing and their LDS slots are zeroed once.  Lengths of one to several
+    chunks, one token more and less."""
+    scale = 1 / math.sqrt(dk)
+    for Lq, Lk in [(1, 1), (65, 64), (130, 191), (257, 320), (300, 129), (512, 513)]:
+        if causal:
+            Lq = Lk
+        q, k, v, do = orc.make_qkv(Lq + 3 * Lk + dk + dv, 2, 2, Lq, Lk, dk, dv, dtype)
+        o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), causal, scale)
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        o = _fa().attention(qg, kg, vg, causal, scale)
+        o.backward(do.cuda())
+        assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2, (Lq, Lk)
+        errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+        assert max(errs) <= 5e-2, (Lq, Lk, errs)
+
+
 @pytest.mark.parametrize("causal,dk,dv", [(False, 64, 128), (False, 128, 128), (True, 128, 128), (True, 64, 64)])
 def test_async_staged_kernels_repeat_bit_for_bit(causal, dk, dv):
     """The kernels are deterministic, so a chunk read before its asynchronous copy has landed (or overwritten while it is
