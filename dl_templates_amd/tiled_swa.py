@@ -33,6 +33,32 @@ def _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale) -> 
                          _lib.dtype_code(q))
 
 
+def _pad_plan(q, v, b_size):
+    """Head dims (dk, dv) to pad q / k and v to before the launch, or None.
+
+    The tuned token-grid kernels (``b_size == 1``) take head dims that are multiples of 32 with both in one class (both
+    <= 64, or both in 65..128); anything else runs on the generic kernels, 6 to 9 times slower (measured at d = 40, 48,
+    80 against 64, 96, 128).  Zero columns appended to q, k, v (and to dO in the backward pass) change no score and no
+    output column, so such calls are padded to the next tuned shape here and the results sliced back: four to eight
+    extra copy passes over the tensors, a few percent of the step.  Tile mode (``b_size > 1``) needs none of this: its
+    kernels pad inside.
+    """
+    dk, dv = q.shape[-1], v.shape[-1]
+    if b_size != 1 or q.dtype not in (torch.bfloat16, torch.float16) or max(dk, dv) > 128:
+        return None
+    up = lambda d: (d + 31) // 32 * 32
+    tk, tv = (up(dk), up(dv)) if max(dk, dv) <= 64 else (max(96, up(dk)), max(96, up(dv)))
+    return None if (tk, tv) == (dk, dv) else (tk, tv)
+
+
+def _pad_last(x, d):
+    return x if x.shape[-1] == d else torch.nn.functional.pad(x, (0, d - x.shape[-1]))
+
+
+def _cut_last(x, d):
+    return x if x.shape[-1] == d else x[..., :d].contiguous()
+
+
 def _forward(q, k, v, shape, rope):
     _lib.require_cuda(q, k, v)
     lib = _lib.load()
@@ -68,17 +94,25 @@ def _backward(q, k, v, o, lse, do, shape, rope):
 
 def tiled_swa_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_size: int, t_height: int, t_width: int,
                   row_size: int, col_size: int, sm_scale: float = 1.0):
+    dv, plan = v.shape[-1], _pad_plan(q, v, b_size)
+    if plan is not None:
+        q, k, v = _pad_last(q, plan[0]), _pad_last(k, plan[0]), _pad_last(v, plan[1])
     shape = _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)
-    return _forward(q, k, v, shape, None)[0]
+    return _cut_last(_forward(q, k, v, shape, None)[0], dv)
 
 
 class TiledSwa(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, b_size: int, t_height: int, t_width: int,
                 row_size: int, col_size: int, sm_scale: float):
+        ctx.dims = (q.shape[-1], v.shape[-1])
+        plan = _pad_plan(q, v, b_size)
+        if plan is not None:   # head dims outside the tuned token-grid shapes: see _pad_plan
+            q, k, v = _pad_last(q, plan[0]), _pad_last(k, plan[0]), _pad_last(v, plan[1])
         shape = _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)
         o, m = _forward(q, k, v, shape, None)
         ctx.save_for_backward(q, k, v, m, o)
+        o = _cut_last(o, ctx.dims[1])
         ctx.b_size = b_size
         ctx.t_height = t_height
         ctx.t_width = t_width
@@ -91,7 +125,8 @@ class TiledSwa(torch.autograd.Function):
     def backward(ctx, do: torch.Tensor):
         q, k, v, m, o = ctx.saved_tensors
         shape = _shape(q, k, v, ctx.b_size, ctx.t_height, ctx.t_width, ctx.row_size, ctx.col_size, ctx.sm_scale)
-        dq, dk, dv = _backward(q, k, v, o, m, do, shape, None)
+        dq, dk, dv = _backward(q, k, v, o, m, _pad_last(do, v.shape[-1]), shape, None)
+        dq, dk, dv = _cut_last(dq, ctx.dims[0]), _cut_last(dk, ctx.dims[0]), _cut_last(dv, ctx.dims[1])
         return dq, dk, dv, None, None, None, None, None, None,
 
 
@@ -143,6 +178,10 @@ class TiledSwaRope(torch.autograd.Function):
     @staticmethod
     def forward(ctx, q, k, v, idx, row_cs_buffer, col_cs_buffer, b_size, t_height, t_width, row_size, col_size,
                 sm_scale):
+        ctx.dims = (q.shape[-1], v.shape[-1])
+        plan = _pad_plan(q, v, b_size)
+        if plan is not None:   # zero columns behind the rotated ones: see _pad_plan
+            q, k, v = _pad_last(q, plan[0]), _pad_last(k, plan[0]), _pad_last(v, plan[1])
         shape = _shape(q, k, v, b_size, t_height, t_width, row_size, col_size, sm_scale)
         assert row_cs_buffer.shape[1] == col_cs_buffer.shape[1]
         assert idx.shape[0] == q.shape[2]
@@ -155,17 +194,19 @@ class TiledSwaRope(torch.autograd.Function):
             o, m = _forward(q, k, v, shape, rope)
             ctx.save_for_backward(q, k, v, m, o, idx, row_cs_buffer, col_cs_buffer)
         ctx.scalars = (b_size, t_height, t_width, row_size, col_size, sm_scale)
-        return o
+        return _cut_last(o, ctx.dims[1])
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, m, o, idx, row_cs_buffer, col_cs_buffer = ctx.saved_tensors
         shape = _shape(q, k, v, *ctx.scalars)
         rope = (idx, row_cs_buffer, col_cs_buffer)
+        do = _pad_last(do, v.shape[-1])
         if ctx.rotated:
             dq, dk, dv = _backward_rot(q, k, v, o, m, do, shape, rope)
         else:
             dq, dk, dv = _backward(q, k, v, o, m, do, shape, rope)
+        dq, dk, dv = _cut_last(dq, ctx.dims[0]), _cut_last(dk, ctx.dims[0]), _cut_last(dv, ctx.dims[1])
         return (dq, dk, dv) + (None,) * 9
 
 

@@ -69,7 +69,7 @@ def test_tiles_with_several_tokens(b_size, th, tw, wr, wc):
     _run(4, 1, 2, b_size, th, tw, wr, wc, 32, 32, torch.bfloat16, scale=0.25)
 
 
-@pytest.mark.parametrize("dk,dv", [(64, 64), (128, 128), (64, 128), (16, 32), (40, 24), (128, 64)])
+@pytest.mark.parametrize("dk,dv", [(64, 64), (128, 128), (64, 128), (16, 32), (40, 24), (128, 64), (80, 80), (72, 120), (48, 96), (8, 56)])
 def test_head_dims(dk, dv):
     _run(5, 1, 2, 1, 12, 12, 3, 3, dk, dv, torch.bfloat16)
 
@@ -248,7 +248,8 @@ def test_rotated_side_outputs_with_awkward_strides():
 
 @pytest.mark.parametrize("d,dv,R,th,tw,W,save", [(32, 32, 8, 12, 20, 3, True), (32, 32, 8, 12, 20, 3, False), (32, 64, 8, 9, 9, 2, True),
                                                   (96, 96, 8, 10, 12, 3, True), (96, 128, 16, 10, 12, 3, False),
-                                                  (64, 32, 16, 8, 8, 2, True), (128, 64, 8, 8, 12, 4, True)])
+                                                  (64, 32, 16, 8, 8, 2, True), (128, 64, 8, 8, 12, 4, True),
+                                                  (80, 80, 8, 10, 12, 3, True), (72, 40, 8, 9, 11, 2, False), (48, 48, 8, 8, 8, 2, True)])
 def test_fused_rope_with_head_dims_below_the_padded_class(d, dv, R, th, tw, W, save, monkeypatch):
     """dk / dv that do not fill their padded class (32 in the 64 class, 96 in the 128 class) and dk != dv, with the
     rotation fused: staged pieces beyond the head dim stay zero, side outputs and gradients stop at the head dim."""

@@ -42,7 +42,14 @@ def _run(seed, B, H, b_size, th, tw, wr, wc, dk, dv, dtype, scale=None):
     assert lse.dtype == torch.float32 and lse.shape == lse_w.shape
     lerr = (lse.cpu() - lse_w).abs().max().item()
     assert lerr <= LSE_TOL, f"lse2 max abs err {lerr}"
-    assert torch.equal(sw.tiled_swa_fwd(qg, kg, vg, b_size, th, tw, wr, wc, scale), got)
+    pub = sw.tiled_swa_fwd(qg, kg, vg, b_size, th, tw, wr, wc, scale)
+    if sw._pad_plan(qg, vg, b_size) is None:
+        assert torch.equal(pub, got)
+    else:
+        # head dims outside the tuned token-grid shapes: the public entry pads them and runs the tuned kernels, the bare
+        # launch above ran the generic ones; both are held to the oracle
+        assert pub.shape == got.shape and pub.is_contiguous()
+        assert (pub.float().cpu() - want).abs().max().item() <= FWD_TOL
     return err
 
 
@@ -78,7 +85,7 @@ def test_tiles_with_several_tokens(b_size, th, tw, wr, wc):
     _run(3, 1, 2, b_size, th, tw, wr, wc, 32, 32, torch.bfloat16, scale=0.25)
 
 
-@pytest.mark.parametrize("dk,dv", [(64, 64), (128, 128), (64, 128), (16, 32), (40, 24), (128, 64)])
+@pytest.mark.parametrize("dk,dv", [(64, 64), (128, 128), (64, 128), (16, 32), (40, 24), (128, 64), (80, 80), (72, 120), (48, 96), (8, 56)])
 def test_head_dims(dk, dv):
     _run(4, 1, 2, 1, 12, 12, 3, 3, dk, dv, torch.bfloat16)
 
