@@ -220,6 +220,27 @@ def test_async_staged_kernels_with_head_dims_below_the_padded_class(causal, dk, 
         assert max(errs) <= 5e-2, (Lq, Lk, errs)
 
 
+@pytest.mark.parametrize("causal,dk,dv,dtype", [(False, 100, 100, torch.bfloat16), (True, 50, 36, torch.float16), (False, 20, 127, torch.bfloat16),
+                                                 (True, 1, 3, torch.float16), (False, 65, 9, torch.bfloat16)])
+def test_head_dims_that_are_not_multiples_of_eight(causal, dk, dv, dtype):
+    """The public entry pads such head dims with zero columns to the next multiple of 8 (the kernels read 16-byte row
+    pieces) and slices the results: shapes, contiguity and values against the oracle."""
+    scale = 1 / math.sqrt(dk)
+    for Lq, Lk in [(1, 1), (130, 191), (300, 129)]:
+        if causal:
+            Lq = Lk
+        q, k, v, do = orc.make_qkv(Lq + Lk + dk + dv, 1, 3, Lq, Lk, dk, dv, dtype)
+        o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), causal, scale)
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        o = _fa().attention(qg, kg, vg, causal, scale)
+        o.backward(do.cuda())
+        assert o.shape == o_w.shape and o.is_contiguous()
+        assert qg.grad.shape == q.shape and kg.grad.shape == k.shape and vg.grad.shape == v.shape
+        assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2, (Lq, Lk)
+        errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+        assert max(errs) <= 5e-2, (Lq, Lk, errs)
+
+
 @pytest.mark.parametrize("causal,dk,dv", [(False, 64, 128), (False, 128, 128), (True, 128, 128), (True, 64, 64)])
 def test_async_staged_kernels_repeat_bit_for_bit(causal, dk, dv):
     """The kernels are deterministic, so a chunk read before its asynchronous copy has landed (or overwritten while it is
