@@ -133,3 +133,100 @@ def test_random_image_layout_cases():
         if pad:
             g_all = buf.grad if packed else leaves[0].grad
             assert g_all[:, :, IW:].abs().max().item() == 0.0, tag
+
+
+def _other_strides(t, mode):
+    """The same values behind other strides: 0 contiguous, 1 a slice of a wider last dim, 2 stored as [B, N, H, D]."""
+    t = t.cuda()
+    if mode == 1:
+        w = torch.zeros(*t.shape[:-1], t.shape[-1] + 8, dtype=t.dtype, device=t.device)
+        w[..., :t.shape[-1]] = t
+        return w[..., :t.shape[-1]]
+    if mode == 2:
+        return t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    return t
+
+
+def _make(seed, B, H, Lq, Lk, dk, dv, dt):
+    q, k, v, do = orc.make_qkv(seed, B, H, Lq, Lk, dk, dv, dt)
+    if dt == torch.float32:   # the kernels round fp32 operands to bf16 on load: compare on values that survive it
+        q, k, v, do = (t.bfloat16().float() for t in (q, k, v, do))
+    return q, k, v, do
+
+
+def test_random_head_dims_strides_and_scales_sliding_window():
+    """Head dims outside the tuned shapes (the entry points zero-pad them), mixed pairs, windows up to 25 columns
+    (beyond 21 the generic kernels run), strided inputs, scales other than 1 / sqrt(d), both ways of keeping q, k
+    for the backward pass of the fused rotation."""
+    from dl_templates_amd import tiled_swa as sw
+    rng = random.Random(5)
+    dims = [8, 16, 24, 32, 40, 48, 56, 64, 72, 80, 96, 104, 120, 128]
+    done = 0
+    while done < N_CASES:
+        S = rng.choice([1, 1, 1, 16])
+        th, tw = rng.randint(1, 20 if S == 1 else 5), rng.randint(1, 36 if S == 1 else 6)
+        WR, WC = rng.randint(0, 12 if S == 1 else 2), rng.randint(0, 12 if S == 1 else 2)
+        d = rng.choice(dims)
+        dv = d if rng.random() < 0.5 else rng.choice(dims)
+        dt = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+        B, H = rng.randint(1, 2), rng.randint(1, 2)
+        use_rope = S == 1 and rng.random() < 0.4 and d >= 32
+        R = rng.choice([r for r in (4, 8, 16, 32) if 4 * r <= d]) if use_rope else 8
+        N = th * tw * S
+        if N > 3000:
+            continue
+        done += 1
+        scale = rng.choice([1 / math.sqrt(d), 0.3, 0.05])
+        keep = rng.random() < 0.5
+        mode = rng.choice([0, 0, 1, 2])
+        tag = (f"case {done}: S={S} grid={th}x{tw} W=({WR},{WC}) d={d}/{dv} B={B} H={H} {dt} rope={use_rope} R={R} "
+               f"keep={keep} strides={mode} scale={scale:.3f}")
+        print(tag, flush=True)
+        q, k, v, do = _make(done * 13 + 2, B, H, N, N, d, dv, dt)
+        qg, kg, vg = (_other_strides(t, mode).detach().requires_grad_(True) for t in (q, k, v))
+        if use_rope:
+            idx = orc.make_rope_idx(done, th, tw, 0.1)
+            rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+            o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, WR, WC, scale)
+            old = sw.TiledSwaRope.save_rotated
+            sw.TiledSwaRope.save_rotated = keep
+            try:
+                o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, WR, WC, scale)
+                o.backward(do.to(dt).cuda())
+            finally:
+                sw.TiledSwaRope.save_rotated = old
+        else:
+            o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), S, th, tw, WR, WC, scale)
+            o = sw.TiledSwa.apply(qg, kg, vg, S, th, tw, WR, WC, scale)
+            o.backward(do.to(dt).cuda())
+        assert o.shape == (B, H, N, dv) and o.dtype == dt, tag
+        assert qg.grad.shape == q.shape and kg.grad.shape == k.shape and vg.grad.shape == v.shape, tag
+        _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
+
+
+def test_random_head_dims_strides_and_scales_flash():
+    """Head dims that are not multiples of 8 (zero-padded by the entry point), above 128 (generic kernels), mixed
+    pairs, strided inputs, scales other than 1 / sqrt(d)."""
+    from dl_templates_amd import flash_attn as fa
+    rng = random.Random(6)
+    dims = [8, 16, 20, 24, 36, 40, 50, 64, 72, 80, 96, 100, 120, 128, 136, 200, 256]
+    for it in range(N_CASES):
+        causal = rng.random() < 0.5
+        Lq = rng.choice([1, 15, 64, 65, 127, 128, 129, 200, 511, 700])
+        Lk = Lq if causal else rng.choice([1, 31, 64, 100, 257, 640, 900])
+        dk = rng.choice(dims)
+        dv = dk if rng.random() < 0.4 else rng.choice(dims)
+        dt = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+        B, H = rng.randint(1, 2), rng.randint(1, 3)
+        scale = rng.choice([1 / math.sqrt(dk), 0.3, 0.05])
+        mode = rng.choice([0, 0, 1, 2])
+        tag = f"case {it}: causal={causal} L=({Lq},{Lk}) d={dk}/{dv} B={B} H={H} {dt} strides={mode} scale={scale:.3f}"
+        print(tag, flush=True)
+        q, k, v, do = _make(it * 5 + 9, B, H, Lq, Lk, dk, dv, dt)
+        o_w, dq_w, dk_w, dv_w = orc.flash_grads(q.float(), k.float(), v.float(), do.float(), causal, scale)
+        qg, kg, vg = (_other_strides(t, mode).detach().requires_grad_(True) for t in (q, k, v))
+        o = fa.attention(qg, kg, vg, causal, scale)
+        o.backward(do.to(dt).cuda())
+        assert o.shape == (B, H, Lq, dv) and o.dtype == dt, tag
+        assert qg.grad.shape == q.shape and kg.grad.shape == k.shape and vg.grad.shape == v.shape, tag
+        _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
