@@ -49,8 +49,11 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
       const TIO* po = reinterpret_cast<const TIO*>(a.o) + b * a.os[0] + h * a.os[1] + tok_addr(a.os, a.p.tm)(nn) + (int64_t)8 * c * a.os[3];
       const TIO* pd = reinterpret_cast<const TIO*>(a.d_o) + b * a.dos[0] + h * a.dos[1] + tok_addr(a.dos, a.p.tm)(nn) + (int64_t)8 * c * a.dos[3];
       if (sizeof(TIO) == 4) {
+        // dO rounded as the products of the main kernel see it (o is what the forward pass stored): delta then equals
+        // sum_k P dP of those products, and gradients that cancel (a query that sees one key) cancel here too
 #pragma unroll
-        for (int j = 0; j < 8; j++) if (j < nvalid) part += (float)po[j * a.os[3]] * (float)pd[j * a.dos[3]];
+        for (int j = 0; j < 8; j++)
+          if (j < nvalid) part += (float)po[j * a.os[3]] * unpack_lo<CT>(pack2<CT>((float)pd[j * a.dos[3]], 0.f));
       } else {
         float fo[8], fd[8];
         unpack8<CT>(Io<TIO, CT>::load8(po, a.o_vec != 0, a.os[3], nvalid), fo);

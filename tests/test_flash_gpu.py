@@ -312,3 +312,17 @@ def test_register_staged_kernels_behind_the_environment_switch():
                        cwd=root, env=env, capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-1000:]
     assert " passed" in r.stdout and "failed" not in r.stdout, r.stdout[-500:]
+
+
+def test_gradients_that_cancel_stay_zero_with_fp32_inputs():
+    """A query that sees a single key has p = 1 and dS = dP - delta = 0, so dq = dk = 0.  fp32 operands are rounded
+    to bf16 on load: delta is formed from the same rounded dO as dP, or the difference of the two roundings
+    (about 1e-1 at head dim 256) would show up as a gradient."""
+    fa = _fa()
+    q, k, v, do = orc.make_qkv(31, 2, 2, 200, 1, 120, 256, torch.float32)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = fa.attention(qg, kg, vg, False, 0.3)
+    o.backward(do.cuda())
+    assert qg.grad.abs().max().item() <= 1e-4 and kg.grad.abs().max().item() <= 1e-3
+    want = do.bfloat16().float().sum(dim=2, keepdim=True)        # dv = sum over the queries of the rounded dO
+    assert (vg.grad.cpu() - want).abs().max().item() <= 1e-3 * want.abs().max().item()
