@@ -200,7 +200,11 @@ int dlt_swa_image_offsets(int32_t t_height, int32_t t_width, int32_t bh, int32_t
 /* ---- flash attention with separate qk / vo head dims -----------------------------------
  * q [B,H,Lq,dk], k [B,H,Lk,dk], v [B,H,Lk,dv], o [B,H,Lq,dv], lse2 fp32 [B,H,Lq].
  * Replaces _attn_fwd (src/flash_attn.py:81-172) and _attention.forward (:455-490); unlike
- * the reference (single N_CTX, :479) Lq != Lk is accepted when causal == 0. */
+ * the reference (single N_CTX, :479) Lq != Lk is accepted when causal == 0.
+ * Every dk, dv in 1..256 is computed; the tuned kernels take 2-byte element types with dk, dv
+ * multiples of 8 up to 128 and 16-byte aligned rows of unit last stride, other calls run on
+ * generic kernels several times slower (a caller may zero-pad dk and dv to the next multiple
+ * of 8: padded dims of q, k add nothing to the scores, padded dims of v give zero outputs). */
 typedef struct {
   int32_t B, H, Lq, Lk;
   int32_t dk, dv;
