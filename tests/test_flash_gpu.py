@@ -297,23 +297,6 @@ def test_bad_arguments_raise():
         _fa().attention(q, k[..., :32], k, False, 1.0)
 
 
-def test_register_staged_kernels_behind_the_environment_switch():
-    """DLT_FLASH_SYNC_STAGING=1 (read once per process) keeps the register-staged kernels for every head-dim class:
-    this file and the flash sweep of the fuzz file pass in a child process that sets it."""
-    import os
-    import subprocess
-    import sys
-    if os.environ.get("DLT_FLASH_SYNC_STAGING") == "1":
-        pytest.skip("already running with the switch set")
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    env = dict(os.environ, DLT_FLASH_SYNC_STAGING="1")
-    r = subprocess.run([sys.executable, "-u", "-m", "pytest", "tests/test_flash_gpu.py", "tests/test_fuzz_gpu.py", "-m", "gpu", "-x", "-q",
-                        "-k", "flash and not environment_switch", "-p", "no:cacheprovider"],
-                       cwd=root, env=env, capture_output=True, text=True, timeout=100)
-    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-1000:]
-    assert " passed" in r.stdout and "failed" not in r.stdout, r.stdout[-500:]
-
-
 def test_gradients_that_cancel_stay_zero_with_fp32_inputs():
     """A query that sees a single key has p = 1 and dS = dP - delta = 0, so dq = dk = 0.  fp32 operands are rounded
     to bf16 on load: delta is formed from the same rounded dO as dP, or the difference of the two roundings
