@@ -377,17 +377,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_kv_kernel
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
-  for (; ci + 1 < W.nchunks; ci++) {
+  // without a mask a full last chunk runs here too (same test-free body): the code below, whose per-pair tests cost
+  // registers the compiler finds by spilling, is then not executed at all
+  const int n_plain = (!CAUSAL && W.nchunks > 0 && !chunk_tail(W.nchunks - 1)) ? W.nchunks : W.nchunks - 1;
+  for (; ci < n_plain; ci++) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
     else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
     swa2_wait_copies();
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
-  if (W.nchunks > 0) {
+  if (ci < W.nchunks) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
-    else if (chunk_tail(ci)) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
-    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
   }
   __syncthreads();
   TIO* dkb = reinterpret_cast<TIO*>(a.dk) + b * a.dks[0] + h * a.dks[1];
@@ -595,17 +597,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
-  for (; ci + 1 < W.nchunks; ci++) {
+  // without a mask a full last chunk runs here too (same test-free body): the code below, whose per-pair tests cost
+  // registers the compiler finds by spilling, is then not executed at all
+  const int n_plain = (!CAUSAL && W.nchunks > 0 && !chunk_tail(W.nchunks - 1)) ? W.nchunks : W.nchunks - 1;
+  for (; ci < n_plain; ci++) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
     else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
     swa2_wait_copies();
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
-  if (W.nchunks > 0) {
+  if (ci < W.nchunks) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
-    else if (chunk_tail(ci)) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
-    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
   }
   __syncthreads();
 
@@ -827,17 +831,19 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
-  for (; ci + 1 < W.nchunks; ci++) {
+  // without a mask a full last chunk runs here too (same test-free body): the code below, whose per-pair tests cost
+  // registers the compiler finds by spilling, is then not executed at all
+  const int n_plain = (!CAUSAL && W.nchunks > 0 && !chunk_tail(W.nchunks - 1)) ? W.nchunks : W.nchunks - 1;
+  for (; ci < n_plain; ci++) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
     else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
     swa2_wait_copies();
     __syncthreads();
     bi = bi + 1 == NBUF ? 0 : bi + 1;
   }
-  if (W.nchunks > 0) {
+  if (ci < W.nchunks) {
     if (CAUSAL) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), FlashTailDyn{}, std::false_type{});
-    else if (chunk_tail(ci)) consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
-    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::false_type{}, std::false_type{});
+    else consume_t(ci, (Swa2Lds)buf_of(bi), buf_of(bi + AHEAD), std::true_type{}, std::false_type{});
   }
   __syncthreads();
   TIO* dqb = reinterpret_cast<TIO*>(a.dq) + b * a.dqs[0] + h * a.dqs[1];
