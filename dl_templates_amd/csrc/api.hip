@@ -309,6 +309,20 @@ int dlt_ensure_lds(const void* kern, int bytes) {
   return DLT_OK;
 }
 
+int dlt_device_cus() {
+  constexpr int MAXDEV = 64;
+  static std::mutex mu;
+  static int cus[MAXDEV] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAXDEV) return 256;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cus[dev] == 0) {
+    int n = 0;
+    cus[dev] = (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) ? n : 256;
+  }
+  return cus[dev];
+}
+
 static __device__ __align__(256) float g_delta_scratch[DLT_NOALLOC_MAX_DELTA];
 
 namespace {

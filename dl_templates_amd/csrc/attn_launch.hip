@@ -250,8 +250,6 @@ int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
 }
 
 // ---- marching token-grid kernels: head dim 64 exactly, windows up to 13 x 13, no rotation or R = 8 ----------
-constexpr int GPU_CUS = 256;   // MI355X
-
 bool swam_eligible(const AttnProblem& p, const Swa1Class& c) {
   if (c.D != 64 || p.dk != 64 || p.dv != 64) return false;
   if (p.g.WR > 6 || p.g.WC > 6) return false;
@@ -264,9 +262,10 @@ void swam_make_plan(const AttnProblem& p, SwamPlan& plan) {
   plan.nstrips = (p.g.TC + 15) / 16;
   const int steps = (p.g.TR + 7) / 8;
   const int64_t cols = (int64_t)p.B * p.H * plan.nstrips;
+  const int gpu_cus = dlt_device_cus();
   int ns = 1;
   for (int cand = 2; cand <= 8 && cand <= steps; cand++)
-    if (cols * ((steps + cand - 1) / cand) >= GPU_CUS) ns = cand;
+    if (cols * ((steps + cand - 1) / cand) >= gpu_cus) ns = cand;
   plan.band = 8 * ns;
   plan.nbands = (steps + ns - 1) / ns;
   dlt_fastdiv_make((uint32_t)(plan.nbands * plan.nstrips), plan.m_bh, plan.s_bh);

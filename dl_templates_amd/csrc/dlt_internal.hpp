@@ -14,6 +14,8 @@ int dlt_set_error(int code, const char* fmt, ...) __attribute__((format(printf, 
 // size than any before is asked for (per kernel and device): it costs tens of microseconds of host time, which would
 // otherwise sit in front of every launch.
 int dlt_ensure_lds(const void* kern, int bytes);
+// compute units of the current device (asked once per device; 256 when the query fails)
+int dlt_device_cus();
 
 #define DLT_REQUIRE(cond, ...)                                   \
   do {                                                           \

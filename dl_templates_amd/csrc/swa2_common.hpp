@@ -122,16 +122,20 @@ DLT_DEV bool swa2_visible(const Swa2Win& W, bool row_vis, int cg, int i, int ncg
 // a wait for ALL outstanding LDS reads (lgkmcnt(0)) and for all outstanding copies (vmcnt(0)), which serialises the
 // operand read-ahead of the loops that overlap copies with products.  Hidden from its counters, the waits for operand
 // reads are exact again; the waits for the copies themselves are explicit (swa2_wait_copies).  M0 (the LDS address of a
-// copy) is written here without the compiler's knowledge (it is a reserved register, not an allocatable one): kernels
-// that use these helpers must contain nothing else that goes through M0 (dynamic indexing of register arrays, the
-// compiler's own LDS-DMA builtin); the generated code of the streaming and flash kernels holds no other use.
+// copy) is a reserved register that cannot be named as an operand or a clobber: the statement saves it, sets it, issues
+// the copy (which reads M0 at issue) and puts the saved value back, so whatever the compiler itself keeps in M0 (dynamic
+// indexing of register arrays, its own LDS-DMA builtin, messages) survives a copy.
 DLT_DEV void dlt_copy16_to_lds(const char* base, uint32_t voff, char* lds) {
   const uint32_t m = (uint32_t)(uintptr_t)(DLT_LDS char*)lds;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %0" ::"s"(base), "v"(voff), "s"(m) : "memory");
+  uint32_t saved;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1\n\ts_mov_b32 m0, %0"
+               : "=&s"(saved) : "s"(base), "v"(voff), "s"(m) : "memory");
 }
 DLT_DEV void dlt_copy4_to_lds(const char* base, uint32_t voff, char* lds) {
   const uint32_t m = (uint32_t)(uintptr_t)(DLT_LDS char*)lds;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %1, %0" ::"s"(base), "v"(voff), "s"(m) : "memory");
+  uint32_t saved;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dword %2, %1\n\ts_mov_b32 m0, %0"
+               : "=&s"(saved) : "s"(base), "v"(voff), "s"(m) : "memory");
 }
 
 // ---- asynchronous staging -------------------------------------------------------------------------------

@@ -42,14 +42,29 @@ int swa2_launch_bwd_t(const Swa2BwdArgs& a, int grid, hipStream_t stream) {
   DLT_CHECK_LAUNCH("token-grid dK/dV launch (streaming kernels)");
   return DLT_OK;
 }
+// ncg: column groups of a wave's window, 4 (windows up to 13 columns) or 6 (up to 21); any other value has no
+// instantiation and is rejected
+template <typename TIO>
+int swa2_pick_fwd(const Swa2FwdArgs& a, int ncg, int grid, hipStream_t stream) {
+  switch (ncg) {
+    case 4: return swa2_launch_fwd_t<TIO, 4>(a, grid, stream);
+    case 6: return swa2_launch_fwd_t<TIO, 6>(a, grid, stream);
+    default: return dlt_set_error(DLT_ERR_UNSUPPORTED, "streaming token-grid kernels: no instantiation for %d column groups", ncg);
+  }
+}
+template <typename TIO>
+int swa2_pick_bwd(const Swa2BwdArgs& a, int ncg, int grid, hipStream_t stream) {
+  switch (ncg) {
+    case 4: return swa2_launch_bwd_t<TIO, 4>(a, grid, stream);
+    case 6: return swa2_launch_bwd_t<TIO, 6>(a, grid, stream);
+    default: return dlt_set_error(DLT_ERR_UNSUPPORTED, "streaming token-grid kernels: no instantiation for %d column groups", ncg);
+  }
+}
 }  // namespace
 
-// ncg: column groups of a wave's window, 4 (windows up to 13 columns) or 6 (up to 21)
 int DLT_SWA2_CAT(dlt_swa2_launch_fwd_, DLT_SWA2_D)(const Swa2FwdArgs& a, int ncg, int grid, hipStream_t stream) {
-  if (a.p.dtype == DLT_BF16) return ncg == 4 ? swa2_launch_fwd_t<bf16_t, 4>(a, grid, stream) : swa2_launch_fwd_t<bf16_t, 6>(a, grid, stream);
-  return ncg == 4 ? swa2_launch_fwd_t<f16_t, 4>(a, grid, stream) : swa2_launch_fwd_t<f16_t, 6>(a, grid, stream);
+  return a.p.dtype == DLT_BF16 ? swa2_pick_fwd<bf16_t>(a, ncg, grid, stream) : swa2_pick_fwd<f16_t>(a, ncg, grid, stream);
 }
 int DLT_SWA2_CAT(dlt_swa2_launch_bwd_, DLT_SWA2_D)(const Swa2BwdArgs& a, int ncg, int grid, hipStream_t stream) {
-  if (a.p.dtype == DLT_BF16) return ncg == 4 ? swa2_launch_bwd_t<bf16_t, 4>(a, grid, stream) : swa2_launch_bwd_t<bf16_t, 6>(a, grid, stream);
-  return ncg == 4 ? swa2_launch_bwd_t<f16_t, 4>(a, grid, stream) : swa2_launch_bwd_t<f16_t, 6>(a, grid, stream);
+  return a.p.dtype == DLT_BF16 ? swa2_pick_bwd<bf16_t>(a, ncg, grid, stream) : swa2_pick_bwd<f16_t>(a, ncg, grid, stream);
 }

@@ -167,17 +167,17 @@ def _backward_rot(q_rot, k_rot, v, o, lse, do, shape, rope):
 class TiledSwaRope(torch.autograd.Function):
     """o = TiledSwa(rope(q), rope(k), v) with the rotation fused into the q / k tile loads.
 
-    ``save_rotated`` (class attribute, default True): the forward pass also stores the rotated q and k
-    (what ``RotaryPE2D`` leaves in place in the reference's composition) and the backward pass reads
-    those, rotating only dq and dk back as they are stored.  False keeps nothing but the caller's q and k
-    and rotates every staged tile again in the backward kernels: two tensors less memory, slower.
+    ``save_rotated`` (optional last argument of ``apply``, default True): the forward pass also stores the
+    rotated q and k (what ``RotaryPE2D`` leaves in place in the reference's composition) and the backward pass
+    reads those, rotating only dq and dk back as they are stored.  False keeps nothing but the caller's q and k
+    and rotates every staged tile again in the backward kernels: two tensors less memory, slower.  It is a
+    per-call argument, kept in the call's own context: nothing is shared between calls or threads.
     """
-
-    save_rotated = True
 
     @staticmethod
     def forward(ctx, q, k, v, idx, row_cs_buffer, col_cs_buffer, b_size, t_height, t_width, row_size, col_size,
-                sm_scale):
+                sm_scale, save_rotated=None):
+        ctx.n_inputs = 12 if save_rotated is None else 13   # backward returns one entry per argument of apply
         ctx.dims = (q.shape[-1], v.shape[-1])
         plan = _pad_plan(q, v, b_size)
         if plan is not None:   # zero columns behind the rotated ones: see _pad_plan
@@ -186,7 +186,7 @@ class TiledSwaRope(torch.autograd.Function):
         assert row_cs_buffer.shape[1] == col_cs_buffer.shape[1]
         assert idx.shape[0] == q.shape[2]
         rope = (idx, row_cs_buffer, col_cs_buffer)
-        ctx.rotated = bool(TiledSwaRope.save_rotated)
+        ctx.rotated = True if save_rotated is None else bool(save_rotated)
         if ctx.rotated:
             o, m, q_rot, k_rot = _forward_rot(q, k, v, shape, rope)
             ctx.save_for_backward(q_rot, k_rot, v, m, o, idx, row_cs_buffer, col_cs_buffer)
@@ -207,7 +207,7 @@ class TiledSwaRope(torch.autograd.Function):
         else:
             dq, dk, dv = _backward(q, k, v, o, m, do, shape, rope)
         dq, dk, dv = _cut_last(dq, ctx.dims[0]), _cut_last(dk, ctx.dims[0]), _cut_last(dv, ctx.dims[1])
-        return (dq, dk, dv) + (None,) * 9
+        return (dq, dk, dv) + (None,) * (ctx.n_inputs - 3)
 
 
 def _image_shape(q, k, v, bh, bw, row_size, col_size, sm_scale):

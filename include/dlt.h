@@ -120,7 +120,10 @@ int dlt_swa_bwd(const void* q, const int64_t q_strides[4], const void* k, const 
  * rejected (DLT_ERR_INVALID, nothing launched) when a stride is negative or the largest offset
  * (B-1) s0 + (H-1) s1 + (N-1) s2 reaches DLT_NOALLOC_MAX_DELTA.  Every call on a GPU shares that GPU's
  * buffer and overwrites all of it that it reads: calls that overlap in time on one GPU (two streams,
- * two threads) race and must be serialised by the caller; results equal dlt_swa_bwd's bit for bit. */
+ * two threads) race and must be serialised by the caller; results equal dlt_swa_bwd's bit for bit.
+ * The first call on a device with a given kernel also resolves the scratch symbol and raises that kernel's
+ * LDS limit (host-side driver calls, no device memory): make one call with the shapes to be used outside any
+ * stream capture before recording the call into a HIP graph. */
 #define DLT_NOALLOC_MAX_DELTA (1 << 20)
 int dlt_swa_bwd_noalloc(const void* q, const int64_t q_strides[4], const void* k, const int64_t k_strides[4],
                         const void* v, const int64_t v_strides[4], const void* o, const int64_t o_strides[4],

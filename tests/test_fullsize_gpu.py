@@ -124,11 +124,10 @@ def test_c4_ragged_grid_border_band_against_cpu_oracle():
 
 
 @pytest.mark.parametrize("save_rotated", [True, False])
-def test_c3_one_batch_fused_rope_against_cpu_oracle(save_rotated, monkeypatch):
+def test_c3_one_batch_fused_rope_against_cpu_oracle(save_rotated):
     """Config 3 with B = 1 (all 8 heads, 64 x 64, d = 64, 13 x 13, rotary 32 of 64 dims, 5 % no-PE tokens): the fused
     op directly against the oracle's composition rope -> attention and its autograd."""
     sw, _, _ = _mods()
-    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save_rotated)
     B, H, th, tw, d, W = 1, 8, 64, 64, 64, 6
     N = th * tw
     q, k, v, do = orc.make_qkv(31, B, H, N, N, d, d, torch.bfloat16)
@@ -136,7 +135,7 @@ def test_c3_one_batch_fused_rope_against_cpu_oracle(save_rotated, monkeypatch):
     rcs, ccs = orc.rope_tables(8, th), orc.rope_tables(8, tw)
     o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, W, W, 0.125)
     qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
-    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, W, W, 0.125)
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, W, W, 0.125, save_rotated)
     o.backward(do.cuda())
     assert (o.float().cpu() - o_w).abs().max().item() <= 2e-2
     rel = lambda a, b: ((a.float().cpu() - b).abs().max() / b.abs().max()).item()
@@ -145,19 +144,18 @@ def test_c3_one_batch_fused_rope_against_cpu_oracle(save_rotated, monkeypatch):
 
 
 @pytest.mark.parametrize("save_rotated", [True, False])
-def test_c3_full_batch_fused_rope_equals_composition(save_rotated, monkeypatch):
+def test_c3_full_batch_fused_rope_equals_composition(save_rotated):
     """Both fused variants (rotated q, k kept for the backward pass / rotated again in every tile load) at the
     full size of config 3 against the composition of the standalone rotation and the plain operator: bit-equal where
     both run on the marching kernels (forward; backward from the kept rotated q, k)."""
     sw, _, fr = _mods()
-    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save_rotated)
     B, H, th, tw, d, W = 2, 8, 64, 64, 64, 6
     N = th * tw
     q, k, v, do = (t.cuda() for t in orc.make_qkv(3, B, H, N, N, d, d, torch.bfloat16))
     idx = orc.make_rope_idx(33, th, tw, 0.05).cuda()
     rcs, ccs = orc.rope_tables(8, th).cuda(), orc.rope_tables(8, tw).cuda()
     qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
-    o = sw.TiledSwaRope.apply(qg, kg, vg, idx, rcs, ccs, 1, th, tw, W, W, 0.125)
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx, rcs, ccs, 1, th, tw, W, W, 0.125, save_rotated)
     o.backward(do)
     q2, k2, v2 = (t.detach().requires_grad_(True) for t in (q, k, v))
     qr = fr.RotaryPE2D.apply(q2.clone().view(-1, N, d), idx, rcs, ccs).view(q.shape)

@@ -188,13 +188,8 @@ def test_random_head_dims_strides_and_scales_sliding_window():
             idx = orc.make_rope_idx(done, th, tw, 0.1)
             rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
             o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, WR, WC, scale)
-            old = sw.TiledSwaRope.save_rotated
-            sw.TiledSwaRope.save_rotated = keep
-            try:
-                o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, WR, WC, scale)
-                o.backward(do.to(dt).cuda())
-            finally:
-                sw.TiledSwaRope.save_rotated = old
+            o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, WR, WC, scale, keep)
+            o.backward(do.to(dt).cuda())
         else:
             o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), S, th, tw, WR, WC, scale)
             o = sw.TiledSwa.apply(qg, kg, vg, S, th, tw, WR, WC, scale)

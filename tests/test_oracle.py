@@ -245,6 +245,32 @@ def test_flash_ref_matches_explicit_softmax_lq_ne_lk():
     assert torch.allclose(dv, p.transpose(-1, -2) @ do, atol=1e-5)
 
 
+def test_flash_lse2_causal_is_the_log_sum_over_keys_up_to_the_query():
+    # per-row evaluation with explicit key lists: a flipped or shifted mask changes the first rows
+    q, k, v, do = orc.make_qkv(14, 1, 2, 17, 17, 8, 8)
+    scale = 0.7
+    got = orc.flash_lse2(q, k, scale, causal=True)
+    s = (q @ k.transpose(-1, -2)) * scale
+    for i in range(17):
+        want = torch.logsumexp(s[..., i, : i + 1], dim=-1) / math.log(2.0)
+        assert torch.allclose(got[..., i], want, atol=1e-5), i
+        if 0 < i < 16:
+            # the transposed mask (keys from the query on) and the strict one (keys before the query) give other values
+            for wrong in (s[..., i, i:], s[..., i, :i]):
+                assert not torch.allclose(got[..., i], torch.logsumexp(wrong, dim=-1) / math.log(2.0), atol=1e-3)
+    # row 0 sees one key: lse2 is that score in the log2 domain
+    assert torch.allclose(got[..., 0], s[..., 0, 0] * math.log2(math.e), atol=1e-5)
+    # exp2(s2 - lse2) over the visible keys are the softmax rows SDPA's causal mode uses
+    p = torch.exp2(s * math.log2(math.e) - got[..., None]).tril()
+    assert torch.allclose(p.sum(-1), torch.ones(1, 2, 17), atol=1e-5)
+    o = orc.flash_ref(q, k, v, True, scale)
+    assert torch.allclose(p @ v, o, atol=1e-5)
+    # and it differs from the dense one everywhere but in the last row
+    dense = orc.flash_lse2(q, k, scale, causal=False)
+    assert torch.allclose(got[..., -1], dense[..., -1], atol=1e-5)
+    assert (got[..., :-1] < dense[..., :-1] - 1e-4).all()
+
+
 def test_composed_rope_swa_grads_are_autograd_of_composition():
     q, k, v, do = orc.make_qkv(12, 1, 1, 16, 16, 16, 8)
     idx = orc.make_rope_idx(13, 4, 4, 0.2)

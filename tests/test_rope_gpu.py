@@ -73,6 +73,21 @@ def test_pe_mask_bit_exact():
     assert np.array_equal(got, orc.pe_mask(idx))
 
 
+def test_committed_fixture_bit_equal():
+    # tests/golden/rope_16x16.npz (fp32, R = 4, 24 dims of which 16 rotate, row-only / column-only / no-PE tokens):
+    # the stored outputs are the bar, the oracle is not called
+    import os
+    f = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "rope_16x16.npz"))
+    fr = _mods()
+    idx = torch.from_numpy(f["idx"]).cuda()
+    row_cs, col_cs = _tables(4, 16, 16)
+    x = torch.from_numpy(f["x"]).cuda()
+    y = fr.RotaryPE2D.apply(x, idx, row_cs.cuda(), col_cs.cuda())
+    assert y.data_ptr() == x.data_ptr()
+    assert np.array_equal(y.cpu().numpy(), f["y"])
+    assert np.array_equal(fr.rope_pe_mask(idx).cpu().numpy(), f["pe_bits"])
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
 def test_c2_shape(dtype):
     # benchmark config 2: B=4, H=8, 64x64 grid, d=64, first 32 dims rotated, 5% no-PE

@@ -117,12 +117,11 @@ def test_strided_grad_and_inputs():
 # the whole head dim at d = 128, rotary partners four 16-byte chunks apart (not within one staging thread's piece)
 @pytest.mark.parametrize("save_rotated", [True, False])
 @pytest.mark.parametrize("d,R", [(64, 8), (64, 16), (128, 16), (128, 8), (128, 32), (64, 4), (64, 3)])
-def test_fused_rope_backward(d, R, save_rotated, monkeypatch):
+def test_fused_rope_backward(d, R, save_rotated):
     """save_rotated: the forward pass keeps the rotated q, k and the backward pass reads them, rotating
     only dq / dk back on store (dlt_swa_fwd_rot / dlt_swa_bwd_rot); otherwise every tile load of the
     backward kernels rotates again (dlt_swa_fwd / dlt_swa_bwd with rope)."""
     sw = _swa()
-    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save_rotated)
     B, H, th, tw = 1, 2, 16, 16
     N = th * tw
     q, k, v, do = orc.make_qkv(9, B, H, N, N, d, d, torch.bfloat16)
@@ -131,7 +130,7 @@ def test_fused_rope_backward(d, R, save_rotated, monkeypatch):
     rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
     o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, 3, 3, 0.125)
     qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
-    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, 3, 3, 0.125)
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, 3, 3, 0.125, save_rotated)
     o.backward(do.cuda())
     assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
     errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
@@ -250,11 +249,10 @@ def test_rotated_side_outputs_with_awkward_strides():
                                                   (96, 96, 8, 10, 12, 3, True), (96, 128, 16, 10, 12, 3, False),
                                                   (64, 32, 16, 8, 8, 2, True), (128, 64, 8, 8, 12, 4, True),
                                                   (80, 80, 8, 10, 12, 3, True), (72, 40, 8, 9, 11, 2, False), (48, 48, 8, 8, 8, 2, True)])
-def test_fused_rope_with_head_dims_below_the_padded_class(d, dv, R, th, tw, W, save, monkeypatch):
+def test_fused_rope_with_head_dims_below_the_padded_class(d, dv, R, th, tw, W, save):
     """dk / dv that do not fill their padded class (32 in the 64 class, 96 in the 128 class) and dk != dv, with the
     rotation fused: staged pieces beyond the head dim stay zero, side outputs and gradients stop at the head dim."""
     sw = _swa()
-    monkeypatch.setattr(sw.TiledSwaRope, "save_rotated", save)
     N = th * tw
     q, k, v, do = orc.make_qkv(d + R, 1, 2, N, N, d, dv, torch.bfloat16)
     idx = orc.make_rope_idx(2, th, tw, 0.1)
@@ -262,7 +260,7 @@ def test_fused_rope_with_head_dims_below_the_padded_class(d, dv, R, th, tw, W, s
     scale = 1 / math.sqrt(d)
     o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, W, W, scale)
     qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
-    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, W, W, scale)
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, W, W, scale, save)
     o.backward(do.cuda())
     assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
     errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))

@@ -83,3 +83,66 @@ def test_sizes_beyond_the_scratch_are_rejected_before_any_launch():
     rc = lib.dlt_swa_bwd_noalloc(None, S(q), P(q), S(q), P(q), S(q), P(q), S(q), P(q), S(q), P(lse), st,
                                  P(q), S(q), P(q), S(q), P(q), S(q), shape, None, _lib.stream_of(q))
     assert rc == 1 and b"NULL" in lib.dlt_last_error()
+
+
+def _prepared(seed, B, H, th, tw, W, d):
+    from dl_templates_amd import tiled_swa as sw
+    N = th * tw
+    q, k, v, do = (t.cuda() for t in orc.make_qkv(seed, B, H, N, N, d, d, torch.bfloat16))
+    shape = sw._shape(q, k, v, 1, th, tw, W, W, 1 / math.sqrt(d))
+    o, lse = sw._forward(q, k, v, shape, None)
+    return q, k, v, o, lse, do, shape
+
+
+def _launch_noalloc(args, outs):
+    from dl_templates_amd import _lib
+    lib, P, S = _lib.load(), _lib.ptr, _lib.strides
+    q, k, v, o, lse, do, shape = args
+    dq, dk, dv = outs
+    _lib.check(lib.dlt_swa_bwd_noalloc(P(q), S(q), P(k), S(k), P(v), S(v), P(o), S(o), P(do), S(do), P(lse), S(lse),
+                                       P(dq), S(dq), P(dk), S(dk), P(dv), S(dv), shape, None, _lib.stream_of(q)))
+
+
+def test_a_warm_call_leaves_device_memory_as_it_was():
+    """After one call outside any capture (which resolves the scratch symbol and sets the kernels' LDS attribute once
+    per device), a further call changes neither the free device memory the driver reports nor torch's allocator."""
+    args = _prepared(7, 1, 4, 32, 32, 6, 64)
+    outs = tuple(torch.empty_like(t) for t in args[:3])
+    _launch_noalloc(args, outs)   # warm
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    for _ in range(3):
+        _launch_noalloc(args, outs)
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, (free0, free1)
+    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == (alloc0, reserved0)
+
+
+def test_captured_in_a_hip_graph_every_replay_equals_the_eager_call():
+    """The call it is meant for: recorded into a HIP graph (after a warm call outside the capture) and replayed, with
+    eager work and synchronisations between the replays; every replay must reproduce the eager gradients bit for bit."""
+    args = _prepared(8, 2, 4, 32, 48, 6, 64)
+    want = tuple(torch.empty_like(t) for t in args[:3])
+    _launch_noalloc(args, want)   # warm call, outside the capture; also the eager result
+    torch.cuda.synchronize()
+    outs = tuple(torch.empty_like(t) for t in args[:3])
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            _launch_noalloc(args, outs)
+    torch.cuda.current_stream().wait_stream(side)
+    small = _prepared(9, 1, 2, 16, 16, 3, 64)
+    for rep in range(4):
+        for t in outs:
+            t.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(("dq", "dk", "dv"), outs, want):
+            assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager call"
+        # eager work on the same scratch between the replays (a smaller call overwrites the head of it)
+        _launch_noalloc(small, tuple(torch.empty_like(t) for t in small[:3]))
+        torch.cuda.synchronize()
