@@ -234,11 +234,11 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
   const float* scal_base = stage_q ? lseb : delb;
   const int ls2 = (int)a.ls[2];
   // lane l < HCW copies the scalar of halo column l (clamped like the rows: positions outside the grid are masked)
-  const uint32_t scal_off = (uint32_t)(dlt_imax(0, dlt_imin(G.c0 - G.WC + lane, G.TC - 1)) * ls2) * 4u;
+  const uint32_t scal_off = (uint32_t)(swa2_scal_col(G, lane) * ls2) * 4u;
   auto issue_scalars = [&](int ch, char* buf) {
-    const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + 4 * ch + (wave & 3), G.TR - 1));
+    const int r = swa2_issue_grid_row(G, ch, wave);
     const char* row = reinterpret_cast<const char*>(scal_base) + (uint32_t)(r * G.TC * ls2) * 4u;   // wave-uniform
-    char* dst = buf + C::BUF + (wave >> 2) * (C::TOK * 4) + (wave & 3) * (C::HCW * 4);
+    char* dst = buf + swa2_scal_dst_off<C>(wave);
     if (lane < C::HCW)
       dlt_copy4_to_lds(row, scal_off, dst);
   };
@@ -254,7 +254,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
   Swa2Lane<C> L;
   swa2_lane_init(L, pc, n, g);
   // scalars of the queries (halo row g, window columns 4 cg .. 4 cg + 3) of a chunk
-  const int scal_lane = (g * C::HCW + 4 * pc) * 4;
+  const int scal_lane = swa2_scal_lane_off<C>(g, pc);
 
   f32x4 acck[VB], accv[VB];
 #pragma unroll

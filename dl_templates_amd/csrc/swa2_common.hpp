@@ -15,30 +15,7 @@
 #pragma once
 #include <type_traits>
 #include "swa1_common.hpp"
-
-constexpr int SWA2_THREADS = 512;
-
-template <int D_, int NCG_>
-struct Swa2Cfg {
-  static constexpr int D = D_, NCG = NCG_;
-  static constexpr int NKB = NCG / 2;            // blocks of 32 streamed tokens (two column groups) per chunk
-  static constexpr int KC = D / 32;              // 32-dim steps of a product that contracts over the head dim
-  static constexpr int VB = D / 16;              // 16-dim blocks of an accumulator
-  static constexpr int HCW = 4 * NCG + 12;       // staged halo columns
-  static constexpr int TOK = 4 * HCW;            // tokens of a chunk
-  static constexpr int ROW = 2 * D;              // bytes of a token row
-  static constexpr int PIECES = ROW / 16;        // 16-byte pieces of a row
-  static constexpr int SWZ = PIECES / 8;         // swizzle multiplier
-  static constexpr int TPI = 64 / PIECES;        // tokens per copy instruction
-  static constexpr int NI = (HCW + TPI - 1) / TPI;   // copy instructions per halo row
-  static constexpr int REGION = TOK * ROW;       // one tensor of a chunk
-  static constexpr int BUF = 2 * REGION;         // both tensors of a chunk
-  static constexpr int LDS = 2 * BUF;            // two chunk buffers
-  static constexpr int SCAL = 2 * TOK * 4;       // per-token scalars of a chunk (dK/dV kernel): lse2 then delta
-  static constexpr int BUF_KV = BUF + SCAL;
-  static constexpr int LDS_KV = 2 * BUF_KV;
-  static constexpr int TILE = 16 * ROW;          // wave-private tile of the store epilogue
-};
+#include "swa2_index.h"
 
 // compile-time loop: f(std::integral_constant<int, I>) for I = I0 .. N - 1
 template <int I, int N, typename F>
@@ -56,64 +33,8 @@ DLT_DEV u32x2 swa2_lds_tr(Swa2Lds p) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-struct Swa2Plan {
-  int32_t nblk_r, nblk_c;
-  uint32_t m_bh, s_bh, m_c, s_c, m_h, s_h;   // exact multiply-shift divisions by nblk_r * nblk_c, nblk_c and H
-};
-
-struct Swa2Geom {
-  int TR, TC, WR, WC;
-  int r0, c0;   // first grid row / column of the band
-  int b, h;
-  int ch_first, ch_last;   // chunks of the band's halo that hold grid rows
-};
-
 DLT_DEV Swa2Geom swa2_geom(const AttnProblem& p, const Swa2Plan& P) {
-  Swa2Geom G;
-  const int lin = xcd_remap(blockIdx.x, gridDim.x);
-  const int per_bh = P.nblk_r * P.nblk_c;
-  const int bh = (int)dlt_fastdiv((uint32_t)lin, P.m_bh, P.s_bh);
-  const int rem = lin - bh * per_bh;
-  const int br = (int)dlt_fastdiv((uint32_t)rem, P.m_c, P.s_c);
-  G.b = (int)dlt_fastdiv((uint32_t)bh, P.m_h, P.s_h);
-  G.h = bh - G.b * p.H;
-  G.TR = p.g.TR; G.TC = p.g.TC; G.WR = p.g.WR; G.WC = p.g.WC;
-  G.r0 = 8 * br;
-  G.c0 = 16 * (rem - br * P.nblk_c);
-  const int lo = dlt_imax(0, G.WR - G.r0), hi = dlt_imin(7 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
-  G.ch_first = lo >> 2;
-  G.ch_last = hi >> 2;
-  return G;
-}
-
-// per-lane window of an own token in the coordinates of the band's halo
-struct Swa2Win {
-  int rlo, rhi;      // visible halo rows [rlo, rhi]
-  int clo, cspan;    // visible window columns [clo, clo + cspan] (cspan < 0: the token lies outside the grid)
-  int ch_lo, ch_hi;  // chunks that hold visible rows of the wave's patch (wave-uniform)
-};
-
-DLT_DEV Swa2Win swa2_window(const Swa2Geom& G, int rg, int pc, int n) {
-  Swa2Win w;
-  const int qr = 4 * rg + (n >> 2), qc = n & 3;
-  const int c_p = G.c0 + 4 * pc;
-  const bool ok = (G.r0 + qr < G.TR) && (c_p + qc < G.TC);
-  w.rlo = dlt_imax(qr, G.WR - G.r0);
-  w.rhi = dlt_imin(qr + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
-  w.clo = dlt_imax(qc, G.WC - c_p);
-  const int chi = dlt_imin(qc + 2 * G.WC, G.TC - 1 - c_p + G.WC);
-  w.cspan = ok ? chi - w.clo : -1;
-  // halo rows of the patch that hold grid rows
-  const int plo = dlt_imax(4 * rg, G.WR - G.r0), phi = dlt_imin(4 * rg + 3 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
-  const bool patch_ok = (G.r0 + 4 * rg < G.TR) && (c_p < G.TC) && plo <= phi;
-  w.ch_lo = patch_ok ? plo >> 2 : 1;
-  w.ch_hi = patch_ok ? phi >> 2 : 0;
-  return w;
-}
-
-// visibility of the streamed token (halo row covered by row_vis, window column 4 cg + i) from the lane's own token
-DLT_DEV bool swa2_visible(const Swa2Win& W, bool row_vis, int cg, int i, int ncg) {
-  return row_vis & (cg < ncg) & ((unsigned)(4 * cg + i - W.clo) <= (unsigned)W.cspan);
+  return swa2_geom_at(p.g.TR, p.g.TC, p.g.WR, p.g.WC, p.H, P, xcd_remap(blockIdx.x, gridDim.x));
 }
 
 // One copy instruction as the hardware sees it: 64 lanes x 16 (or 4) bytes from `base + voff` (base wave-uniform)
@@ -138,11 +59,7 @@ DLT_DEV void dlt_copy4_to_lds(const char* base, uint32_t voff, char* lds) {
                : "=&s"(saved) : "s"(base), "v"(voff), "s"(m) : "memory");
 }
 
-// ---- asynchronous staging -------------------------------------------------------------------------------
-// Wave w copies halo row (w & 3) of tensor (w >> 2) of every chunk in NI instructions of 64 lanes; instruction i,
-// lane l writes LDS slot 64 i + l of the row = physical piece l % PIECES of halo column TPI i + l / PIECES, and
-// therefore fetches the logical piece (l % PIECES) ^ (SWZ (token & 7)) of that token.  Lanes past the last halo
-// column of the last instruction stay idle.
+// ---- asynchronous staging (maps in swa2_index.h) ----------------------------------------------------------
 template <typename C>
 struct Swa2Stage {
   uint32_t off[C::NI];   // byte offset of the lane's piece inside a grid row of the tensor, per instruction
@@ -152,13 +69,8 @@ struct Swa2Stage {
 template <typename C>
 DLT_DEV void swa2_stage_init(Swa2Stage<C>& st, const Swa2Geom& G, int wave, int lane, int sn2) {
 #pragma unroll
-  for (int i = 0; i < C::NI; i++) {
-    const int hc = C::TPI * i + lane / C::PIECES;
-    const int tok = (wave & 3) * C::HCW + hc;
-    const int cc = dlt_imax(0, dlt_imin(G.c0 - G.WC + hc, G.TC - 1));   // clamped: positions outside the grid are masked
-    st.off[i] = (uint32_t)(cc * sn2 + 16 * ((lane % C::PIECES) ^ (C::SWZ * (tok & 7))));
-  }
-  st.last_on = C::TPI * (C::NI - 1) + lane / C::PIECES < C::HCW;
+  for (int i = 0; i < C::NI; i++) st.off[i] = swa2_stage_off<C>(G, wave, lane, sn2, i);
+  st.last_on = swa2_stage_last_on<C>(lane);
 }
 
 // one of the NI copy instructions of a halo row (to be spread between the products of a chunk: issued together they
@@ -171,11 +83,10 @@ DLT_DEV void swa2_issue_one(const Swa2Stage<C>& st, const char* row, char* dst) 
   }
 }
 DLT_DEV const char* swa2_issue_row(const Swa2Geom& G, int ch, const char* base, uint32_t rowstride, int wave) {
-  const int r = dlt_imax(0, dlt_imin(G.r0 - G.WR + 4 * ch + (wave & 3), G.TR - 1));
-  return base + (uint32_t)r * rowstride;   // wave-uniform
+  return base + (uint32_t)swa2_issue_grid_row(G, ch, wave) * rowstride;   // wave-uniform
 }
 template <typename C>
-DLT_DEV char* swa2_issue_dst(char* buf, int wave) { return buf + (wave >> 2) * C::REGION + (wave & 3) * (C::HCW * C::ROW); }
+DLT_DEV char* swa2_issue_dst(char* buf, int wave) { return buf + swa2_issue_dst_off<C>(wave); }
 
 // copy halo row (wave & 3) of chunk `ch` of the wave's tensor into its place in `buf`
 template <typename C>
@@ -198,36 +109,12 @@ DLT_DEV void swa2_wait_copies() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"
     __builtin_amdgcn_sched_group_barrier(0x002, (nv), 0);  \
   }
 
-// ---- operand reads -----------------------------------------------------------------------------------------
-// Lane constants of a wave whose window starts at halo column 4 pc.
-template <typename C>
-struct Swa2Lane {
-  int a[C::KC];    // A operand (token = MFMA row, head dim along k): byte offset of k-piece c of the lane's token row for an
-                   // even column group (odd groups: a[c ^ (KC / 2)])
-  int tr[C::VB];   // transposing read (head dim = MFMA row, tokens along k): byte offset for dims 16 d .. 16 d + 15
-};
-
-template <typename C>
-DLT_DEV void swa2_lane_init(Swa2Lane<C>& L, int pc, int n, int g) {
-  // A operand: lane (n, g) reads token (halo row n >> 2, column 4 (pc + cg) + (n & 3)) of a chunk, pieces 4 c + g;
-  // token & 7 = (n & 3) | 4 ((n >> 2) + pc + cg & 1)  (HCW = 4 mod 8)
-  const int tok = (n >> 2) * C::HCW + 4 * pc + (n & 3);
-  const int par = ((n >> 2) + pc) & 1;
-#pragma unroll
-  for (int c = 0; c < C::KC; c++) L.a[c] = tok * C::ROW + 16 * ((4 * c + g) ^ (C::SWZ * ((n & 3) | (4 * par))));
-  // transposing read: lane (n, g) addresses token (halo row g, column 4 (pc + cg0) + (n >> 2)), cg0 even, 8 bytes at dim
-  // 16 d + 4 (n & 3): piece 2 d + ((n & 3) >> 1); token & 7 = (n >> 2) | 4 ((g + pc) & 1)
-  const int tok2 = g * C::HCW + 4 * pc + (n >> 2);
-  const int sw = C::SWZ * ((n >> 2) | (4 * ((g + pc) & 1)));
-#pragma unroll
-  for (int d = 0; d < C::VB; d++) L.tr[d] = tok2 * C::ROW + 16 * ((2 * d + ((n & 3) >> 1)) ^ sw) + 8 * (n & 1);
-}
-
+// ---- operand reads (lane constants and offsets in swa2_index.h) ------------------------------------------------
 // A-operand pieces of the 16 tokens at column group CG of a chunk region: k[c] = head dims 32 c + 8 g .. + 7
 template <typename C, int CG>
 DLT_DEV void swa2_read_a(Swa2Lds region, const Swa2Lane<C>& L, u32x4 (&k)[C::KC]) {
 #pragma unroll
-  for (int c = 0; c < C::KC; c++) k[c] = swa2_lds16(region + 4 * C::ROW * CG + L.a[(CG & 1) ? (c ^ (C::KC / 2)) : c]);
+  for (int c = 0; c < C::KC; c++) k[c] = swa2_lds16(region + swa2_read_a_off<C, CG>(L, c));
 }
 
 // A operands with tokens along k for the 32 tokens (4 halo rows x 8 columns) at column groups 2 KB, 2 KB + 1 of a chunk
@@ -237,8 +124,8 @@ DLT_DEV void swa2_read_tr(Swa2Lds region, const Swa2Lane<C>& L, u32x4 (&v)[ND]) 
 #pragma unroll
   for (int i = 0; i < ND; i++) {
     const int d = D0 + i;
-    const u32x2 lo = swa2_lds_tr(region + 8 * C::ROW * KB + L.tr[d]);
-    const u32x2 hi = swa2_lds_tr(region + 8 * C::ROW * KB + 4 * C::ROW + L.tr[d ^ (C::VB / 2)]);
+    const u32x2 lo = swa2_lds_tr(region + swa2_read_tr_off<C, KB>(L, d, 0));
+    const u32x2 hi = swa2_lds_tr(region + swa2_read_tr_off<C, KB>(L, d, 1));
     v[i].x = lo.x; v[i].y = lo.y; v[i].z = hi.x; v[i].w = hi.y;
   }
 }
@@ -262,7 +149,7 @@ DLT_DEV void swa2_store_own(char* sW, const f32x4 (&acc)[C::VB], float mul, TIO*
     u32x2 w;
     w.x = pack2<CT>(acc[d][0] * mul, acc[d][1] * mul);
     w.y = pack2<CT>(acc[d][2] * mul, acc[d][3] * mul);
-    *reinterpret_cast<u32x2*>(sW + n * C::ROW + 16 * ((2 * d + (g >> 1)) ^ (n & 7)) + 8 * (g & 1)) = w;
+    *reinterpret_cast<u32x2*>(sW + swa2_tile_write_off<C>(n, g, d)) = w;
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -272,7 +159,7 @@ DLT_DEV void swa2_store_own(char* sW, const f32x4 (&acc)[C::VB], float mul, TIO*
 #pragma unroll
   for (int it = 0; it < 16 / RPI; it++) {
     const int row = lane / C::PIECES + RPI * it;
-    const u32x4 v = lds_read16(sW + row * C::ROW + 16 * (c ^ (row & 7)));
+    const u32x4 v = lds_read16(sW + swa2_tile_read_off<C>(row, c));
     const int r = r_p + (row >> 2), col = c_p + (row & 3);
     if (r < G.TR && col < G.TC) *reinterpret_cast<u32x4*>(base + (int64_t)(r * G.TC + col) * sn + 8 * c) = v;
   }
