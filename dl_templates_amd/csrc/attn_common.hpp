@@ -72,6 +72,7 @@ DLT_DEV void keep_branch() { asm volatile(""); }
 
 DLT_DEV void pin_loaded(const u32x4& v) { asm volatile("" ::"v"(v)); }
 DLT_DEV void pin_loaded(float v) { asm volatile("" ::"v"(v)); }
+DLT_DEV void pin_loaded(const f32x4& v) { asm volatile("" ::"v"(v)); }
 template <int N>
 DLT_DEV void pin_loaded(const u32x4 (&f)[N]) {
 #pragma unroll

@@ -10,7 +10,7 @@
 // Both recompute P = exp2(s * scale - lse2) per 32-token block; tokens of the ring side are the MFMA rows, so P / dS
 // leave the first products in the layout the second products take as B operand.
 // ROPE 0: no rotation; 3: q and k arrive rotated (saved by the forward pass), dq / dk get the transposed rotation as
-// they are stored.
+// they are stored.  TL: the rotary tables are copied into LDS in the prologue and read from there.
 #pragma once
 #include "swam_fwd_kernel.hpp"
 
@@ -36,20 +36,23 @@ DLT_DEV void swam_frag_issue(SwamFrag& w, const char* base, int sn2, int tok, in
 DLT_DEV void swam_frag_pin(const SwamFrag& w) { pin_loaded(w.f[0]); pin_loaded(w.f[1]); }
 
 // table rows for the two transposed tile rows a lane stores (piece lane & 7 of tokens tok[0], tok[1])
-DLT_DEV void swam_store_tabs(SwamTab (&tb)[2], const int32_t (&id)[2], int lane, const RopeDev& rope) {
+template <bool TL>
+DLT_DEV void swam_store_tabs(SwamTab (&tb)[2], const int32_t (&id)[2], int lane, const RopeDev& rope, SwamLds tabs) {
   const int c = lane & 7;
 #pragma unroll
-  for (int it = 0; it < 2; it++) swam_tab_issue(tb[it], id[it], (c >> 1) & 1, rope);
+  for (int it = 0; it < 2; it++) swam_tab_get<TL>(tb[it], id[it], (c >> 1) & 1, rope, tabs);
 }
 
 // =============================================================================================== dQ
-template <typename TIO, int ROPE>
+template <typename TIO, int ROPE, bool TL>
 __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   constexpr int D = 64;
   constexpr bool ROT = ROPE == 3;
+  static_assert(!TL || ROT, "LDS tables only with rotation");
   constexpr int REGION = swam_region(D), SLOT = swam_slot(D);
   extern __shared__ __align__(16) char smem[];
+  SwamLds tabs = (SwamLds)(smem + swam_ring(D));
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -126,10 +129,16 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
   Own cur;
   float del_n;
   {
+    f32x4 tab16;
+    if (TL) tab16 = swam_tab_fetch(rope, tid);
     SwamItem it[SWAM_NSLOT];
 #pragma unroll
     for (int c = 0; c < SWAM_NSLOT; c++) swam_issue(it[c], st, G, c, side[c & 1]);
     own_issue(cur, G.r0 + 4 * rg);
+    if (TL) {
+      pin_loaded(tab16);
+      swam_tab_store(smem + swam_ring(D), tid, tab16);   // visible after the barrier that ends the prologue
+    }
     // chunk by chunk (loads return in order): the LDS writes of a chunk overlap the arrival of the later ones
 #pragma unroll
     for (int c = 0; c < SWAM_NSLOT; c++) {
@@ -220,7 +229,7 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
 #pragma unroll
     for (int it = 0; it < 2; it++) tok[it] = swam_own_tok(G, r_p, c_p, (lane >> 3) + 8 * it);
     SwamTab tb[2];
-    if (ROT) swam_store_tabs(tb, id, lane, rope);
+    if (ROT) swam_store_tabs<TL>(tb, id, lane, rope, tabs);
     u32x4 v[2], pv[2];
     swam_tile_transpose<CT, ROT>(scratch_of(s), r.acc, sm_scale, lane, v, pv);
     if (ROT) {
@@ -262,15 +271,18 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
 }
 
 // =============================================================================================== dK / dV
-template <typename TIO, int ROPE>
+template <typename TIO, int ROPE, bool TL>
 __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   constexpr int D = 64;
   constexpr bool ROT = ROPE == 3;
+  static_assert(!TL || ROT, "LDS tables only with rotation");
   constexpr int REGION = swam_region(D), SLOT = swam_slot(D);
   extern __shared__ __align__(16) char smem[];
   float* sLse = reinterpret_cast<float*>(smem + swam_ring(D));   // [slot][token of the chunk]
   float* sDel = sLse + SWAM_NSLOT * SWAM_TOK;
+  constexpr int TAB_OFF = swam_ring(D) + 2 * SWAM_NSLOT * SWAM_TOK * 4;
+  SwamLds tabs = (SwamLds)(smem + TAB_OFF);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
@@ -347,6 +359,8 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
   // ---- prologue
   Own cur;
   {
+    f32x4 tab16;
+    if (TL) tab16 = swam_tab_fetch(rope, tid);
     SwamItem it[SWAM_NSLOT];
     float sc[3] = {0.f, 0.f, 0.f};
 #pragma unroll
@@ -355,6 +369,10 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
     for (int i = 0; i < 3; i++)
       if (kpar + 2 * i < SWAM_NSLOT) sc[i] = scalar_issue(kpar + 2 * i);
     own_issue(cur, G.r0 + 4 * rg);
+    if (TL) {
+      pin_loaded(tab16);
+      swam_tab_store(smem + TAB_OFF, tid, tab16);   // visible after the barrier that ends the prologue
+    }
 #pragma unroll
     for (int c = 0; c < SWAM_NSLOT; c++) {
       swam_pin(it[c]);
@@ -458,7 +476,7 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_kv_kernel(const SwamBwd
 #pragma unroll
     for (int it = 0; it < 2; it++) tok[it] = swam_own_tok(G, r_p, c_p, (lane >> 3) + 8 * it);
     SwamTab tb[2];
-    if (ROT) swam_store_tabs(tb, id, lane, rope);
+    if (ROT) swam_store_tabs<TL>(tb, id, lane, rope, tabs);
     u32x4 v[2], pv[2], w[2], unused[2];
     swam_tile_transpose<CT, false>(scratch_of(s), r.dv, 1.0f, lane, w, unused);
     swam_tile_transpose<CT, ROT>(scratch_of(s), r.dk, sm_scale, lane, v, pv);

@@ -16,6 +16,8 @@
 #pragma once
 #include "swa1_common.hpp"
 
+typedef DLT_LDS const char* SwamLds;   // 32-bit LDS address: constant parts of an offset fold into the instruction
+
 constexpr int SWAM_HCW = 28;               // staged halo columns: 16 own + 2 * 6
 constexpr int SWAM_TOK = 4 * SWAM_HCW;     // tokens of a chunk
 constexpr int SWAM_NSLOT = 5;
@@ -149,6 +151,39 @@ DLT_DEV void swam_tab_issue(SwamTab& tb, int32_t id, int axis, const RopeDev& ro
   }
 }
 
+// ---- rotary tables resident in LDS --------------------------------------------------------------------
+// Both tables (8 rotary pairs: 64 bytes per position) are copied into LDS once per workgroup when they fit
+// SWAM_TAB_BYTES: row table first, the column table behind it.  A table row then costs four LDS reads instead of a
+// global load that can only be requested once the token's index has arrived (index -> table row is a dependent chain
+// in front of every rotation: in the prologue, between the steps, in front of the rotating stores).
+constexpr int SWAM_TAB_BYTES = 8192;
+DLT_DEV bool swam_tab_fits(const RopeDev& rope) { return (rope.row_len + rope.col_len) * 64 <= SWAM_TAB_BYTES; }
+
+// the 16 bytes thread `tid` of the 512 copies (threads past the tables' end re-read the last row: no access out of bounds)
+DLT_DEV f32x4 swam_tab_fetch(const RopeDev& rope, int tid) {
+  const int row = tid >> 2, q = tid & 3;
+  const int rc = dlt_imin(row, rope.row_len + rope.col_len - 1);
+  const float* p = rc < rope.row_len ? rope.row_cs + (int64_t)rc * rope.rs0 : rope.col_cs + (int64_t)(rc - rope.row_len) * rope.cs0;
+  p += 4 * q;
+  return f32x4{p[0], p[1], p[2], p[3]};
+}
+DLT_DEV void swam_tab_store(char* tabs, int tid, const f32x4& v) { *reinterpret_cast<f32x4*>(tabs + 16 * tid) = v; }
+
+// table row of a token from the LDS copy (TL) or from global memory
+template <bool TL>
+DLT_DEV void swam_tab_get(SwamTab& tb, int32_t id, int axis, const RopeDev& rope, SwamLds tabs) {
+  if constexpr (TL) {
+    int pos = axis == 0 ? dlt_rope_row(id) : dlt_rope_col(id);
+    tb.rot = pos >= 0;
+    pos = dlt_imax(0, dlt_imin(pos, (axis == 0 ? rope.row_len : rope.col_len) - 1));
+    SwamLds p = tabs + ((axis == 0 ? 0 : rope.row_len) + pos) * 64;
+#pragma unroll
+    for (int j = 0; j < 4; j++) tb.t[j] = *reinterpret_cast<DLT_LDS const f32x4*>(p + 16 * j);
+  } else {
+    swam_tab_issue(tb, id, axis, rope);
+  }
+}
+
 // rotate the pair (lo, hi) = (first, second element of each of 8 rotary pairs); `inverse`: transposed rotation
 template <typename CT>
 DLT_DEV void swam_rotate_pair(u32x4& lo, u32x4& hi, const SwamTab& tb, bool inverse) {
@@ -201,8 +236,6 @@ DLT_DEV void swam_lane_init(SwamLane& L, int pc, int n, int g) {
     L.tr[d] = tok2 * 128 + 16 * piece + 8 * (n & 1);
   }
 }
-
-typedef DLT_LDS const char* SwamLds;   // 32-bit LDS address: constant parts of an offset fold into the instruction
 
 DLT_DEV u32x4 swam_lds16(SwamLds p) { return *reinterpret_cast<DLT_LDS const u32x4*>(p); }
 DLT_DEV u32x2 swam_lds_tr(SwamLds p) {

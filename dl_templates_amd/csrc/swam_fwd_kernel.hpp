@@ -64,20 +64,25 @@ DLT_DEV void swam_own_rotate(SwamOwn& w, const SwamTab& tb, int g, bool inverse)
   w.f[0] = pack8<CT>(self);
 }
 
-// ROPE: 0 no rotation, 2 q and k rotated on their way in (k: between HBM and LDS, q: own fragments)
-template <typename TIO, int ROPE>
+// ROPE: 0 no rotation, 2 q and k rotated on their way in (k: between HBM and LDS, q: own fragments); TL: the rotary
+// tables are copied into LDS (behind the ring) at kernel start and every table row is read from there
+template <typename TIO, int ROPE, bool TL>
 __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArgs a) {
+  static_assert(!TL || ROPE != 0, "LDS tables only with rotation");
   typedef typename ComputeOf<TIO>::type CT;
   constexpr int D = 64;
   constexpr bool ROT = ROPE != 0;
   constexpr int REGION = swam_region(D), SLOT = swam_slot(D);
   extern __shared__ __align__(16) char smem[];
+  SwamLds tabs = (SwamLds)(smem + swam_ring(D));
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int pc = wave & 3, rg = wave >> 2;   // patch column, row group
   const SwamGeom G = swam_geom(a.p, a.plan);
+  f32x4 tab16;
+  if (TL) tab16 = swam_tab_fetch(a.p.rope, tid);   // first load of the kernel: the tables do not depend on any index
 
   const char* qb = reinterpret_cast<const char*>(a.q) + 2 * (G.b * a.qs[0] + G.h * a.qs[1]);
   const char* kb_ = reinterpret_cast<const char*>(a.k) + 2 * (G.b * a.ks[0] + G.h * a.ks[1]);
@@ -159,7 +164,13 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
     for (int c = 0; c < SWAM_NSLOT; c++) swam_issue(it[c], st, G, c, side[c & 1]);
     swam_own_issue<ROT>(qo, qb, sn2q, G, G.r0 + 4 * rg, c_p, n, g);
     SwamTab tb[3], tbq;
-    if (ROT) {
+    if (TL) {
+      // the tables into LDS (loads return in order: this one was requested first), visible to every wave after the barrier
+      pin_loaded(tab16);
+      swam_tab_store(smem + swam_ring(D), tid, tab16);
+      __syncthreads();
+    }
+    if (ROT && !TL) {
 #pragma unroll
       for (int i = 0; i < 3; i++)
         if (kpar + 2 * i < SWAM_NSLOT) swam_tab_issue(tb[i], idk[i], st.qd, rope);
@@ -187,6 +198,12 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
 #pragma unroll
       for (int c = 0; c < SWAM_NSLOT; c++) swam_pin(it[c]);
       swam_own_pin(qo, ROT);
+      if (TL) {
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+          if (kpar + 2 * i < SWAM_NSLOT) swam_tab_get<true>(tb[i], idk[i], st.qd, rope, tabs);
+        swam_tab_get<true>(tbq, idq, g >> 1, rope, tabs);
+      }
       if (kpar == 0) {
         rotate_k(it[0], tb[0]); commit_chunk(it[0], 0);
         rotate_k(it[2], tb[1]); commit_chunk(it[2], 2);
@@ -345,8 +362,8 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
     SwamTab tbk, tbq;
     if (ROT) {
       asm volatile("" ::"v"(idk_nn), "v"(idq_nn));
-      swam_tab_issue(tbk, idk_next, st.qd, rope);
-      swam_tab_issue(tbq, idq_next, g >> 1, rope);
+      swam_tab_get<TL>(tbk, idk_next, st.qd, rope, tabs);
+      swam_tab_get<TL>(tbq, idq_next, g >> 1, rope, tabs);
     }
     const OutRows w = transpose_o(r, s);   // LDS only: overlaps the table loads
     if (ROT) {

@@ -156,6 +156,30 @@ def test_fused_rope_backward(d, R, save_rotated):
             assert max(_rel(q2.grad, qg.grad.float().cpu()), _rel(k2.grad, kg.grad.float().cpu())) <= 1e-2
 
 
+@pytest.mark.parametrize("table_len", [64, 65, 200])
+def test_fused_rope_table_lengths_around_the_lds_copy(table_len):
+    """Head dim 64 with 8 rotary pairs: the marching kernels keep both rotary tables in LDS while row + column table
+    have at most 128 positions (64 + 64: the copy is exactly full) and read table rows from global memory beyond that
+    (65 + 65, 200 + 200).  Positions near the end of the tables are used so that a clipped or shifted copy shows."""
+    sw = _swa()
+    B, H, th, tw = 1, 2, 24, 20
+    N = th * tw
+    q, k, v, do = orc.make_qkv(21, B, H, N, N, 64, 64, torch.bfloat16)
+    off_r, off_c = table_len - th, table_len - tw      # rows / columns index the last positions of the tables
+    rr, cc = torch.meshgrid(torch.arange(th, dtype=torch.int32) + off_r, torch.arange(tw, dtype=torch.int32) + off_c, indexing="ij")
+    idx = ((rr << 16) | cc).reshape(-1).to(torch.int32)
+    idx[3] = -1
+    idx[17] = ((off_r + 2) << 16) | 0xFFFF
+    rcs, ccs = orc.rope_tables(8, table_len), orc.rope_tables(8, table_len)
+    o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q.float(), k.float(), v.float(), do.float(), idx, rcs, ccs, 1, th, tw, 4, 5, 0.125)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, 4, 5, 0.125)
+    o.backward(do.cuda())
+    assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert max(errs) <= GRAD_TOL, errs
+
+
 def test_rotated_side_outputs_and_backward_from_them():
     """dlt_swa_fwd_rot stores exactly what the standalone rotation produces, leaves q / k alone, accepts
     strided side outputs, and dlt_swa_bwd_rot from those tensors equals dlt_swa_bwd from the originals."""
