@@ -105,7 +105,10 @@ template <typename TIO, int DK, int DV, int NP>
 __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr int PQ = DK * 2 + 16, PV = DV * 2 + 16;
+  // fp32 tensors: q and k are staged as hi + lo bf16 pairs (stage_tile_split) and a score is three products, as in the
+  // forward kernel whose log-sum-exp the probabilities are recomputed against; dK / dQ contract over the hi parts
+  constexpr bool SPLIT = sizeof(TIO) == 4;
+  constexpr int PQ = DK * (SPLIT ? 4 : 2) + 16, PV = DV * 2 + 16;
   constexpr int OWN = 64 * NP;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16, VB = DV / 16;
 
@@ -138,17 +141,20 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
 
   // ---- own keys / values -> B-operand fragments (head dim along k)
-  stage_tile<TIO, CT, DK>(sOwnK, PQ, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, OWN,
+  stage_tile_qk<TIO, CT, DK>(sOwnK, PQ, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, fwd_rope, tid);
   stage_tile<TIO, CT, DV>(sOwnV, PV, vb_, tok_addr(a.vs, a.p.tm), a.vs[3], a.p.dv, a.v_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, no_rope, tid);
   __syncthreads();
-  u32x4 kf[NP][KC], vf[NP][VC];
+  u32x4 kf[NP][KC], klo[SPLIT ? NP : 1][KC], vf[NP][VC];
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = wave * 16 * NP + 16 * p + n;
 #pragma unroll
-    for (int c = 0; c < KC; c++) kf[p][c] = lds_read16(sOwnK + row * PQ + (32 * c + 8 * g) * 2);
+    for (int c = 0; c < KC; c++) {
+      kf[p][c] = lds_read16(sOwnK + row * PQ + (32 * c + 8 * g) * 2);
+      if constexpr (SPLIT) klo[p][c] = lds_read16(sOwnK + row * PQ + DK * 2 + (32 * c + 8 * g) * 2);
+    }
 #pragma unroll
     for (int c = 0; c < VC; c++) vf[p][c] = lds_read16(sOwnV + row * PV + (32 * c + 8 * g) * 2);
   }
@@ -176,7 +182,7 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
       for (int ri = 0; ri < nr; ri++) {
         const int64_t row_tok0 = (int64_t)(kr0 + ri) * G.XLq + cx0;
         auto tok = [&](int xi) { return cx0 + xi < G.XLq ? row_tok0 + xi : (int64_t)-1; };
-        stage_tile<TIO, CT, DK>(sQ + ri * CX * PQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, stage_w, tok, fwd_rope, tid);
+        stage_tile_qk<TIO, CT, DK>(sQ + ri * CX * PQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, stage_w, tok, fwd_rope, tid);
         stage_tile<TIO, CT, DV>(sDO + ri * CX * PV, PV, dob, tok_addr(a.dos, a.p.tm), a.dos[3], a.p.dv, a.do_vec != 0, stage_w, tok, no_rope, tid);
         stage_scalars(sLse + ri * CX, lseb, a.ls[2], stage_w, tok, tid);
         stage_scalars(sDel + ri * CX, delb, a.ls[2], stage_w, tok, tid);
@@ -189,12 +195,15 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
         for (int kx0 = kstart; kx0 < kend; kx0 += 32) {
           if (kx0 + 32 <= wxlo) continue;
           const int kb = ri * CX + (kx0 - cx0);
-          u32x4 qa[2][KC], da[2][VC];
+          u32x4 qa[2][KC], ql[SPLIT ? 2 : 1][KC], da[2][VC];
           float lq[8], dq_[8];
 #pragma unroll
           for (int mb = 0; mb < 2; mb++) {
 #pragma unroll
-            for (int c = 0; c < KC; c++) qa[mb][c] = lds_read16(sQ + (kb + 16 * mb + n) * PQ + (32 * c + 8 * g) * 2);
+            for (int c = 0; c < KC; c++) {
+              qa[mb][c] = lds_read16(sQ + (kb + 16 * mb + n) * PQ + (32 * c + 8 * g) * 2);
+              if constexpr (SPLIT) ql[mb][c] = lds_read16(sQ + (kb + 16 * mb + n) * PQ + DK * 2 + (32 * c + 8 * g) * 2);
+            }
 #pragma unroll
             for (int c = 0; c < VC; c++) da[mb][c] = lds_read16(sDO + (kb + 16 * mb + n) * PV + (32 * c + 8 * g) * 2);
 #pragma unroll
@@ -212,7 +221,13 @@ __global__ __launch_bounds__(256) void attn_bwd_kv_kernel(const BwdArgs a) {
               s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
               dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-              for (int c = 0; c < KC; c++) s[mb] = Mma<CT>::mfma(qa[mb][c], kf[p][c], s[mb]);
+              for (int c = 0; c < KC; c++) {
+                if constexpr (SPLIT) {   // same order as the forward kernel: lo * hi, hi * lo, hi * hi
+                  s[mb] = Mma<CT>::mfma(qa[mb][c], klo[p][c], s[mb]);
+                  s[mb] = Mma<CT>::mfma(ql[mb][c], kf[p][c], s[mb]);
+                }
+                s[mb] = Mma<CT>::mfma(qa[mb][c], kf[p][c], s[mb]);
+              }
 #pragma unroll
               for (int c = 0; c < VC; c++) dp[mb] = Mma<CT>::mfma(da[mb][c], vf[p][c], dp[mb]);
             }
@@ -254,7 +269,8 @@ template <typename TIO, int DK, int DV, int NP>
 __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   extern __shared__ __align__(16) char smem[];
-  constexpr int PQ = DK * 2 + 16, PV = DV * 2 + 16;
+  constexpr bool SPLIT = sizeof(TIO) == 4;   // see the dK / dV kernel
+  constexpr int PQ = DK * (SPLIT ? 4 : 2) + 16, PV = DV * 2 + 16;
   constexpr int OWN = 64 * NP;
   constexpr int KC = DK / 32, VC = DV / 32, KB = DK / 16;
 
@@ -282,18 +298,21 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
   RopeDev inv_rope = a.p.rope;  inv_rope.inverse = 1;
   RopeDev no_rope = a.p.rope;   no_rope.enabled = 0;
 
-  stage_tile<TIO, CT, DK>(sOwnQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, OWN,
+  stage_tile_qk<TIO, CT, DK>(sOwnQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, fwd_rope, tid);
   stage_tile<TIO, CT, DV>(sOwnDO, PV, dob, tok_addr(a.dos, a.p.tm), a.dos[3], a.p.dv, a.do_vec != 0, OWN,
                           [&](int row) { return T.own_token(row); }, no_rope, tid);
   __syncthreads();
-  u32x4 qf[NP][KC], dof[NP][VC];
+  u32x4 qf[NP][KC], qlo[SPLIT ? NP : 1][KC], dof[NP][VC];
   float lse_q[NP], del_q[NP];
 #pragma unroll
   for (int p = 0; p < NP; p++) {
     const int row = wave * 16 * NP + 16 * p + n;
 #pragma unroll
-    for (int c = 0; c < KC; c++) qf[p][c] = lds_read16(sOwnQ + row * PQ + (32 * c + 8 * g) * 2);
+    for (int c = 0; c < KC; c++) {
+      qf[p][c] = lds_read16(sOwnQ + row * PQ + (32 * c + 8 * g) * 2);
+      if constexpr (SPLIT) qlo[p][c] = lds_read16(sOwnQ + row * PQ + DK * 2 + (32 * c + 8 * g) * 2);
+    }
 #pragma unroll
     for (int c = 0; c < VC; c++) dof[p][c] = lds_read16(sOwnDO + row * PV + (32 * c + 8 * g) * 2);
     const int64_t t = T.own_token(wave * 16 * NP + 16 * p + n);
@@ -322,7 +341,7 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
       for (int ri = 0; ri < nr; ri++) {
         const int64_t row_tok0 = (int64_t)(kr0 + ri) * G.XLk + cx0;
         auto tok = [&](int xi) { return cx0 + xi < G.XLk ? row_tok0 + xi : (int64_t)-1; };
-        stage_tile<TIO, CT, DK>(sK + ri * CX * PQ, PQ, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, fwd_rope, tid);
+        stage_tile_qk<TIO, CT, DK>(sK + ri * CX * PQ, PQ, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, fwd_rope, tid);
         stage_tile<TIO, CT, DV>(sV + ri * CX * PV, PV, vb_, tok_addr(a.vs, a.p.tm), a.vs[3], a.p.dv, a.v_vec != 0, stage_w, tok, no_rope, tid);
       }
       __syncthreads();
@@ -333,11 +352,14 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
         for (int kx0 = kstart; kx0 < kend; kx0 += 32) {
           if (kx0 + 32 <= wxlo) continue;
           const int kb = ri * CX + (kx0 - cx0);
-          u32x4 ka[2][KC], va[2][VC], kt[KB];
+          u32x4 ka[2][KC], kl[SPLIT ? 2 : 1][KC], va[2][VC], kt[KB];
 #pragma unroll
           for (int mb = 0; mb < 2; mb++) {
 #pragma unroll
-            for (int c = 0; c < KC; c++) ka[mb][c] = lds_read16(sK + (kb + 16 * mb + n) * PQ + (32 * c + 8 * g) * 2);
+            for (int c = 0; c < KC; c++) {
+              ka[mb][c] = lds_read16(sK + (kb + 16 * mb + n) * PQ + (32 * c + 8 * g) * 2);
+              if constexpr (SPLIT) kl[mb][c] = lds_read16(sK + (kb + 16 * mb + n) * PQ + DK * 2 + (32 * c + 8 * g) * 2);
+            }
 #pragma unroll
             for (int c = 0; c < VC; c++) va[mb][c] = lds_read16(sV + (kb + 16 * mb + n) * PV + (32 * c + 8 * g) * 2);
           }
@@ -352,7 +374,13 @@ __global__ __launch_bounds__(256) void attn_bwd_q_kernel(const BwdArgs a) {
               s[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
               dp[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-              for (int c = 0; c < KC; c++) s[mb] = Mma<CT>::mfma(ka[mb][c], qf[p][c], s[mb]);
+              for (int c = 0; c < KC; c++) {
+                if constexpr (SPLIT) {
+                  s[mb] = Mma<CT>::mfma(kl[mb][c], qf[p][c], s[mb]);
+                  s[mb] = Mma<CT>::mfma(ka[mb][c], qlo[p][c], s[mb]);
+                }
+                s[mb] = Mma<CT>::mfma(ka[mb][c], qf[p][c], s[mb]);
+              }
 #pragma unroll
               for (int c = 0; c < VC; c++) dp[mb] = Mma<CT>::mfma(va[mb][c], dof[p][c], dp[mb]);
             }

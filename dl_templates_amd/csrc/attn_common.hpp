@@ -333,6 +333,56 @@ DLT_DEV void stage_tile(char* s, int pitch, const TIO* base, const SN& sn, int64
   }
 }
 
+// fp32 tensors whose values enter a score product: every value is staged as TWO bf16 numbers, hi = bf16(x) and
+// lo = bf16(x - hi), hi at the row's start and lo D * 2 bytes further on (row pitch >= 4 D bytes).  The products
+// hi * hi + hi * lo + lo * hi then carry x to about 16 significant bits (the reference casts these operands to fp16, 11
+// bits: src/tiled_swa.py:111-112); a single bf16 keeps 8, which shows in the softmax when the logits are large.  The
+// rotation, when fused, is applied to the fp32 values before the split.
+template <int D, typename TokFn, typename SN>
+DLT_DEV void stage_tile_split(char* s, int pitch, const float* base, const SN& sn, int64_t sd, int dact, bool vec, int nrows,
+                              TokFn tok, const RopeDev& rope, int tid) {
+  constexpr int CH = D / 8;
+  constexpr int RSTEP = 256 / CH;
+  const int c = tid % CH;
+  const RopeChunk rc = rope_chunk_setup(rope, c, vec);
+  const int nvalid = dlt_imin(8, dact - 8 * c);
+  auto load8f = [&](const float* p, int nv, float* f) {
+    if (vec) {
+      const float4 a = reinterpret_cast<const float4*>(p)[0], b = reinterpret_cast<const float4*>(p)[1];
+      f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; j++) f[j] = j < nv ? p[j * sd] : 0.f;
+    }
+  };
+  for (int row = tid / CH; row < nrows; row += RSTEP) {
+    const int64_t t = tok(row);
+    float self[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (t >= 0 && nvalid > 0) {
+      const float* p = base + tok_offset(sn, t);
+      load8f(p + (int64_t)8 * c * sd, nvalid, self);
+      if (rc.mode != 0) {
+        float partner8[8];
+        if (rc.mode == 1) load8f(p + (int64_t)8 * rc.partner_c * sd, 8, partner8);
+        rope_apply8(rope, rc, c, rope.idx[t], self, partner8, [&](int d) { return p[(int64_t)d * sd]; });
+      }
+    }
+    float lo[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) lo[j] = self[j] - (float)(bf16_t)self[j];
+    lds_write16(s + row * pitch + c * 16, pack8<bf16_t>(self));
+    lds_write16(s + row * pitch + D * 2 + c * 16, pack8<bf16_t>(lo));
+  }
+}
+
+// q / k tiles: plain staging, or the hi + lo pair for fp32 tensors (row pitch DK * 4 + 16 then)
+template <typename TIO, typename CT, int D, typename TokFn, typename SN>
+DLT_DEV void stage_tile_qk(char* s, int pitch, const TIO* base, const SN& sn, int64_t sd, int dact, bool vec, int nrows,
+                           TokFn tok, const RopeDev& rope, int tid) {
+  if constexpr (sizeof(TIO) == 4) stage_tile_split<D>(s, pitch, base, sn, sd, dact, vec, nrows, tok, rope, tid);
+  else stage_tile<TIO, CT, D>(s, pitch, base, sn, sd, dact, vec, nrows, tok, rope, tid);
+}
+
 // ---- LDS -> HBM store of an output tile ------------------------------------------------------
 // TL: element type of the LDS tile (the output type, or float for fp32 outputs).
 template <typename TO, typename TL, int D, typename TokFn, typename SN>

@@ -29,7 +29,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   typedef typename ComputeOf<TIO>::type CT;
   typedef typename TileOf<TIO>::type TL;
   extern __shared__ __align__(16) char smem[];
-  constexpr int PQ = DK * 2 + 16, PK = DK * 2 + 16, PV = DV * 2 + 16;
+  // fp32 tensors: q and k are staged as hi + lo bf16 pairs (stage_tile_split) and a score is three products
+  constexpr bool SPLIT = sizeof(TIO) == 4;
+  constexpr int PQ = DK * (SPLIT ? 4 : 2) + 16, PK = PQ, PV = DV * 2 + 16;
   constexpr int PO = DV * (int)sizeof(TL) + 16;
   constexpr int OWN = 64 * NP;
   constexpr int KC = DK / 32, VB = DV / 16;
@@ -56,14 +58,17 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
   no_rope.enabled = 0;
 
   // ---- own queries -> LDS -> B-operand fragments
-  stage_tile<TIO, CT, DK>(sQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, OWN,
-                          [&](int row) { return T.own_token(row); }, a.p.rope, tid);
+  stage_tile_qk<TIO, CT, DK>(sQ, PQ, qb, tok_addr(a.qs, a.p.tm), a.qs[3], a.p.dk, a.q_vec != 0, OWN,
+                             [&](int row) { return T.own_token(row); }, a.p.rope, tid);
   __syncthreads();
-  u32x4 qf[NP][KC];
+  u32x4 qf[NP][KC], qlo[SPLIT ? NP : 1][KC];
 #pragma unroll
   for (int p = 0; p < NP; p++)
 #pragma unroll
-    for (int c = 0; c < KC; c++) qf[p][c] = lds_read16(sQ + (wave * 16 * NP + 16 * p + n) * PQ + (32 * c + 8 * g) * 2);
+    for (int c = 0; c < KC; c++) {
+      qf[p][c] = lds_read16(sQ + (wave * 16 * NP + 16 * p + n) * PQ + (32 * c + 8 * g) * 2);
+      if constexpr (SPLIT) qlo[p][c] = lds_read16(sQ + (wave * 16 * NP + 16 * p + n) * PQ + DK * 2 + (32 * c + 8 * g) * 2);
+    }
 
   float m_run[NP], l_run[NP];
   f32x4 acc[NP][VB];
@@ -89,7 +94,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
       for (int ri = 0; ri < nr; ri++) {
         const int64_t row_tok0 = (int64_t)(kr0 + ri) * G.XLk + cx0;
         auto tok = [&](int xi) { return cx0 + xi < G.XLk ? row_tok0 + xi : (int64_t)-1; };
-        stage_tile<TIO, CT, DK>(sK + ri * CX * PK, PK, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, a.p.rope, tid);
+        stage_tile_qk<TIO, CT, DK>(sK + ri * CX * PK, PK, kb_, tok_addr(a.ks, a.p.tm), a.ks[3], a.p.dk, a.k_vec != 0, stage_w, tok, a.p.rope, tid);
         stage_tile<TIO, CT, DV>(sV + ri * CX * PV, PV, vb_, tok_addr(a.vs, a.p.tm), a.vs[3], a.p.dv, a.v_vec != 0, stage_w, tok, no_rope, tid);
       }
       __syncthreads();
@@ -101,11 +106,14 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
         for (int kx0 = kstart; kx0 < kend; kx0 += 32) {
           if (kx0 + 32 <= wxlo) continue;
           const int kb = ri * CX + (kx0 - cx0);
-          u32x4 ka[2][KC], vt[VB];
+          u32x4 ka[2][KC], kl[SPLIT ? 2 : 1][KC], vt[VB];
 #pragma unroll
           for (int mb = 0; mb < 2; mb++)
 #pragma unroll
-            for (int c = 0; c < KC; c++) ka[mb][c] = lds_read16(sK + (kb + 16 * mb + n) * PK + (32 * c + 8 * g) * 2);
+            for (int c = 0; c < KC; c++) {
+              ka[mb][c] = lds_read16(sK + (kb + 16 * mb + n) * PK + (32 * c + 8 * g) * 2);
+              if constexpr (SPLIT) kl[mb][c] = lds_read16(sK + (kb + 16 * mb + n) * PK + DK * 2 + (32 * c + 8 * g) * 2);
+            }
 #pragma unroll
           for (int d = 0; d < VB; d++) vt[d] = lds_read_tokens_as_k(sV, PV, kb, 16 * d, n, g);
 
@@ -115,6 +123,12 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
             f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < KC; c++) {
+              if constexpr (SPLIT) {   // the small terms first
+                s0 = Mma<CT>::mfma(kl[0][c], qf[p][c], s0);
+                s1 = Mma<CT>::mfma(kl[1][c], qf[p][c], s1);
+                s0 = Mma<CT>::mfma(ka[0][c], qlo[p][c], s0);
+                s1 = Mma<CT>::mfma(ka[1][c], qlo[p][c], s1);
+              }
               s0 = Mma<CT>::mfma(ka[0][c], qf[p][c], s0);
               s1 = Mma<CT>::mfma(ka[1][c], qf[p][c], s1);
             }

@@ -511,7 +511,8 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
   if (flash_eligible(p, t, false)) return flash_forward(p, t, dc, stream);
   const int np = (p.g.mode == DLT_GEOM_SWA || dc.id == 4) ? 1 : 2;
   const int own = 64 * np;
-  const int PQ = dc.DK * 2 + 16, PK = dc.DK * 2 + 16, PV = dc.DV * 2 + 16, PO = dc.DV * es + 16;
+  // fp32 tensors: q and k rows are staged as hi + lo bf16 pairs (must match SPLIT in attn_fwd_kernel.hpp)
+  const int PQ = dc.DK * (p.dtype == DLT_FP32 ? 4 : 2) + 16, PK = PQ, PV = dc.DV * 2 + 16, PO = dc.DV * es + 16;
   FwdArgs a;
   a.p = p;
   rc = make_plan(p, own, own * (PQ > PO ? PQ : PO), PK + PV, p.g.XLq, p.g.XLk, a.plan);
@@ -579,7 +580,8 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
   if (flash_eligible(p, t, true)) return flash_backward(p, t, dc, stream);
   const int np = 1;
   const int own = 64 * np;
-  const int PQ = dc.DK * 2 + 16, PV = dc.DV * 2 + 16;
+  // fp32 tensors: q and k rows are staged as hi + lo bf16 pairs (must match SPLIT in attn_bwd_kernel.hpp)
+  const int PQ = dc.DK * (p.dtype == DLT_FP32 ? 4 : 2) + 16, PV = dc.DV * 2 + 16;
   const int tile_k = dc.DK * es + 16, tile_v = dc.DV * es + 16;
   int own_bytes = own * (PQ + PV);
   if (own * tile_k > own_bytes) own_bytes = own * tile_k;

@@ -29,7 +29,9 @@ extern "C" {
 #define DLT_ERR_LAUNCH 3      /* the HIP runtime reported an error on launch    */
 
 /* element type of q/k/v/o and their gradients; arithmetic is bf16 (fp16 for DLT_FP16)
- * MFMA with fp32 accumulation, fp32 inputs are rounded to bf16 when staged. */
+ * MFMA with fp32 accumulation.  fp32 q and k enter the score products as hi + lo bf16 pairs
+ * (about 16 significant bits; the reference casts to fp16, src/tiled_swa.py:111-112), fp32 v
+ * and dO are rounded to bf16 when staged. */
 typedef enum { DLT_BF16 = 0, DLT_FP16 = 1, DLT_FP32 = 2 } dlt_dtype_t;
 
 const char* dlt_last_error(void);

@@ -298,9 +298,10 @@ def test_bad_arguments_raise():
 
 
 def test_gradients_that_cancel_stay_zero_with_fp32_inputs():
-    """A query that sees a single key has p = 1 and dS = dP - delta = 0, so dq = dk = 0.  fp32 operands are rounded
-    to bf16 on load: delta is formed from the same rounded dO as dP, or the difference of the two roundings
-    (about 1e-1 at head dim 256) would show up as a gradient."""
+    """A query that sees a single key has p = 1 and dS = dP - delta = 0, so dq = dk = 0.  fp32 operands of the second
+    products are rounded to bf16 on load: delta is formed from the same rounded dO as dP, or the difference of the two
+    roundings (about 1e-1 at head dim 256) would show up as a gradient; and the backward kernels recompute the scores from
+    the same hi + lo pairs as the forward kernel, so p is 1 and not exp of a rounding difference."""
     fa = _fa()
     q, k, v, do = orc.make_qkv(31, 2, 2, 200, 1, 120, 256, torch.float32)
     qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))

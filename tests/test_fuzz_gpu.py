@@ -148,10 +148,8 @@ def _other_strides(t, mode):
 
 
 def _make(seed, B, H, Lq, Lk, dk, dv, dt):
-    q, k, v, do = orc.make_qkv(seed, B, H, Lq, Lk, dk, dv, dt)
-    if dt == torch.float32:   # the kernels round fp32 operands to bf16 on load: compare on values that survive it
-        q, k, v, do = (t.bfloat16().float() for t in (q, k, v, do))
-    return q, k, v, do
+    # raw N(0, 1) draws in every element type: fp32 tensors enter the score products as hi + lo bf16 pairs
+    return orc.make_qkv(seed, B, H, Lq, Lk, dk, dv, dt)
 
 
 def test_random_head_dims_strides_and_scales_sliding_window():
@@ -225,3 +223,43 @@ def test_random_head_dims_strides_and_scales_flash():
         assert o.shape == (B, H, Lq, dv) and o.dtype == dt, tag
         assert qg.grad.shape == q.shape and kg.grad.shape == k.shape and vg.grad.shape == v.shape, tag
         _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
+
+
+# fp32 tensors with raw N(0, 1) values, sm_scale 0.3 and head dims of 72 and more: logits of 10 and beyond, where one
+# bf16 rounding of q and k moved the forward result by 2e-2 ... 5e-2 (the reference casts to fp16, src/tiled_swa.py:111-112).
+FP32_SWA = [(16, 2, 6, 1, 1, 96, 96, 2, 1, False, 8, 0), (1, 5, 29, 5, 4, 120, 120, 1, 2, True, 4, 0), (1, 9, 14, 3, 12, 80, 112, 1, 2, False, 8, 1),
+            (1, 7, 11, 2, 2, 128, 128, 2, 1, True, 16, 2)]
+FP32_FLASH = [(True, 127, 127, 96, 256, 1, 1, 1), (False, 511, 900, 256, 128, 2, 2, 0), (True, 64, 64, 72, 100, 2, 2, 1),
+              (False, 700, 64, 200, 200, 2, 3, 0), (True, 64, 64, 72, 72, 2, 3, 2), (False, 129, 900, 136, 136, 1, 2, 0)]
+
+
+@pytest.mark.parametrize("S,th,tw,WR,WC,d,dv,B,H,use_rope,R,mode", FP32_SWA)
+def test_fp32_raw_values_large_logits_sliding_window(S, th, tw, WR, WC, d, dv, B, H, use_rope, R, mode):
+    from dl_templates_amd import tiled_swa as sw
+    N, scale, dt = th * tw * S, 0.3, torch.float32
+    tag = f"S={S} grid={th}x{tw} W=({WR},{WC}) d={d}/{dv} B={B} H={H} rope={use_rope} R={R} strides={mode}"
+    q, k, v, do = orc.make_qkv(d + th, B, H, N, N, d, dv, dt)
+    qg, kg, vg = (_other_strides(t, mode).detach().requires_grad_(True) for t in (q, k, v))
+    if use_rope:
+        idx = orc.make_rope_idx(3, th, tw, 0.1)
+        rcs, ccs = orc.rope_tables(R, th), orc.rope_tables(R, tw)
+        o_w, dq_w, dk_w, dv_w = orc.rope_swa_grads(q, k, v, do, idx, rcs, ccs, 1, th, tw, WR, WC, scale)
+        o = sw.TiledSwaRope.apply(qg, kg, vg, idx.cuda(), rcs.cuda(), ccs.cuda(), 1, th, tw, WR, WC, scale)
+    else:
+        o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q, k, v, do, S, th, tw, WR, WC, scale)
+        o = sw.TiledSwa.apply(qg, kg, vg, S, th, tw, WR, WC, scale)
+    o.backward(do.cuda())
+    _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
+
+
+@pytest.mark.parametrize("causal,Lq,Lk,dk,dv,B,H,mode", FP32_FLASH)
+def test_fp32_raw_values_large_logits_flash(causal, Lq, Lk, dk, dv, B, H, mode):
+    from dl_templates_amd import flash_attn as fa
+    scale, dt = 0.3, torch.float32
+    tag = f"causal={causal} L=({Lq},{Lk}) d={dk}/{dv} B={B} H={H} strides={mode}"
+    q, k, v, do = orc.make_qkv(dk + Lq, B, H, Lq, Lk, dk, dv, dt)
+    o_w, dq_w, dk_w, dv_w = orc.flash_grads(q, k, v, do, causal, scale)
+    qg, kg, vg = (_other_strides(t, mode).detach().requires_grad_(True) for t in (q, k, v))
+    o = fa.attention(qg, kg, vg, causal, scale)
+    o.backward(do.cuda())
+    _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
