@@ -243,21 +243,22 @@ class FlashWorkload:
 
 
 # ------------------------------------------------------------------------------------------ RoPE
-def bench_rope(steps, warmup):
-    """Config 2: B=4, H=8, 64x64, d=64, first 32 dims rotated, 5% no-PE, q and k in one launch.
+def bench_rope(steps, warmup, R=8):
+    """Config 2 (R = 8): B=4, H=8, 64x64, d=64, first 32 dims rotated, 5% no-PE, q and k in one launch.
     `cold` cycles through > 512 MB of distinct (q, k) pairs so that the 256 MB infinity cache
-    cannot hold the working set; `hot` reuses one pair."""
+    cannot hold the working set; `hot` reuses one pair.  R = 16 is the same launch with the whole 64-dim row rotated:
+    every byte of a fetched 128-byte line is used, so algorithmic and real traffic coincide."""
     from dl_templates_amd import _lib
     from dl_templates_amd.rope2d import FusedRotaryPositionEncodingContext as Ctx
     from dl_templates_amd.fused_rope2d import FusedInplaceRotaryPositionEncoding2D as Rope
     dev = torch.device("cuda:0")
-    B, H, N, C, R = 4, 8, 4096, 64, 8
+    B, H, N, C = 4, 8, 4096, 64
     g = torch.Generator().manual_seed(2)
     idx = Rope.encode_idx(64, 64).clone()
     idx[torch.rand(N, generator=g) < 0.05] = -1
     n_pe = int((idx >= 0).sum())
     idx = idx.to(dev)
-    rcs, ccs = Ctx(16, 64).cs_components.to(dev), Ctx(16, 64).cs_components.to(dev)
+    rcs, ccs = Ctx(2 * R, 64).cs_components.to(dev), Ctx(2 * R, 64).cs_components.to(dev)
     desc, keep = _lib.rope_desc(idx, rcs, ccs)
     lib = _lib.load()
     nbuf = 17  # 17 * 2 * 16.8 MB = 570 MB
@@ -281,13 +282,21 @@ def bench_rope(steps, warmup):
 
     # algorithmic bytes: read + write of the 4R rotated dims of tokens with a rotated axis, idx once, x2 tensors
     alg_bytes = 2 * (2 * 2 * (B * H) * n_pe * 4 * R) + 4 * N
-    out = {"alg_bytes": alg_bytes, "n_pe_tokens": n_pe}
+    # real traffic: reads fetch whole 128-byte lines, writes carry the bytes stored.  With R = 8 only the first 64 bytes of
+    # each 128-byte token row rotate, so a rotated token costs 128 bytes read + 64 written = 1.5 x its algorithmic bytes
+    # (the counters in profiles/ read 1.56 x for the launch, tables and idx included); with 4 R = C the two coincide
+    real_bytes = 2 * (2 * (B * H) * n_pe * (max(C, 4 * R) + 4 * R)) + 4 * N
+    line_factor = real_bytes / alg_bytes
+    out = {"alg_bytes": alg_bytes, "n_pe_tokens": n_pe, "rotary_pairs_per_axis": R,
+           "real_bytes_over_alg_bytes": line_factor}
     for name, fn in (("cold", cold), ("hot", hot)):
         ms_ev, _ = Timer.run(fn, steps * 5, warmup * 5)
         kb = kernel_breakdown(fn, steps * 5)
         kms = kb["rope2d"]["avg_ms"]
         out[name] = {"us_per_launch_back_to_back": ms_ev * 1e3, "us_kernel_events": kms * 1e3,
-                     "gbps": alg_bytes / (kms * 1e-3) / 1e9, "frac_of_hbm_peak": alg_bytes / (kms * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+                     "gbps": alg_bytes / (kms * 1e-3) / 1e9, "frac_of_hbm_peak": alg_bytes / (kms * 1e-3) / 1e9 / PEAK_HBM_GBPS,
+                     "gbps_back_to_back": alg_bytes / (ms_ev * 1e-3) / 1e9,
+                     "real_traffic_gbps_back_to_back": alg_bytes * line_factor / (ms_ev * 1e-3) / 1e9}
     del keep
     return out
 
@@ -540,7 +549,15 @@ def main():
 
     rope = bench_rope(K, W)
     extra["rope2d_c2"] = rope
+    extra["rope2d_whole_row_r16"] = bench_rope(K, W, R=16)
     extra["copy_bandwidth"] = copy_bandwidth()
+    # the rotation against what a plain copy sustains on this box: real traffic of a cold launch over the 1 GiB copy rate
+    # (HBM, far beyond the caches) and over a cold copy of the launch's own size
+    cb = extra["copy_bandwidth"]
+    for key in ("rope2d_c2", "rope2d_whole_row_r16"):
+        r_ = extra[key]["cold"]
+        r_["frac_of_1GiB_copy_rate"] = r_["real_traffic_gbps_back_to_back"] / cb["1GiB_hbm"]["gbps_read_plus_write"]
+        r_["frac_of_cold_copy_of_same_size"] = r_["real_traffic_gbps_back_to_back"] / cb["24MiB_cold"]["gbps_read_plus_write"]
 
     # the extra configs: long enough runs (tens of milliseconds of GPU time behind a warm-up) that the clock ramp after an
     # idle phase does not weigh on the mean
