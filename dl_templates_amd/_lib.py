@@ -27,8 +27,9 @@ EXPORTS = (
     "dlt_swa_fwd", "dlt_swa_bwd", "dlt_swa_neighbors", "dlt_flash_fwd", "dlt_flash_bwd",
     "dlt_timing_enable", "dlt_timing_collect", "dlt_debug_copy",
     "dlt_swa_fwd_image", "dlt_swa_bwd_image", "dlt_swa_image_offsets", "dlt_swa_fwd_rot", "dlt_swa_bwd_rot",
-    "dlt_swa_bwd_noalloc",
+    "dlt_swa_bwd_noalloc", "dlt_dry_run", "dlt_last_kernel_family",
 )
+KERNEL_FAMILIES = ("none", "marching", "streaming", "tile", "flash", "generic")   # DLT_FAMILY_* of include/dlt.h
 NOALLOC_MAX_DELTA = 1 << 20  # DLT_NOALLOC_MAX_DELTA of include/dlt.h
 KERNEL_NAMES = ("rope2d", "attn_fwd", "attn_delta", "attn_bwd_kv", "attn_bwd_q")
 
@@ -131,6 +132,10 @@ def _declare(lib) -> None:
     lib.dlt_timing_enable.argtypes = [c_int]
     lib.dlt_timing_collect.restype = c_int
     lib.dlt_timing_collect.argtypes = [POINTER(KernelTime), c_int, POINTER(c_int)]
+    lib.dlt_dry_run.restype = c_int
+    lib.dlt_dry_run.argtypes = [c_int]
+    lib.dlt_last_kernel_family.restype = c_int
+    lib.dlt_last_kernel_family.argtypes = []
 
 
 def load():

@@ -309,6 +309,16 @@ int dlt_ensure_lds(const void* kern, int bytes) {
   return DLT_OK;
 }
 
+namespace {
+thread_local int g_family = DLT_FAMILY_NONE;
+thread_local bool g_dry = false;
+}  // namespace
+bool dlt_route_note(int family) { g_family = family; return g_dry; }
+bool dlt_route_dry() { return g_dry; }
+void dlt_route_reset() { g_family = DLT_FAMILY_NONE; }
+extern "C" int dlt_dry_run(int on) { g_dry = on != 0; return DLT_OK; }
+extern "C" int dlt_last_kernel_family(void) { return g_family; }
+
 int dlt_device_cus() {
   constexpr int MAXDEV = 64;
   static std::mutex mu;

@@ -177,6 +177,7 @@ bool swa1_strides_fit(const AttnProblem& p, const AttnTensors& t) {
 }
 
 int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c_in, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_TILE)) return DLT_OK;
   Swa1Class c = c_in;
   if (p.rope_prerot && c.rope_mode != 0) c.rope_mode = 3;  // rotated q, k: plain tile loads, gradients rotated back on store
   const int es = dlt_elem_size(p.dtype);
@@ -228,6 +229,7 @@ int swa1_backward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c
 }
 
 int swa1_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_TILE)) return DLT_OK;
   const int es = dlt_elem_size(p.dtype);
   Swa1FwdArgs a;
   a.p = p;
@@ -274,6 +276,7 @@ void swam_make_plan(const AttnProblem& p, SwamPlan& plan) {
 }
 
 int swam_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_MARCHING)) return DLT_OK;
   SwamFwdArgs a;
   a.p = p;
   swam_make_plan(p, a.plan);
@@ -309,6 +312,7 @@ bool swa2_rows_ok(const AttnProblem& p, const void* ptr, const int64_t* st) {
 }
 
 int swa2_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_STREAMING)) return DLT_OK;
   Swa2FwdArgs a;
   a.p = p;
   swa2_make_plan(p, a.plan);
@@ -322,6 +326,7 @@ int swa2_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream)
 }
 
 int swa2_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_STREAMING)) return DLT_OK;
   Swa2BwdArgs a;
   a.p = p;
   swa2_make_plan(p, a.plan);
@@ -340,6 +345,7 @@ int swa2_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream
 
 // backward on the marching kernels: plain inputs, or rotated inputs with the gradients rotated back on store
 int swam_backward(const AttnProblem& p, const AttnTensors& t, bool rot, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_MARCHING)) return DLT_OK;
   SwamBwdArgs a;
   a.p = p;
   swam_make_plan(p, a.plan);
@@ -384,6 +390,7 @@ bool flash_eligible(const AttnProblem& p, const AttnTensors& t, bool with_do) {
 }
 
 int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_FLASH)) return DLT_OK;
   FlashArgs a;
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
   for (int i = 0; i < 5; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
@@ -411,6 +418,7 @@ int flash_forward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc
 }
 
 int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& dc, hipStream_t stream) {
+  if (dlt_route_note(DLT_FAMILY_FLASH)) return DLT_OK;
   BwdArgs d;
   d.p = p;
   d.o = t.o; d.d_o = t.d_o; d.delta = t.delta;
@@ -472,6 +480,7 @@ int flash_backward(const AttnProblem& p, const AttnTensors& t, const DimClass& d
 }  // namespace
 
 int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
+  dlt_route_reset();
   DimClass dc;
   int rc = pick_dims(p, dc);
   if (rc != DLT_OK) return rc;
@@ -509,6 +518,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
     return dlt_attn_forward(p2, t2, stream);
   }
   if (flash_eligible(p, t, false)) return flash_forward(p, t, dc, stream);
+  if (dlt_route_note(DLT_FAMILY_GENERIC)) return DLT_OK;
   const int np = (p.g.mode == DLT_GEOM_SWA || dc.id == 4) ? 1 : 2;
   const int own = 64 * np;
   // fp32 tensors: q and k rows are staged as hi + lo bf16 pairs (must match SPLIT in attn_fwd_kernel.hpp)
@@ -539,6 +549,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
 }
 
 int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
+  dlt_route_reset();
   DimClass dc;
   int rc = pick_dims(p, dc);
   if (rc != DLT_OK) return rc;
@@ -578,6 +589,7 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
     return dlt_rope_inplace_4d(t.dk, t.dks, p.B, p.H, (int64_t)p.g.TR * p.g.XLk, p.dk, &r, 1, p.dtype, stream);
   }
   if (flash_eligible(p, t, true)) return flash_backward(p, t, dc, stream);
+  if (dlt_route_note(DLT_FAMILY_GENERIC)) return DLT_OK;
   const int np = 1;
   const int own = 64 * np;
   // fp32 tensors: q and k rows are staged as hi + lo bf16 pairs (must match SPLIT in attn_bwd_kernel.hpp)

@@ -14,6 +14,11 @@ int dlt_set_error(int code, const char* fmt, ...) __attribute__((format(printf, 
 // size than any before is asked for (per kernel and device): it costs tens of microseconds of host time, which would
 // otherwise sit in front of every launch.
 int dlt_ensure_lds(const void* kern, int bytes);
+// Routing record of the calling thread: every attention launch path notes its kernel family (DLT_FAMILY_*) here first.
+// Returns true under dlt_dry_run(1): the caller then returns DLT_OK without launching anything.
+bool dlt_route_note(int family);
+bool dlt_route_dry();
+void dlt_route_reset();
 // compute units of the current device (asked once per device; 256 when the query fails)
 int dlt_device_cus();
 

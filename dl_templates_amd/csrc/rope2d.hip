@@ -295,6 +295,7 @@ int rope_impl(void* const x[2], const int64_t* const st[2], const int64_t nb[2],
 
 int dlt_rope_rotate_copy(const void* src, const int64_t* ss, void* dst, const int64_t* ds, int B, int H, int64_t N, int C,
                          const RopeDev& rope, int dtype, hipStream_t stream) {
+  if (dlt_route_dry()) return DLT_OK;
   RopeCopyArgs a;
   a.src = src; a.dst = dst;
   for (int i = 0; i < 4; i++) { a.ss[i] = ss[i]; a.ds[i] = ds[i]; }
@@ -331,6 +332,7 @@ int dlt_rope_rotate_copy(const void* src, const int64_t* ss, void* dst, const in
 // when (B, H) collapses into one batch stride, else one per b.
 int dlt_rope_inplace_4d(void* x, const int64_t* st, int B, int H, int64_t N, int C, const dlt_rope_t* rope, int inverse,
                         int dtype, hipStream_t stream) {
+  if (dlt_route_dry()) return DLT_OK;
   const bool flat = B == 1 || st[0] == (int64_t)H * st[1];
   const int64_t s3[3] = {st[1], st[2], st[3]};
   const int es = dlt_elem_size(dtype);

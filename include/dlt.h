@@ -251,6 +251,23 @@ typedef struct {
  * FETCH_SIZE / WRITE_SIZE counters report per byte.  No counterpart in the reference. */
 int dlt_debug_copy(void* dst, const void* src, int64_t bytes, void* stream);
 
+/* Which kernel family an attention call runs on.  No counterpart in the reference (Triton picks a configuration by
+ * autotuning, src/tiled_swa.py:570-573); here the host routes every call by shape, element type, strides and
+ * alignment, and a C caller cannot see from the outside that, say, head dim 80 or a 23-column window lands on the
+ * generic kernels (several times slower than the tuned ones).  dlt_last_kernel_family() returns the family the calling
+ * thread's latest forward / backward call (dlt_swa_*, dlt_flash_*) was routed to.  With dlt_dry_run(1) (per thread) those
+ * calls validate their arguments and route, but launch nothing and touch no memory: pointers only need the alignment
+ * of the real ones, so the query also works in a process without a GPU.
+ *   MARCHING  token grids (b_size 1), head dim 64, windows up to 13 x 13 (rotation: 8 rotary pairs, rotated q / k kept)
+ *   STREAMING token grids, head dim 64 / 128, windows up to 21 columns, no rotation
+ *   TILE      token grids, head dims in multiples of 32 up to 128, windows up to 21 columns (rotation in the tile loads)
+ *   FLASH     dense / causal / tiles of 16 k tokens, 2-byte element types, head dims up to 128 (multiples of 8)
+ *   GENERIC   everything else */
+enum { DLT_FAMILY_NONE = 0, DLT_FAMILY_MARCHING = 1, DLT_FAMILY_STREAMING = 2, DLT_FAMILY_TILE = 3, DLT_FAMILY_FLASH = 4,
+       DLT_FAMILY_GENERIC = 5 };
+int dlt_dry_run(int on);
+int dlt_last_kernel_family(void);
+
 int dlt_timing_enable(int on);
 int dlt_timing_collect(dlt_kernel_time_t* out, int max, int* n);
 
