@@ -116,6 +116,7 @@ int make_plan(const AttnProblem& p, int own, int own_bytes, int per_tok, int XL_
 
 // ---- token-grid (b_size == 1) fast path ----------------------------------------------------
 struct Swa1Class { int D, wclass, pbit, rope_mode; };
+constexpr int SWA2_MAX_PASSES = 4;   // column passes of the streaming kernels: windows up to 93 columns
 
 // Can the token-grid kernels take this problem?  They need 16-byte vector access to the
 // streamed tensors, both head dims in one padded class, a window of at most 21 columns and,
@@ -131,9 +132,11 @@ bool swa1_eligible(const AttnProblem& p, const bool* streamed_vec, int n_streame
   for (int i = 0; i < n_streamed; i++)
     if (!streamed_vec[i]) return false;
   if ((int64_t)p.g.TR * p.g.TC >= ((int64_t)1 << 31) / 1024) return false;  // 32-bit element offsets inside a slab
+  // column groups of a wave's window: up to 4 / 6 per class; wider windows (class 2) only run on the streaming kernels,
+  // which walk them in column passes
   const int ncg = (4 + 2 * p.g.WC + 3) / 4;
-  if (ncg > 6) return false;
-  c.wclass = ncg <= 4 ? 0 : 1;
+  if (ncg > SWA2_MAX_PASSES * 6) return false;
+  c.wclass = ncg <= 4 ? 0 : ncg <= 6 ? 1 : 2;
   c.pbit = 1;
   c.rope_mode = 0;
   if (p.rope.enabled && p.rope.R > 0) {
@@ -294,12 +297,22 @@ int swam_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
 
 // ---- streaming kernels: head dim 64 or 128 exactly, no rotation, windows up to 21 columns ---------------------------
 bool swa2_eligible(const AttnProblem& p, const Swa1Class& c) {
-  return (c.D == 64 || c.D == 128) && p.dk == c.D && p.dv == c.D && c.rope_mode == 0 && p.g.WC <= 10;
+  return (c.D == 64 || c.D == 128) && p.dk == c.D && p.dv == c.D && c.rope_mode == 0;
 }
-// column groups of a wave's window: 4 x 4 columns cover windows up to 13 columns, 6 x 4 up to 21
-int swa2_ncg(const AttnProblem& p) { return p.g.WC <= 6 ? 4 : 6; }
+// Kernel class (column groups of a wave's window per pass: 4 x 4 columns cover windows up to 13 columns, 6 x 4 up to 21)
+// and number of column passes.  Wider windows take the split that computes the fewest groups (7 groups: 2 passes of 4,
+// not 2 of 6), the larger class on a tie (fewer passes).
+void swa2_split(const AttnProblem& p, int& ncg_class, int& npass) {
+  const int ncg = (4 + 2 * p.g.WC + 3) / 4;
+  if (ncg <= 4) { ncg_class = 4; npass = 1; return; }
+  const int n4 = (ncg + 3) / 4, n6 = (ncg + 5) / 6;
+  if (4 * n4 < 6 * n6 && n4 <= SWA2_MAX_PASSES) { ncg_class = 4; npass = n4; }
+  else { ncg_class = 6; npass = n6; }
+}
+int swa2_ncg(const AttnProblem& p) { int c, n; swa2_split(p, c, n); return c; }
 
 void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan) {
+  { int c; swa2_split(p, c, plan.npass); }
   plan.nblk_r = (p.g.TR + 7) / 8;
   plan.nblk_c = (p.g.TC + 15) / 16;
   dlt_fastdiv_make((uint32_t)(plan.nblk_r * plan.nblk_c), plan.m_bh, plan.s_bh);
@@ -499,8 +512,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
                               (t.q_rot == nullptr || (swam_rows_ok(p, t.q_rot, t.qrs) && swam_rows_ok(p, t.k_rot, t.krs)));
         if (swam_eligible(p, c) && rows_fit) return swam_forward(p, t, c, stream);
         if (swa2_eligible(p, c) && t.q_rot == nullptr && swa2_rows_ok(p, t.out_o, t.os)) return swa2_forward(p, t, stream);
-        rc = swa1_forward(p, t, c, stream);
-        if (rc != -1) return rc;
+        if (c.wclass < 2) return swa1_forward(p, t, c, stream);
       }
     }
   }
@@ -569,7 +581,7 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
       if (swa2_eligible(p, c) && swa2_rows_ok(p, t.o, t.os) && swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) &&
           swa2_rows_ok(p, t.dv, t.dvs) && t.ls[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * t.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1))
         return swa2_backward(p, t, stream);
-      return swa1_backward(p, t, c, stream);
+      if (c.wclass < 2) return swa1_backward(p, t, c, stream);
     }
   }
   if (p.rope_prerot && p.rope.enabled && p.rope.R > 0 && !p.tm.img) {

@@ -38,23 +38,24 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int pc = wave & 3, rg = wave >> 2;
-  const Swa2Geom G = swa2_geom(a.p, a.plan);
+  const Swa2Geom G0 = swa2_geom(a.p, a.plan);
 
-  const char* qb = reinterpret_cast<const char*>(a.q) + 2 * (G.b * a.qs[0] + G.h * a.qs[1]);
-  const char* kb_ = reinterpret_cast<const char*>(a.k) + 2 * (G.b * a.ks[0] + G.h * a.ks[1]);
-  const char* vb_ = reinterpret_cast<const char*>(a.v) + 2 * (G.b * a.vs[0] + G.h * a.vs[1]);
-  const char* ob = reinterpret_cast<const char*>(a.o) + 2 * (G.b * a.os[0] + G.h * a.os[1]);
-  const char* dob = reinterpret_cast<const char*>(a.d_o) + 2 * (G.b * a.dos[0] + G.h * a.dos[1]);
-  TIO* dqb = reinterpret_cast<TIO*>(a.dq) + G.b * a.dqs[0] + G.h * a.dqs[1];
-  const float* lseb = a.lse + G.b * a.ls[0] + G.h * a.ls[1];
-  float* delb = a.delta + G.b * a.ls[0] + G.h * a.ls[1];
+  const char* qb = reinterpret_cast<const char*>(a.q) + 2 * (G0.b * a.qs[0] + G0.h * a.qs[1]);
+  const char* kb_ = reinterpret_cast<const char*>(a.k) + 2 * (G0.b * a.ks[0] + G0.h * a.ks[1]);
+  const char* vb_ = reinterpret_cast<const char*>(a.v) + 2 * (G0.b * a.vs[0] + G0.h * a.vs[1]);
+  const char* ob = reinterpret_cast<const char*>(a.o) + 2 * (G0.b * a.os[0] + G0.h * a.os[1]);
+  const char* dob = reinterpret_cast<const char*>(a.d_o) + 2 * (G0.b * a.dos[0] + G0.h * a.dos[1]);
+  TIO* dqb = reinterpret_cast<TIO*>(a.dq) + G0.b * a.dqs[0] + G0.h * a.dqs[1];
+  const float* lseb = a.lse + G0.b * a.ls[0] + G0.h * a.ls[1];
+  float* delb = a.delta + G0.b * a.ls[0] + G0.h * a.ls[1];
   const float scale = a.scale_log2;
 
   // staging: waves 0-3 copy the four halo rows of K, waves 4-7 those of V
   const bool stage_k = wave < 4;
   const char* sbase = stage_k ? kb_ : vb_;
   const int ssn2 = (int)(stage_k ? a.ks[2] : a.vs[2]) * 2;
-  const uint32_t srow = (uint32_t)(G.TC * ssn2);
+  const uint32_t srow = (uint32_t)(G0.TC * ssn2);
+  Swa2Geom G = G0;   // column pass 0 (see the forward kernel)
   Swa2Stage<C> st;
   swa2_stage_init(st, G, wave, lane, ssn2);
   swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF, wave);
@@ -81,14 +82,15 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
     del_n = wave_sum4(part);
     if (g == 0 && tq >= 0) delb[(int64_t)tq * a.ls[2]] = del_n;
   }
-  const Swa2Win W = swa2_window(G, rg, pc, n);
+  const Swa2Win W0 = swa2_window(G0, rg, pc, n);
+  Swa2Win W = W0;
   Swa2Lane<C> L;
   swa2_lane_init(L, pc, n, g);
 
   f32x4 acc[VB];
 #pragma unroll
   for (int d = 0; d < VB; d++) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int ncg = (4 + 2 * G.WC + 3) >> 2;
+  int ncg = swa2_pass_ncg(G0.WC, NCG, 0);
 
   swa2_wait_copies();   // also: the own fragments have arrived
   // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
@@ -184,17 +186,28 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
     swa2_wait_copies();
     __syncthreads();
   };
-  int ch = G.ch_first;
-  for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
-  for (; ch <= act_hi; ch++) {
-    consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF, smem + ((ch + 1) & 1) * C::BUF, std::true_type{});
+  for (int pass = 0;;) {
+    int ch = G.ch_first;
+    for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
+    for (; ch <= act_hi; ch++) {
+      consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF, smem + ((ch + 1) & 1) * C::BUF, std::true_type{});
+      swa2_wait_copies();
+      __syncthreads();
+    }
+    for (; ch < G.ch_last; ch++) copy_only(ch);
+    if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
+      consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF, smem + ((G.ch_last + 1) & 1) * C::BUF, std::false_type{});
+    __syncthreads();   // every wave is done with both chunk buffers
+    if (++pass >= a.plan.npass) break;
+    // next column pass: the same rows again, 4 NCG columns further to the right
+    G = swa2_pass_geom(G0, NCG, pass);
+    W = swa2_pass_window(W0, NCG, pass);
+    ncg = swa2_pass_ncg(G0.WC, NCG, pass);
+    swa2_stage_init(st, G, wave, lane, ssn2);
+    swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF, wave);
     swa2_wait_copies();
     __syncthreads();
   }
-  for (; ch < G.ch_last; ch++) copy_only(ch);
-  if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
-    consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF, smem + ((G.ch_last + 1) & 1) * C::BUF, std::false_type{});
-  __syncthreads();
 
   swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, acc, a.p.sm_scale, dqb, a.dqs[2], G, r_p, c_p, lane);
 }
@@ -212,29 +225,30 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int pc = wave & 3, rg = wave >> 2;
-  const Swa2Geom G = swa2_geom(a.p, a.plan);
+  const Swa2Geom G0 = swa2_geom(a.p, a.plan);
 
-  const char* qb = reinterpret_cast<const char*>(a.q) + 2 * (G.b * a.qs[0] + G.h * a.qs[1]);
-  const char* kb_ = reinterpret_cast<const char*>(a.k) + 2 * (G.b * a.ks[0] + G.h * a.ks[1]);
-  const char* vb_ = reinterpret_cast<const char*>(a.v) + 2 * (G.b * a.vs[0] + G.h * a.vs[1]);
-  const char* dob = reinterpret_cast<const char*>(a.d_o) + 2 * (G.b * a.dos[0] + G.h * a.dos[1]);
-  TIO* dkb = reinterpret_cast<TIO*>(a.dk) + G.b * a.dks[0] + G.h * a.dks[1];
-  TIO* dvb = reinterpret_cast<TIO*>(a.dv) + G.b * a.dvs[0] + G.h * a.dvs[1];
-  const float* lseb = a.lse + G.b * a.ls[0] + G.h * a.ls[1];
-  const float* delb = a.delta + G.b * a.ls[0] + G.h * a.ls[1];
+  const char* qb = reinterpret_cast<const char*>(a.q) + 2 * (G0.b * a.qs[0] + G0.h * a.qs[1]);
+  const char* kb_ = reinterpret_cast<const char*>(a.k) + 2 * (G0.b * a.ks[0] + G0.h * a.ks[1]);
+  const char* vb_ = reinterpret_cast<const char*>(a.v) + 2 * (G0.b * a.vs[0] + G0.h * a.vs[1]);
+  const char* dob = reinterpret_cast<const char*>(a.d_o) + 2 * (G0.b * a.dos[0] + G0.h * a.dos[1]);
+  TIO* dkb = reinterpret_cast<TIO*>(a.dk) + G0.b * a.dks[0] + G0.h * a.dks[1];
+  TIO* dvb = reinterpret_cast<TIO*>(a.dv) + G0.b * a.dvs[0] + G0.h * a.dvs[1];
+  const float* lseb = a.lse + G0.b * a.ls[0] + G0.h * a.ls[1];
+  const float* delb = a.delta + G0.b * a.ls[0] + G0.h * a.ls[1];
   const float scale = a.scale_log2;
 
   // staging: waves 0-3 copy the four halo rows of Q and of lse2, waves 4-7 those of dO and of delta
   const bool stage_q = wave < 4;
   const char* sbase = stage_q ? qb : dob;
   const int ssn2 = (int)(stage_q ? a.qs[2] : a.dos[2]) * 2;
-  const uint32_t srow = (uint32_t)(G.TC * ssn2);
+  const uint32_t srow = (uint32_t)(G0.TC * ssn2);
+  Swa2Geom G = G0;   // column pass 0 (see the forward kernel)
   Swa2Stage<C> st;
   swa2_stage_init(st, G, wave, lane, ssn2);
   const float* scal_base = stage_q ? lseb : delb;
   const int ls2 = (int)a.ls[2];
   // lane l < HCW copies the scalar of halo column l (clamped like the rows: positions outside the grid are masked)
-  const uint32_t scal_off = (uint32_t)(swa2_scal_col(G, lane) * ls2) * 4u;
+  uint32_t scal_off = (uint32_t)(swa2_scal_col(G, lane) * ls2) * 4u;
   auto issue_scalars = [&](int ch, char* buf) {
     const int r = swa2_issue_grid_row(G, ch, wave);
     const char* row = reinterpret_cast<const char*>(scal_base) + (uint32_t)(r * G.TC * ls2) * 4u;   // wave-uniform
@@ -250,7 +264,8 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
   u32x4 kf[KC], vf[KC];
   swa2_own_frags<KC>(kf, kb_, (int)a.ks[2] * 2, tk, g);
   swa2_own_frags<KC>(vf, vb_, (int)a.vs[2] * 2, tk, g);
-  const Swa2Win W = swa2_window(G, rg, pc, n);
+  const Swa2Win W0 = swa2_window(G0, rg, pc, n);
+  Swa2Win W = W0;
   Swa2Lane<C> L;
   swa2_lane_init(L, pc, n, g);
   // scalars of the queries (halo row g, window columns 4 cg .. 4 cg + 3) of a chunk
@@ -259,7 +274,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
   f32x4 acck[VB], accv[VB];
 #pragma unroll
   for (int d = 0; d < VB; d++) { acck[d] = f32x4{0.f, 0.f, 0.f, 0.f}; accv[d] = f32x4{0.f, 0.f, 0.f, 0.f}; }
-  const int ncg = (4 + 2 * G.WC + 3) >> 2;
+  int ncg = swa2_pass_ncg(G0.WC, NCG, 0);
 
   swa2_wait_copies();
   // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
@@ -392,17 +407,30 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_kv(D)) void swa2_bwd_kv_
     swa2_wait_copies();
     __syncthreads();
   };
-  int ch = G.ch_first;
-  for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
-  for (; ch <= act_hi; ch++) {
-    consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF_KV, smem + ((ch + 1) & 1) * C::BUF_KV, std::true_type{});
+  for (int pass = 0;;) {
+    int ch = G.ch_first;
+    for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
+    for (; ch <= act_hi; ch++) {
+      consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF_KV, smem + ((ch + 1) & 1) * C::BUF_KV, std::true_type{});
+      swa2_wait_copies();
+      __syncthreads();
+    }
+    for (; ch < G.ch_last; ch++) copy_only(ch);
+    if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
+      consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF_KV, smem + ((G.ch_last + 1) & 1) * C::BUF_KV, std::false_type{});
+    __syncthreads();   // every wave is done with both chunk buffers
+    if (++pass >= a.plan.npass) break;
+    // next column pass: the same rows again, 4 NCG columns further to the right
+    G = swa2_pass_geom(G0, NCG, pass);
+    W = swa2_pass_window(W0, NCG, pass);
+    ncg = swa2_pass_ncg(G0.WC, NCG, pass);
+    swa2_stage_init(st, G, wave, lane, ssn2);
+    scal_off = (uint32_t)(swa2_scal_col(G, lane) * ls2) * 4u;
+    swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF_KV, wave);
+    issue_scalars(G.ch_first, smem + (G.ch_first & 1) * C::BUF_KV);
     swa2_wait_copies();
     __syncthreads();
   }
-  for (; ch < G.ch_last; ch++) copy_only(ch);
-  if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
-    consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF_KV, smem + ((G.ch_last + 1) & 1) * C::BUF_KV, std::false_type{});
-  __syncthreads();
 
   swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, accv, 1.f, dvb, a.dvs[2], G, r_p, c_p, lane);
   swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, acck, a.p.sm_scale, dkb, a.dks[2], G, r_p, c_p, lane);

@@ -30,13 +30,13 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
   const int lane = tid & 63, n = lane & 15, g = lane >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int pc = wave & 3, rg = wave >> 2;
-  const Swa2Geom G = swa2_geom(a.p, a.plan);
+  const Swa2Geom G0 = swa2_geom(a.p, a.plan);
 
-  const char* qb = reinterpret_cast<const char*>(a.q) + 2 * (G.b * a.qs[0] + G.h * a.qs[1]);
-  const char* kb_ = reinterpret_cast<const char*>(a.k) + 2 * (G.b * a.ks[0] + G.h * a.ks[1]);
-  const char* vb_ = reinterpret_cast<const char*>(a.v) + 2 * (G.b * a.vs[0] + G.h * a.vs[1]);
-  TIO* ob = reinterpret_cast<TIO*>(a.o) + G.b * a.os[0] + G.h * a.os[1];
-  float* lseb = a.lse + G.b * a.ls[0] + G.h * a.ls[1];
+  const char* qb = reinterpret_cast<const char*>(a.q) + 2 * (G0.b * a.qs[0] + G0.h * a.qs[1]);
+  const char* kb_ = reinterpret_cast<const char*>(a.k) + 2 * (G0.b * a.ks[0] + G0.h * a.ks[1]);
+  const char* vb_ = reinterpret_cast<const char*>(a.v) + 2 * (G0.b * a.vs[0] + G0.h * a.vs[1]);
+  TIO* ob = reinterpret_cast<TIO*>(a.o) + G0.b * a.os[0] + G0.h * a.os[1];
+  float* lseb = a.lse + G0.b * a.ls[0] + G0.h * a.ls[1];
   const int64_t os2 = a.os[2], ls2 = a.ls[2];
   const float scale = a.scale_log2;
 
@@ -44,7 +44,9 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
   const bool stage_k = wave < 4;
   const char* sbase = stage_k ? kb_ : vb_;
   const int ssn2 = (int)(stage_k ? a.ks[2] : a.vs[2]) * 2;
-  const uint32_t srow = (uint32_t)(G.TC * ssn2);
+  const uint32_t srow = (uint32_t)(G0.TC * ssn2);
+  // column pass 0 (the only one unless the window is wider than the class: swa2_pass_geom)
+  Swa2Geom G = G0;
   Swa2Stage<C> st;
   swa2_stage_init(st, G, wave, lane, ssn2);
   swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF, wave);
@@ -54,7 +56,8 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
   const int tq = (r_p + (n >> 2) < G.TR && c_p + (n & 3) < G.TC) ? (r_p + (n >> 2)) * G.TC + c_p + (n & 3) : -1;
   u32x4 qf[KC];
   swa2_own_frags<KC>(qf, qb, (int)a.qs[2] * 2, tq, g);
-  const Swa2Win W = swa2_window(G, rg, pc, n);
+  const Swa2Win W0 = swa2_window(G0, rg, pc, n);
+  Swa2Win W = W0;
   Swa2Lane<C> L;
   swa2_lane_init(L, pc, n, g);
 
@@ -64,7 +67,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
   for (int d = 0; d < VB; d++) acc[d] = f32x4{0.f, 0.f, 0.f, 0.f};
   const unsigned one2 = pack2<CT>(1.f, 1.f);
   const u32x4 ones = n == 0 ? u32x4{one2, one2, one2, one2} : u32x4{0u, 0u, 0u, 0u};
-  const int ncg = (4 + 2 * G.WC + 3) >> 2;   // column groups of the wave window that can hold a visible token
+  int ncg = swa2_pass_ncg(G0.WC, NCG, 0);   // column groups of the wave window that can hold a visible token
 
   swa2_wait_copies();   // also: the own fragments have arrived
   // the compiler does not see that wait: tell it that the own fragments are loaded, or it waits for them (and with them
@@ -168,17 +171,28 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
     swa2_wait_copies();
     __syncthreads();
   };
-  int ch = G.ch_first;
-  for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
-  for (; ch <= act_hi; ch++) {
-    consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF, smem + ((ch + 1) & 1) * C::BUF, std::true_type{});
+  for (int pass = 0;;) {
+    int ch = G.ch_first;
+    for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
+    for (; ch <= act_hi; ch++) {
+      consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF, smem + ((ch + 1) & 1) * C::BUF, std::true_type{});
+      swa2_wait_copies();
+      __syncthreads();
+    }
+    for (; ch < G.ch_last; ch++) copy_only(ch);
+    if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
+      consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF, smem + ((G.ch_last + 1) & 1) * C::BUF, std::false_type{});
+    __syncthreads();   // every wave is done with both chunk buffers
+    if (++pass >= a.plan.npass) break;
+    // next column pass: the same rows again, 4 NCG columns further to the right
+    G = swa2_pass_geom(G0, NCG, pass);
+    W = swa2_pass_window(W0, NCG, pass);
+    ncg = swa2_pass_ncg(G0.WC, NCG, pass);
+    swa2_stage_init(st, G, wave, lane, ssn2);
+    swa2_issue(st, G, G.ch_first, sbase, srow, smem + (G.ch_first & 1) * C::BUF, wave);
     swa2_wait_copies();
     __syncthreads();
   }
-  for (; ch < G.ch_last; ch++) copy_only(ch);
-  if (G.ch_last >= W.ch_lo && G.ch_last <= W.ch_hi)
-    consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF, smem + ((G.ch_last + 1) & 1) * C::BUF, std::false_type{});
-  __syncthreads();
 
   // ---- epilogue (the loop ended with a barrier: the chunk buffers are free)
   const float lt = wave_sum4(acc_l[0]);   // only row 0 of the ones operand is set: the other lane groups hold zeros

@@ -45,6 +45,7 @@ struct Swa2Cfg {
 struct Swa2Plan {
   int32_t nblk_r, nblk_c;
   uint32_t m_bh, s_bh, m_c, s_c, m_h, s_h;   // exact multiply-shift divisions by nblk_r * nblk_c, nblk_c and H
+  int32_t npass;   // column passes: a window of more than NCG column groups is walked in npass slices of NCG groups
 };
 
 struct Swa2Geom {
@@ -96,6 +97,24 @@ DLT_HD Swa2Win swa2_window(const Swa2Geom& G, int rg, int pc, int n) {
   w.ch_hi = patch_ok ? phi >> 2 : 0;
   return w;
 }
+
+// Windows wider than the class (more than NCG column groups per wave) are walked in column passes: pass s covers the
+// window columns 4 NCG s .. 4 NCG (s + 1) - 1 of every wave.  Everything that addresses columns sees a pass through a
+// geometry whose column half-width is reduced by the pass's offset (halo column 0 of the pass = grid column
+// c0 - WC + 4 NCG s) and a window whose first visible column is moved by the same amount; rows are untouched, and the
+// running softmax / the gradient accumulators simply carry on from pass to pass.
+DLT_HD Swa2Geom swa2_pass_geom(const Swa2Geom& G, int ncg_class, int pass) {
+  Swa2Geom P = G;
+  P.WC = G.WC - 4 * ncg_class * pass;
+  return P;
+}
+DLT_HD Swa2Win swa2_pass_window(const Swa2Win& W, int ncg_class, int pass) {
+  Swa2Win P = W;
+  P.clo = W.clo - 4 * ncg_class * pass;
+  return P;
+}
+// column groups of pass `pass` that can hold a visible token (window of WC columns to each side)
+DLT_HD int swa2_pass_ncg(int WC, int ncg_class, int pass) { return dlt_imin(ncg_class, ((4 + 2 * WC + 3) >> 2) - ncg_class * pass); }
 
 // visibility of the streamed token (halo row covered by row_vis, window column 4 cg + i) from the lane's own token
 DLT_HD bool swa2_visible(const Swa2Win& W, bool row_vis, int cg, int i, int ncg) {

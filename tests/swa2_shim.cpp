@@ -6,7 +6,7 @@
 //     every 16-byte slot (4-byte slot for scalars) holds;
 //   * the operand reads (A operand, transposing read, scalar reads) against that model;
 //   * the store epilogue's tile writes and reads;
-//   * the window geometry against dlt_key_range.
+//   * the window geometry against dlt_key_range: over all column passes every key of a window is visible exactly once.
 // and reports the first violated condition.  Built by tests/test_swa2_index_cpu.py with the host compiler; not part of
 // the library.
 #include <cstdio>
@@ -25,11 +25,11 @@ int fail(const char* fmt, int a = 0, int b = 0, int c = 0, int d = 0, int e = 0,
 struct Slot { int tensor, r, c, piece; };   // tensor -1: never written
 
 template <typename C>
-int model(int TR, int TC, int WR, int WC, int sn2, int ls2, long long slab_bytes, long long scal_elems, int lds_bytes, int lds_kv_bytes) {
+int model(int TR, int TC, int WR, int WC, int npass, int sn2, int ls2, long long slab_bytes, long long scal_elems, int lds_bytes, int lds_kv_bytes) {
   if (lds_bytes != C::LDS) return fail("launcher asks for %d bytes of LDS, the class needs %d", lds_bytes, C::LDS);
   if (lds_kv_bytes != C::LDS_KV) return fail("launcher asks for %d bytes of LDS (dK/dV), the class needs %d", lds_kv_bytes, C::LDS_KV);
-  const int ncg = (4 + 2 * WC + 3) >> 2;
-  if (ncg > C::NCG) return fail("window of %d column groups on a class with %d", ncg, C::NCG);
+  const int ncg_total = (4 + 2 * WC + 3) >> 2;
+  if (ncg_total > C::NCG * npass) return fail("window of %d column groups on a class with %d in %d column passes", ncg_total, C::NCG, npass);
   Swa2Plan P;
   P.nblk_r = (TR + 7) / 8;
   P.nblk_c = (TC + 15) / 16;
@@ -42,7 +42,8 @@ int model(int TR, int TC, int WR, int WC, int sn2, int ls2, long long slab_bytes
   std::vector<Slot> lds(C::LDS_KV / 4);
   const int nwg = P.nblk_r * P.nblk_c;
   for (int lin = 0; lin < nwg; lin++) {
-    const Swa2Geom G = swa2_geom_at(TR, TC, WR, WC, H, P, lin);
+    const Swa2Geom G0 = swa2_geom_at(TR, TC, WR, WC, H, P, lin);
+    const Swa2Geom& G = G0;
     if (G.b != 0 || G.h != 0) return fail("workgroup %d decoded to batch %d head %d", lin, G.b, G.h);
     if (G.r0 >= TR || G.c0 >= TC) return fail("workgroup %d starts outside the grid (%d, %d)", lin, G.r0, G.c0);
     if (G.ch_first > G.ch_last) return fail("workgroup %d: empty chunk range", lin);
@@ -50,35 +51,46 @@ int model(int TR, int TC, int WR, int WC, int sn2, int ls2, long long slab_bytes
     for (int wave = 0; wave < 8; wave++) {
       const int pc = wave & 3, rg = wave >> 2;
       for (int n = 0; n < 16; n++) {
-        const Swa2Win W = swa2_window(G, rg, pc, n);
+        const Swa2Win W0 = swa2_window(G, rg, pc, n);
         const int r = G.r0 + 4 * rg + (n >> 2), c = G.c0 + 4 * pc + (n & 3);
         const bool own = r < TR && c < TC;
-        int rlo, rhi, xlo, xhi;
+        int rlo = 0, rhi = -1, xlo = 0, xhi = 0;
         if (own) dlt_key_range(dg, r, c, rlo, rhi, xlo, xhi);
-        for (int ch = 0; ch <= (7 + 2 * WR) >> 2; ch++)
-          for (int hr = 0; hr < 4; hr++) {
-            const int hrow = 4 * ch + hr, kr = G.r0 - WR + hrow;
-            const bool row_vis = hrow >= W.rlo && hrow <= W.rhi;
-            for (int cg = 0; cg < C::NCG; cg++)
-              for (int i = 0; i < 4; i++) {
-                const int kc = G.c0 - WC + 4 * (pc + cg) + i;
-                if (!own) continue;   // own positions outside the grid compute values that are never stored
-                const bool want = kr >= rlo && kr <= rhi && kc >= xlo && kc < xhi;
-                const bool got = swa2_visible(W, row_vis, cg, i, ncg);
-                if (want != got) return fail("visibility of key (%d, %d) from own token (%d, %d): kernel %d, geometry %d", kr, kc, r, c, got, want);
-                if (got && (ch < G.ch_first || ch > G.ch_last || ch < W.ch_lo || ch > W.ch_hi))
-                  return fail("visible key row %d (chunk %d) outside the chunk range the wave consumes [%d, %d]", kr, ch, W.ch_lo, W.ch_hi);
-              }
-          }
-        // every key of the window lies inside the wave's NCG column groups and the band's chunks
+        int hits = 0;
+        for (int pass = 0; pass < npass; pass++) {
+          const Swa2Geom Gp = swa2_pass_geom(G0, C::NCG, pass);
+          const Swa2Win W = swa2_pass_window(W0, C::NCG, pass);
+          const int ncg = swa2_pass_ncg(WC, C::NCG, pass);
+          for (int ch = 0; ch <= (7 + 2 * WR) >> 2; ch++)
+            for (int hr = 0; hr < 4; hr++) {
+              const int hrow = 4 * ch + hr, kr = G.r0 - WR + hrow;
+              const bool row_vis = hrow >= W.rlo && hrow <= W.rhi;
+              for (int cg = 0; cg < C::NCG; cg++)
+                for (int i = 0; i < 4; i++) {
+                  const int kc = G.c0 - Gp.WC + 4 * (pc + cg) + i;
+                  if (!own) continue;   // own positions outside the grid compute values that are never stored
+                  const bool want = kr >= rlo && kr <= rhi && kc >= xlo && kc < xhi;
+                  const bool got = swa2_visible(W, row_vis, cg, i, ncg);
+                  if (want != got && (got || cg < ncg)) return fail("visibility of key (%d, %d) from own token (%d, %d): kernel %d, geometry %d", kr, kc, r, c, got, want);
+                  hits += got;
+                  if (got && (ch < G.ch_first || ch > G.ch_last || ch < W.ch_lo || ch > W.ch_hi))
+                    return fail("visible key row %d (chunk %d) outside the chunk range the wave consumes [%d, %d]", kr, ch, W.ch_lo, W.ch_hi);
+                }
+            }
+        }
+        // every key of the window is seen in exactly one (pass, column group) and lies inside the band's chunks
         if (own) {
-          if (xlo < G.c0 - WC + 4 * pc || xhi > G.c0 - WC + 4 * (pc + C::NCG)) return fail("window columns [%d, %d) exceed the wave window of own token (%d, %d)", xlo, xhi, r, c);
+          if (hits != (rhi - rlo + 1) * (xhi - xlo)) return fail("own token (%d, %d): %d keys visible over all passes, the window holds %d", r, c, hits, (rhi - rlo + 1) * (xhi - xlo));
+          if (xlo < G.c0 - WC + 4 * pc || xhi > G.c0 - WC + 4 * (pc + C::NCG * npass)) return fail("window columns [%d, %d) exceed the wave window of own token (%d, %d)", xlo, xhi, r, c);
           if (rlo < G.r0 - WR + 4 * G.ch_first || rhi > G.r0 - WR + 4 * G.ch_last + 3) return fail("window rows [%d, %d] exceed the band's chunks", rlo, rhi);
         }
       }
     }
     // ---- chunks: copies into the buffer (ch & 1), then the reads of every wave
+    for (int pass = 0; pass < npass; pass++)
     for (int kv = 0; kv < 2; kv++) {   // 0: forward / dQ layout (BUF), 1: dK/dV layout (BUF_KV, with scalars)
+      const Swa2Geom G = swa2_pass_geom(G0, C::NCG, pass);   // what the kernels address columns with in this pass
+      const int WC = G.WC;
       const int bufsz = kv ? C::BUF_KV : C::BUF, total = kv ? C::LDS_KV : C::LDS;
       for (int ch = G.ch_first; ch <= G.ch_last; ch++) {
         for (Slot& s : lds) s.tensor = -1;
@@ -233,10 +245,10 @@ extern "C" {
 // 0: every condition holds; 1: see swa2_model_message().  lds_bytes / lds_kv_bytes: what the launcher passes for the
 // class (checked against the class constants); slab_bytes: bytes of one (batch, head) slab of a streamed tensor;
 // scal_elems: elements of one (batch, head) slab of lse2 / delta.
-int swa2_model(int D, int NCG, int TR, int TC, int WR, int WC, int sn2, int ls2, long long slab_bytes, long long scal_elems,
+int swa2_model(int D, int NCG, int npass, int TR, int TC, int WR, int WC, int sn2, int ls2, long long slab_bytes, long long scal_elems,
                int lds_bytes, int lds_kv_bytes) {
   g_msg[0] = 0;
-#define CASE(d, n) if (D == d && NCG == n) return model<Swa2Cfg<d, n>>(TR, TC, WR, WC, sn2, ls2, slab_bytes, scal_elems, lds_bytes, lds_kv_bytes);
+#define CASE(d, n) if (D == d && NCG == n) return model<Swa2Cfg<d, n>>(TR, TC, WR, WC, npass, sn2, ls2, slab_bytes, scal_elems, lds_bytes, lds_kv_bytes);
   CASE(64, 4) CASE(64, 6) CASE(64, 8) CASE(64, 10) CASE(128, 4) CASE(128, 6)
 #undef CASE
   return fail("no class (%d, %d)", D, NCG);

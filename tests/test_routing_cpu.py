@@ -1,7 +1,7 @@
 """Which kernel family a call is routed to, asked through the C ABI without a GPU: under dlt_dry_run(1) the entry points
 validate and route but launch nothing, and dlt_last_kernel_family() names the family.  The cases pin the routing table
 that include/dlt.h documents, so that a call landing on the (several times slower) generic kernels is visible to a C
-caller: head dims outside the tuned shapes, windows wider than 21 columns, rows that are not 16-byte aligned, fp32."""
+caller: head dims outside the tuned shapes, windows wider than 93 columns, rows that are not 16-byte aligned, fp32."""
 import ctypes
 import os
 
@@ -71,6 +71,9 @@ def test_token_grid_routing_table(L, backward):
     assert _swa(L, 1, 96, 160, 10, 10, 128, 128, FP16, **kw) == "streaming"
     # head dim 64 beyond the marching kernels' 13 x 13 window, head dims in multiples of 32 below a class
     assert _swa(L, 1, 40, 40, 9, 9, 64, 64, BF16, **kw) == "streaming"
+    # windows wider than 21 columns: the streaming kernels in column passes (any number of rows)
+    assert _swa(L, 1, 40, 40, 11, 11, 64, 64, BF16, **kw) == "streaming"
+    assert _swa(L, 1, 40, 90, 30, 34, 128, 128, FP16, **kw) == "streaming"
     assert _swa(L, 1, 40, 40, 3, 3, 96, 96, BF16, **kw) == "tile"
     assert _swa(L, 1, 40, 40, 3, 3, 32, 64, BF16, **kw) == "tile"
     # rotation inside the tile loads (nothing kept), rotation at head dim 128 or with 16 rotary pairs
@@ -80,7 +83,9 @@ def test_token_grid_routing_table(L, backward):
     # than 21 columns, fp32, rows that are not 16-byte aligned, tiles that are not multiples of 16 tokens
     assert _swa(L, 1, 40, 40, 3, 3, 80, 80, BF16, **kw) == "generic"
     assert _swa(L, 1, 40, 40, 3, 3, 64, 128, BF16, **kw) == "generic"
-    assert _swa(L, 1, 40, 40, 11, 11, 64, 64, BF16, **kw) == "generic"
+    assert _swa(L, 1, 8, 200, 3, 47, 64, 64, BF16, **kw) == "generic"                     # 95 columns: more than 4 passes of 6 groups
+    assert _swa(L, 1, 40, 40, 11, 11, 96, 96, BF16, **kw) == "generic"                    # wide window below the class's head dim
+    assert _swa(L, 1, 40, 40, 3, 11, 64, 64, BF16, rope_R=8, **kw) == "generic"           # wide window with rotation
     assert _swa(L, 1, 40, 40, 3, 3, 64, 64, FP32, **kw) == "generic"
     assert _swa(L, 1, 40, 40, 3, 3, 64, 64, BF16, align=2, **kw) == "generic"
     assert _swa(L, 1, 40, 40, 3, 3, 64, 64, BF16, pad=1, **kw) == "generic"

@@ -80,6 +80,21 @@ def test_ragged_and_boundary_grids_head_dim_128(th, tw, wr, wc, dtype):
     _run(21, 1, 2, 1, th, tw, wr, wc, 128, 128, dtype)
 
 
+# windows wider than 21 columns: the streaming kernels walk them in column passes of 4 or 6 column groups (23 / 29
+# columns: 2 x 4 groups; 37 / 45: 2 x 6; 69: 3 x 6), the running softmax and the gradient accumulators carrying on from
+# pass to pass; grids narrower than the window, ragged grids, a one-row window
+WIDE = [(9, 50, 3, 11), (24, 40, 11, 11), (12, 70, 2, 14), (10, 45, 4, 18), (7, 60, 1, 22), (5, 80, 0, 34), (20, 20, 12, 12),
+        (17, 33, 5, 13)]
+
+
+@pytest.mark.parametrize("d", [64, 128])
+@pytest.mark.parametrize("th,tw,wr,wc", WIDE)
+def test_windows_wider_than_21_columns(th, tw, wr, wc, d):
+    from dl_templates_amd import _lib
+    _run(40 + wc, 1, 2, 1, th, tw, wr, wc, d, d, torch.bfloat16)
+    assert _lib.KERNEL_FAMILIES[_lib.load().dlt_last_kernel_family()] == "streaming"
+
+
 @pytest.mark.parametrize("b_size,th,tw,wr,wc", [(16, 8, 8, 1, 1), (4, 6, 5, 1, 2), (3, 5, 4, 2, 1), (32, 3, 4, 1, 1), (2, 9, 9, 6, 6), (100, 2, 3, 1, 1)])
 def test_tiles_with_several_tokens(b_size, th, tw, wr, wc):
     _run(3, 1, 2, b_size, th, tw, wr, wc, 32, 32, torch.bfloat16, scale=0.25)
