@@ -310,6 +310,12 @@ void swa2_split(const AttnProblem& p, int& ncg_class, int& npass) {
   else { ncg_class = 6; npass = n6; }
 }
 int swa2_ncg(const AttnProblem& p) { int c, n; swa2_split(p, c, n); return c; }
+// the problem without its rotation would run on the streaming kernels
+// and is large enough that the four extra launches (two out-of-place rotations, two in-place inverse rotations) do not
+// cost more than the tile kernels' repeated rotation (measured: a gain from about 10^5 tokens per call on)
+bool swa2_compose_ok(const AttnProblem& p, const Swa1Class& c) {
+  return (c.D == 64 || c.D == 128) && p.dk == c.D && p.dv == c.D && (int64_t)p.B * p.H * p.g.TR * p.g.TC >= 131072;
+}
 
 void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan) {
   { int c; swa2_split(p, c, plan.npass); }
@@ -512,7 +518,13 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
                               (t.q_rot == nullptr || (swam_rows_ok(p, t.q_rot, t.qrs) && swam_rows_ok(p, t.k_rot, t.krs)));
         if (swam_eligible(p, c) && rows_fit) return swam_forward(p, t, c, stream);
         if (swa2_eligible(p, c) && t.q_rot == nullptr && swa2_rows_ok(p, t.out_o, t.os)) return swa2_forward(p, t, stream);
-        if (c.wclass < 2) return swa1_forward(p, t, c, stream);
+        // Rotation the marching kernels do not take, with the rotated q / k wanted by the caller: rotating both out of place
+        // first (below) and running the streaming kernels on the result is faster than the tile kernels, which rotate every
+        // halo row again in each workgroup that stages it (128 x 128 grid, d = 128, 21 x 21, 16 rotary pairs, fwd+bwd:
+        // 0.90 -> 0.64 ms)
+        const bool compose = c.rope_mode != 0 && t.q_rot != nullptr && swa2_compose_ok(p, c) && swa2_rows_ok(p, t.out_o, t.os) &&
+                             swa2_rows_ok(p, t.q_rot, t.qrs) && swa2_rows_ok(p, t.k_rot, t.krs);
+        if (c.wclass < 2 && !compose) return swa1_forward(p, t, c, stream);
       }
     }
   }
@@ -581,7 +593,12 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
       if (swa2_eligible(p, c) && swa2_rows_ok(p, t.o, t.os) && swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) &&
           swa2_rows_ok(p, t.dv, t.dvs) && t.ls[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * t.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1))
         return swa2_backward(p, t, stream);
-      if (c.wclass < 2) return swa1_backward(p, t, c, stream);
+      // rotated q, k that the marching kernels do not take: the streaming kernels on the rotated tensors, then dq / dk
+      // rotated back in place (below), instead of the tile kernels (see the forward pass)
+      const bool compose = p.rope_prerot && c.rope_mode != 0 && swa2_compose_ok(p, c) && swa2_rows_ok(p, t.o, t.os) &&
+                           swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) && swa2_rows_ok(p, t.dv, t.dvs) && t.ls[2] >= 0 &&
+                           ((int64_t)p.g.TR * p.g.TC - 1) * t.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1);
+      if (c.wclass < 2 && !compose) return swa1_backward(p, t, c, stream);
     }
   }
   if (p.rope_prerot && p.rope.enabled && p.rope.R > 0 && !p.tm.img) {

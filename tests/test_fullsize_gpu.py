@@ -174,6 +174,36 @@ def test_c3_full_batch_fused_rope_equals_composition(save_rotated):
     assert torch.isfinite(o.float()).all() and torch.isfinite(qg.grad.float()).all()
 
 
+@pytest.mark.parametrize("d,R,W,family", [(128, 16, 10, "streaming"), (64, 16, 4, "marching"), (64, 8, 9, "streaming")])
+def test_large_grid_fused_rope_runs_as_rotation_plus_plain_kernels(d, R, W, family):
+    """Fused rotation that the marching kernels do not take (head dim 128, 16 rotary pairs, or a window beyond 13 x 13), on
+    a grid large enough (131 072 tokens) that the library rotates q and k out of place once and runs the plain operator's
+    kernels (streaming, or marching for a window up to 13 x 13 at head dim 64) on the result, the gradients rotated back in
+    place: bit-equal to the same composition made of the public pieces
+    (RotaryPE2D on clones + TiledSwa), which the smaller tests hold to the oracle."""
+    from dl_templates_amd import _lib
+    sw, _, fr = _mods()
+    B, H, th, tw = 1, 8, 128, 128
+    N = th * tw
+    q, k, v, do = (t.cuda() for t in orc.make_qkv(d + R, B, H, N, N, d, d, torch.bfloat16))
+    idx = orc.make_rope_idx(34, th, tw, 0.05).cuda()
+    rcs, ccs = orc.rope_tables(R, th).cuda(), orc.rope_tables(R, tw).cuda()
+    scale = 1 / math.sqrt(d)
+    qg, kg, vg = (t.detach().requires_grad_(True) for t in (q, k, v))
+    o = sw.TiledSwaRope.apply(qg, kg, vg, idx, rcs, ccs, 1, th, tw, W, W, scale)
+    assert _lib.KERNEL_FAMILIES[_lib.load().dlt_last_kernel_family()] == family
+    o.backward(do)
+    assert _lib.KERNEL_FAMILIES[_lib.load().dlt_last_kernel_family()] == family
+    q2, k2, v2 = (t.detach().requires_grad_(True) for t in (q, k, v))
+    qr = fr.RotaryPE2D.apply(q2.clone().view(-1, N, d), idx, rcs, ccs).view(q.shape)
+    kr = fr.RotaryPE2D.apply(k2.clone().view(-1, N, d), idx, rcs, ccs).view(k.shape)
+    o2 = sw.TiledSwa.apply(qr, kr, v2, 1, th, tw, W, W, scale)
+    o2.backward(do)
+    assert torch.equal(o, o2)
+    assert torch.equal(qg.grad, q2.grad) and torch.equal(kg.grad, k2.grad) and torch.equal(vg.grad, v2.grad)
+    assert torch.equal(qg, q) and torch.equal(kg, k)      # the caller's q and k are left as they were
+
+
 def test_c5_flash_kernels_vs_generic_dense_kernels():
     _, fa, _ = _mods()
     B, H, Lq, Lk, dk, dv = 2, 16, 4096, 8192, 64, 128
