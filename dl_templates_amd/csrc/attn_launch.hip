@@ -299,11 +299,14 @@ int swam_forward(const AttnProblem& p, const AttnTensors& t, const Swa1Class& c,
 bool swa2_eligible(const AttnProblem& p, const Swa1Class& c) {
   return (c.D == 64 || c.D == 128) && p.dk == c.D && p.dv == c.D && c.rope_mode == 0;
 }
+// token slots per grid row, and the largest column extent of a window in slots (tiles of S tokens: S WC + S - 1)
+int swa2_slots(const AttnProblem& p) { return p.g.TC * p.g.S; }
+int swa2_extent(const AttnProblem& p) { return p.g.S * p.g.WC + p.g.S - 1; }
 // Kernel class (column groups of a wave's window per pass: 4 x 4 columns cover windows up to 13 columns, 6 x 4 up to 21)
 // and number of column passes.  Wider windows take the split that computes the fewest groups (7 groups: 2 passes of 4,
 // not 2 of 6), the larger class on a tie (fewer passes).
 void swa2_split(const AttnProblem& p, int& ncg_class, int& npass) {
-  const int ncg = (4 + 2 * p.g.WC + 3) / 4;
+  const int ncg = (4 + 2 * swa2_extent(p) + 3) / 4;
   if (ncg <= 4) { ncg_class = 4; npass = 1; return; }
   const int n4 = (ncg + 3) / 4, n6 = (ncg + 5) / 6;
   if (4 * n4 < 6 * n6 && n4 <= SWA2_MAX_PASSES) { ncg_class = 4; npass = n4; }
@@ -319,15 +322,37 @@ bool swa2_compose_ok(const AttnProblem& p, const Swa1Class& c) {
 
 void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan) {
   { int c; swa2_split(p, c, plan.npass); }
+  plan.S = p.g.S; plan.WCt = p.g.WC;
+  dlt_fastdiv_make((uint32_t)p.g.S, plan.m_S, plan.s_S);
   plan.nblk_r = (p.g.TR + 7) / 8;
-  plan.nblk_c = (p.g.TC + 15) / 16;
+  plan.nblk_c = (swa2_slots(p) + 15) / 16;
   dlt_fastdiv_make((uint32_t)(plan.nblk_r * plan.nblk_c), plan.m_bh, plan.s_bh);
   dlt_fastdiv_make((uint32_t)plan.nblk_c, plan.m_c, plan.s_c);
   dlt_fastdiv_make((uint32_t)p.H, plan.m_h, plan.s_h);
 }
 
 bool swa2_rows_ok(const AttnProblem& p, const void* ptr, const int64_t* st) {
-  return tvec_ok(ptr, st, p.dk, 2) && st[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * st[2] * 2 + 2 * p.dk <= (((int64_t)1 << 31) - 1);
+  return tvec_ok(ptr, st, p.dk, 2) && st[2] >= 0 && ((int64_t)p.g.TR * swa2_slots(p) - 1) * st[2] * 2 + 2 * p.dk <= (((int64_t)1 << 31) - 1);
+}
+bool swa2_scalars_ok(const AttnProblem& p, const AttnTensors& t) {
+  return t.ls[2] >= 0 && ((int64_t)p.g.TR * swa2_slots(p) - 1) * t.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1);
+}
+
+// Tiles of 2 ... 15 tokens (the regime of the reference's small-tile kernel, src/tiled_swa.py:15-133, b_size < 16 at
+// :611): the streaming kernels on the grid of token slots, with the window of a token given by its tile
+// (csrc/swa2_index.h).  Head dim 64 or 128 exactly, 2-byte types, no rotation, plain token layout.
+bool swa2_tiles_eligible(const AttnProblem& p, const AttnTensors& t, bool backward) {
+  if (p.g.mode != DLT_GEOM_SWA || p.g.S < 2 || p.g.S > 15 || p.tm.img) return false;
+  if (p.dtype != DLT_BF16 && p.dtype != DLT_FP16) return false;
+  if (!(p.sm_scale > 0.f)) return false;
+  if (!((p.dk == 64 || p.dk == 128) && p.dv == p.dk)) return false;
+  if (p.rope.enabled && p.rope.R > 0) return false;
+  if ((4 + 2 * swa2_extent(p) + 3) / 4 > SWA2_MAX_PASSES * 6) return false;
+  if ((int64_t)p.g.TR * swa2_slots(p) >= ((int64_t)1 << 31) / 1024) return false;
+  if (!swa2_rows_ok(p, t.q, t.qs) || !swa2_rows_ok(p, t.k, t.ks) || !swa2_rows_ok(p, t.v, t.vs)) return false;
+  if (!backward) return t.q_rot == nullptr && swa2_rows_ok(p, t.out_o, t.os);
+  return swa2_rows_ok(p, t.o, t.os) && swa2_rows_ok(p, t.d_o, t.dos) && swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) &&
+         swa2_rows_ok(p, t.dv, t.dvs) && swa2_scalars_ok(p, t);
 }
 
 int swa2_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream) {
@@ -542,6 +567,7 @@ int dlt_attn_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t str
     return dlt_attn_forward(p2, t2, stream);
   }
   if (flash_eligible(p, t, false)) return flash_forward(p, t, dc, stream);
+  if (swa2_tiles_eligible(p, t, false)) return swa2_forward(p, t, stream);
   if (dlt_route_note(DLT_FAMILY_GENERIC)) return DLT_OK;
   const int np = (p.g.mode == DLT_GEOM_SWA || dc.id == 4) ? 1 : 2;
   const int own = 64 * np;
@@ -591,13 +617,12 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
         return swam_backward(p, t, c.rope_mode != 0, stream);
       // lse2 / delta rows are copied with 32-bit byte offsets inside a (batch, head) slab
       if (swa2_eligible(p, c) && swa2_rows_ok(p, t.o, t.os) && swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) &&
-          swa2_rows_ok(p, t.dv, t.dvs) && t.ls[2] >= 0 && ((int64_t)p.g.TR * p.g.TC - 1) * t.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1))
+          swa2_rows_ok(p, t.dv, t.dvs) && swa2_scalars_ok(p, t))
         return swa2_backward(p, t, stream);
       // rotated q, k that the marching kernels do not take: the streaming kernels on the rotated tensors, then dq / dk
       // rotated back in place (below), instead of the tile kernels (see the forward pass)
       const bool compose = p.rope_prerot && c.rope_mode != 0 && swa2_compose_ok(p, c) && swa2_rows_ok(p, t.o, t.os) &&
-                           swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) && swa2_rows_ok(p, t.dv, t.dvs) && t.ls[2] >= 0 &&
-                           ((int64_t)p.g.TR * p.g.TC - 1) * t.ls[2] * 4 + 4 <= (((int64_t)1 << 31) - 1);
+                           swa2_rows_ok(p, t.dq, t.dqs) && swa2_rows_ok(p, t.dk, t.dks) && swa2_rows_ok(p, t.dv, t.dvs) && swa2_scalars_ok(p, t);
       if (c.wclass < 2 && !compose) return swa1_backward(p, t, c, stream);
     }
   }
@@ -618,6 +643,7 @@ int dlt_attn_backward(const AttnProblem& p, const AttnTensors& t, hipStream_t st
     return dlt_rope_inplace_4d(t.dk, t.dks, p.B, p.H, (int64_t)p.g.TR * p.g.XLk, p.dk, &r, 1, p.dtype, stream);
   }
   if (flash_eligible(p, t, true)) return flash_backward(p, t, dc, stream);
+  if (swa2_tiles_eligible(p, t, true)) return swa2_backward(p, t, stream);
   if (dlt_route_note(DLT_FAMILY_GENERIC)) return DLT_OK;
   const int np = 1;
   const int own = 64 * np;

@@ -34,7 +34,8 @@ DLT_DEV u32x2 swa2_lds_tr(Swa2Lds p) {
 }
 
 DLT_DEV Swa2Geom swa2_geom(const AttnProblem& p, const Swa2Plan& P) {
-  return swa2_geom_at(p.g.TR, p.g.TC, p.g.WR, p.g.WC, p.H, P, xcd_remap(blockIdx.x, gridDim.x));
+  // token slots per grid row and the largest column extent of a window in slots (tiles of P.S tokens)
+  return swa2_geom_at(p.g.TR, p.g.TC * P.S, p.g.WR, P.S * P.WCt + P.S - 1, p.H, P, xcd_remap(blockIdx.x, gridDim.x));
 }
 
 // One copy instruction as the hardware sees it: 64 lanes x 16 (or 4) bytes from `base + voff` (base wave-uniform)

@@ -123,7 +123,9 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
     if (__builtin_amdgcn_ballot_w64((mloc - m_run) * scale > 8.f)) {
       keep_branch();
       const float m_new = fmaxf(m_run, mloc);
-      const float alpha = fast_exp2((m_run - m_new) * scale);   // m_new is finite here
+      // a lane that has not seen a key yet keeps its (zero) accumulators as they are: with column passes, or with tiles of
+      // several tokens, a query's first keys may lie in a later pass than those of the lane that triggers the update
+      const float alpha = m_new == -INFINITY ? 1.f : fast_exp2((m_run - m_new) * scale);
       m_run = m_new;
 #pragma unroll
       for (int d = 0; d < VB; d++) acc[d] *= alpha;

@@ -4,7 +4,11 @@
 //
 // A workgroup of 8 waves owns a band of 8 grid rows x 16 grid columns; wave w owns the 4x4 patch at rows
 // 4 (w >> 2), columns 4 (w & 3).  The halo of the band (8 + 2 WR rows x HCW columns, first halo column = c0 - WC)
-// streams through LDS in chunks of 4 halo rows.  LDS rows are 2 D bytes with no padding; the 16-byte piece c of token
+// streams through LDS in chunks of 4 halo rows.
+//
+// Tiles of S tokens (1 < S < 16): a grid row then holds TC = tiles * S token slots ("columns" below are slots), a token
+// in tile t sees the slots of tiles t - WCt .. t + WCt, i.e. S WCt + (x mod S) slots to its left and S WCt + S - 1 - (x mod S)
+// to its right; WC is the largest of these extents, S WCt + S - 1, and positions the halo.  S = 1: WC = WCt.  LDS rows are 2 D bytes with no padding; the 16-byte piece c of token
 // row t (t = halo row inside the chunk * HCW + halo column) is stored at piece c ^ (SWZ (t & 7)).
 #pragma once
 #include "dlt_geom.h"
@@ -46,18 +50,29 @@ struct Swa2Plan {
   int32_t nblk_r, nblk_c;
   uint32_t m_bh, s_bh, m_c, s_c, m_h, s_h;   // exact multiply-shift divisions by nblk_r * nblk_c, nblk_c and H
   int32_t npass;   // column passes: a window of more than NCG column groups is walked in npass slices of NCG groups
+  int32_t S, WCt;  // tokens per tile, window half-width in tiles
+  uint32_t m_S, s_S;   // division by S
 };
 
 struct Swa2Geom {
-  int TR, TC, WR, WC;
+  int TR, TC, WR, WC;   // grid rows, token slots per row, window half-height in rows, largest column extent in slots
   int r0, c0;   // first grid row / column of the band
   int b, h;
   int ch_first, ch_last;   // chunks of the band's halo that hold grid rows
+  int S, WCt;
+  uint32_t m_S, s_S;
 };
 
-// geometry of workgroup `lin` (its index after the XCD remap)
+// plan fields of a token grid (one token per tile)
+DLT_HD void swa2_plan_tokens(Swa2Plan& P, int WC) {
+  P.S = 1; P.WCt = WC;
+  dlt_fastdiv_make(1u, P.m_S, P.s_S);
+}
+
+// geometry of workgroup `lin` (its index after the XCD remap); TC: token slots per grid row, WC: S WCt + S - 1
 DLT_HD Swa2Geom swa2_geom_at(int TR, int TC, int WR, int WC, int H, const Swa2Plan& P, int lin) {
   Swa2Geom G;
+  G.S = P.S; G.WCt = P.WCt; G.m_S = P.m_S; G.s_S = P.s_S;
   const int per_bh = P.nblk_r * P.nblk_c;
   const int bh = (int)dlt_fastdiv((uint32_t)lin, P.m_bh, P.s_bh);
   const int rem = lin - bh * per_bh;
@@ -87,8 +102,12 @@ DLT_HD Swa2Win swa2_window(const Swa2Geom& G, int rg, int pc, int n) {
   const bool ok = (G.r0 + qr < G.TR) && (c_p + qc < G.TC);
   w.rlo = dlt_imax(qr, G.WR - G.r0);
   w.rhi = dlt_imin(qr + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
-  w.clo = dlt_imax(qc, G.WC - c_p);
-  const int chi = dlt_imin(qc + 2 * G.WC, G.TC - 1 - c_p + G.WC);
+  // window columns: the wave window starts at slot c_p - WC, the own token sits at window column WC + qc
+  const int x = c_p + qc;
+  const int xm = x - G.S * (int)dlt_fastdiv((uint32_t)x, G.m_S, G.s_S);   // slot inside its tile
+  const int reach = G.S * G.WCt;
+  w.clo = dlt_imax(G.WC + qc - reach - xm, G.WC - c_p);
+  const int chi = dlt_imin(G.WC + qc + reach + (G.S - 1 - xm), G.TC - 1 - c_p + G.WC);
   w.cspan = ok ? chi - w.clo : -1;
   // halo rows of the patch that hold grid rows
   const int plo = dlt_imax(4 * rg, G.WR - G.r0), phi = dlt_imin(4 * rg + 3 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);

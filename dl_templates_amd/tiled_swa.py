@@ -40,11 +40,18 @@ def _pad_plan(q, v, b_size):
     <= 64, or both in 65..128); anything else runs on the generic kernels, 6 to 9 times slower (measured at d = 40, 48,
     80 against 64, 96, 128).  Zero columns appended to q, k, v (and to dO in the backward pass) change no score and no
     output column, so such calls are padded to the next tuned shape here and the results sliced back: four to eight
-    extra copy passes over the tensors, a few percent of the step.  Tile mode (``b_size > 1``) needs none of this: its
+    extra copy passes over the tensors, a few percent of the step.  Tiles of 16 k tokens need none of this: their
     kernels pad inside.
     """
     dk, dv = q.shape[-1], v.shape[-1]
-    if b_size != 1 or q.dtype not in (torch.bfloat16, torch.float16) or max(dk, dv) > 128:
+    if q.dtype not in (torch.bfloat16, torch.float16) or max(dk, dv) > 128:
+        return None
+    if 2 <= b_size <= 15:
+        # tiles of fewer than 16 tokens run on the streaming token-grid kernels at head dim 64 or 128 exactly (both equal);
+        # the generic kernels they would use otherwise are 2 to 4 times slower
+        t = 64 if max(dk, dv) <= 64 else 128
+        return None if (dk, dv) == (t, t) else (t, t)
+    if b_size != 1:
         return None
     up = lambda d: (d + 31) // 32 * 32
     tk, tv = (up(dk), up(dv)) if max(dk, dv) <= 64 else (max(96, up(dk)), max(96, up(dv)))

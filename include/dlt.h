@@ -253,13 +253,14 @@ int dlt_debug_copy(void* dst, const void* src, int64_t bytes, void* stream);
 
 /* Which kernel family an attention call runs on.  No counterpart in the reference (Triton picks a configuration by
  * autotuning, src/tiled_swa.py:570-573); here the host routes every call by shape, element type, strides and
- * alignment, and a C caller cannot see from the outside that, say, head dim 80 or a 23-column window lands on the
+ * alignment, and a C caller cannot see from the outside that, say, head dim 80 or a 9-token tile at head dim 96 lands on the
  * generic kernels (several times slower than the tuned ones).  dlt_last_kernel_family() returns the family the calling
  * thread's latest forward / backward call (dlt_swa_*, dlt_flash_*) was routed to.  With dlt_dry_run(1) (per thread) those
  * calls validate their arguments and route, but launch nothing and touch no memory: pointers only need the alignment
  * of the real ones, so the query also works in a process without a GPU.
  *   MARCHING  token grids (b_size 1), head dim 64, windows up to 13 x 13 (rotation: 8 rotary pairs, rotated q / k kept)
- *   STREAMING token grids, head dim 64 / 128, windows up to 21 columns, no rotation
+ *   STREAMING token grids, head dim 64 / 128, windows up to 93 columns (beyond 21 columns in column passes), no rotation;
+ *             tiles of 2 ... 15 tokens at head dim 64 / 128 (the grid of token slots, up to 24 column groups of 4 slots)
  *   TILE      token grids, head dims in multiples of 32 up to 128, windows up to 21 columns (rotation in the tile loads)
  *   FLASH     dense / causal / tiles of 16 k tokens, 2-byte element types, head dims up to 128 (multiples of 8)
  *   GENERIC   everything else */

@@ -25,20 +25,24 @@ int fail(const char* fmt, int a = 0, int b = 0, int c = 0, int d = 0, int e = 0,
 struct Slot { int tensor, r, c, piece; };   // tensor -1: never written
 
 template <typename C>
-int model(int TR, int TC, int WR, int WC, int npass, int sn2, int ls2, long long slab_bytes, long long scal_elems, int lds_bytes, int lds_kv_bytes) {
+int model(int TR, int TCt, int WR, int WCt, int S, int npass, int sn2, int ls2, long long slab_bytes, long long scal_elems, int lds_bytes, int lds_kv_bytes) {
   if (lds_bytes != C::LDS) return fail("launcher asks for %d bytes of LDS, the class needs %d", lds_bytes, C::LDS);
   if (lds_kv_bytes != C::LDS_KV) return fail("launcher asks for %d bytes of LDS (dK/dV), the class needs %d", lds_kv_bytes, C::LDS_KV);
+  // token slots per grid row and the largest column extent of a window in slots (tiles of S tokens)
+  const int TC = TCt * S, WC = S * WCt + S - 1;
   const int ncg_total = (4 + 2 * WC + 3) >> 2;
   if (ncg_total > C::NCG * npass) return fail("window of %d column groups on a class with %d in %d column passes", ncg_total, C::NCG, npass);
   Swa2Plan P;
   P.nblk_r = (TR + 7) / 8;
   P.nblk_c = (TC + 15) / 16;
   const int H = 1;
+  P.npass = npass; P.S = S; P.WCt = WCt;
+  dlt_fastdiv_make((uint32_t)S, P.m_S, P.s_S);
   dlt_fastdiv_make((uint32_t)(P.nblk_r * P.nblk_c), P.m_bh, P.s_bh);
   dlt_fastdiv_make((uint32_t)P.nblk_c, P.m_c, P.s_c);
   dlt_fastdiv_make((uint32_t)H, P.m_h, P.s_h);
   DltGeom dg;
-  dg.mode = DLT_GEOM_SWA; dg.TR = TR; dg.XLq = dg.XLk = TC; dg.S = 1; dg.TC = TC; dg.WR = WR; dg.WC = WC;
+  dg.mode = DLT_GEOM_SWA; dg.TR = TR; dg.XLq = dg.XLk = TC; dg.S = S; dg.TC = TCt; dg.WR = WR; dg.WC = WCt;
   std::vector<Slot> lds(C::LDS_KV / 4);
   const int nwg = P.nblk_r * P.nblk_c;
   for (int lin = 0; lin < nwg; lin++) {
@@ -245,10 +249,11 @@ extern "C" {
 // 0: every condition holds; 1: see swa2_model_message().  lds_bytes / lds_kv_bytes: what the launcher passes for the
 // class (checked against the class constants); slab_bytes: bytes of one (batch, head) slab of a streamed tensor;
 // scal_elems: elements of one (batch, head) slab of lse2 / delta.
-int swa2_model(int D, int NCG, int npass, int TR, int TC, int WR, int WC, int sn2, int ls2, long long slab_bytes, long long scal_elems,
+// TC, WC: tiles per grid row and window half-width in tiles; S: tokens per tile
+int swa2_model(int D, int NCG, int npass, int TR, int TC, int WR, int WC, int S, int sn2, int ls2, long long slab_bytes, long long scal_elems,
                int lds_bytes, int lds_kv_bytes) {
   g_msg[0] = 0;
-#define CASE(d, n) if (D == d && NCG == n) return model<Swa2Cfg<d, n>>(TR, TC, WR, WC, npass, sn2, ls2, slab_bytes, scal_elems, lds_bytes, lds_kv_bytes);
+#define CASE(d, n) if (D == d && NCG == n) return model<Swa2Cfg<d, n>>(TR, TC, WR, WC, S, npass, sn2, ls2, slab_bytes, scal_elems, lds_bytes, lds_kv_bytes);
   CASE(64, 4) CASE(64, 6) CASE(64, 8) CASE(64, 10) CASE(128, 4) CASE(128, 6)
 #undef CASE
   return fail("no class (%d, %d)", D, NCG);

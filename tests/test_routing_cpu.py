@@ -79,8 +79,9 @@ def test_token_grid_routing_table(L, backward):
     # rotation inside the tile loads (nothing kept), rotation at head dim 128 or with 16 rotary pairs
     assert _swa(L, 1, 40, 40, 3, 3, 64, 64, BF16, rope_R=8, **kw) == ("marching" if not backward else "tile")
     assert _swa(L, 1, 40, 40, 3, 3, 128, 128, BF16, rope_R=16, prerot=True, **kw) == "tile"
-    # what falls to the generic kernels: head dims that are not multiples of 32 or straddle the classes, windows wider
-    # than 21 columns, fp32, rows that are not 16-byte aligned, tiles that are not multiples of 16 tokens
+    # what falls to the generic kernels: head dims that are not multiples of 32 or straddle the classes, windows of more
+    # than 93 columns (or wide ones below a class's head dim, or with rotation), fp32, rows that are not 16-byte
+    # aligned, tiles that are neither multiples of 16 tokens nor 2 ... 15 tokens at head dim 64 / 128
     assert _swa(L, 1, 40, 40, 3, 3, 80, 80, BF16, **kw) == "generic"
     assert _swa(L, 1, 40, 40, 3, 3, 64, 128, BF16, **kw) == "generic"
     assert _swa(L, 1, 8, 200, 3, 47, 64, 64, BF16, **kw) == "generic"                     # 95 columns: more than 4 passes of 6 groups
@@ -89,8 +90,11 @@ def test_token_grid_routing_table(L, backward):
     assert _swa(L, 1, 40, 40, 3, 3, 64, 64, FP32, **kw) == "generic"
     assert _swa(L, 1, 40, 40, 3, 3, 64, 64, BF16, align=2, **kw) == "generic"
     assert _swa(L, 1, 40, 40, 3, 3, 64, 64, BF16, pad=1, **kw) == "generic"
-    assert _swa(L, 9, 8, 8, 1, 1, 64, 64, BF16, **kw) == "generic"
+    assert _swa(L, 9, 8, 8, 1, 1, 32, 32, BF16, **kw) == "generic"
     assert _swa(L, 24, 8, 8, 1, 1, 64, 64, BF16, **kw) == "generic"
+    # tiles of 2 ... 15 tokens at head dim 64 / 128: the streaming kernels on the grid of token slots
+    assert _swa(L, 9, 8, 8, 1, 1, 64, 64, BF16, **kw) == "streaming"
+    assert _swa(L, 4, 32, 32, 2, 2, 128, 128, FP16, **kw) == "streaming"
     # tiles of 16 k tokens: the flash family in tile mode (its kernels pad head dims inside)
     assert _swa(L, 16, 16, 16, 1, 1, 32, 32, FP16, **kw) == "flash"
     assert _swa(L, 64, 16, 16, 1, 1, 64, 64, BF16, **kw) == "flash"

@@ -25,7 +25,7 @@ def shim(tmp_path_factory):
     subprocess.run([cxx, "-O2", "-std=c++17", "-Wno-unknown-pragmas", "-shared", "-fPIC", os.path.join(HERE, "swa2_shim.cpp"), "-o", out],
                    check=True)
     lib = ctypes.CDLL(out)
-    lib.swa2_model.argtypes = [ctypes.c_int] * 9 + [ctypes.c_longlong] * 2 + [ctypes.c_int] * 2
+    lib.swa2_model.argtypes = [ctypes.c_int] * 10 + [ctypes.c_longlong] * 2 + [ctypes.c_int] * 2
     lib.swa2_model_message.restype = ctypes.c_char_p
     return lib
 
@@ -40,12 +40,13 @@ def _classes(WC):
     return [(d, n, -(-need // n)) for d, n in ALL if -(-need // n) <= 4]
 
 
-def _run(shim, D, NCG, npass, TR, TC, WR, WC, pad=0, ls2=1):
+def _run(shim, D, NCG, npass, TR, TC, WR, WC, pad=0, ls2=1, S=1):
+    """TC, WC in tiles of S tokens."""
     sn2 = 2 * D + pad
-    slab = (TR * TC - 1) * sn2 + 2 * D
-    scal = (TR * TC - 1) * ls2 + 1
-    rc = shim.swa2_model(D, NCG, npass, TR, TC, WR, WC, sn2, ls2, slab, scal, shim.swa2_class_lds(D, NCG, 0), shim.swa2_class_lds(D, NCG, 1))
-    assert rc == 0, f"D={D} NCG={NCG} x {npass} grid {TR}x{TC} window ({WR},{WC}) stride {sn2}: {shim.swa2_model_message().decode()}"
+    slab = (TR * TC * S - 1) * sn2 + 2 * D
+    scal = (TR * TC * S - 1) * ls2 + 1
+    rc = shim.swa2_model(D, NCG, npass, TR, TC, WR, WC, S, sn2, ls2, slab, scal, shim.swa2_class_lds(D, NCG, 0), shim.swa2_class_lds(D, NCG, 1))
+    assert rc == 0, f"D={D} NCG={NCG} x {npass} grid {TR}x{TC} tiles of {S} window ({WR},{WC}) stride {sn2}: {shim.swa2_model_message().decode()}"
 
 
 # grids of the GPU tests (ragged, one token, narrower than a band, windows wider than the grid) and of the benchmark
@@ -80,12 +81,23 @@ def test_benchmark_grids_and_strided_rows(shim):
         _run(shim, D, NCG, npass, 21, 37, 5, WC, pad=6 * D, ls2=3)
 
 
+@pytest.mark.parametrize("S", [2, 3, 4, 8, 9, 15])
+def test_tiles_of_fewer_than_16_tokens(shim, S):
+    """A token sees whole tiles: S WC + (x mod S) slots to its left, S WC + S - 1 - (x mod S) to its right."""
+    for TR, TC, WR, WC in [(5, 7, 1, 1), (9, 3, 2, 0), (3, 11, 0, 2), (10, 6, 3, 1), (1, 1, 0, 0)]:
+        need = (4 + 2 * (S * WC + S - 1) + 3) // 4
+        for D, NCG in [(64, 4), (64, 6), (128, 4), (128, 6)]:
+            npass = -(-need // NCG)
+            if npass <= 4:
+                _run(shim, D, NCG, npass, TR, TC, WR, WC, S=S)
+
+
 def test_the_model_notices_a_wrong_launch(shim):
     # a window wider than class x passes, and an LDS size below what the class needs
-    rc = shim.swa2_model(64, 4, 1, 16, 16, 3, 7, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
+    rc = shim.swa2_model(64, 4, 1, 16, 16, 3, 7, 1, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
     assert rc == 1 and b"column groups" in shim.swa2_model_message()
-    rc = shim.swa2_model(64, 6, 1, 16, 16, 3, 7, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 6, 1))
+    rc = shim.swa2_model(64, 6, 1, 16, 16, 3, 7, 1, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 6, 1))
     assert rc == 1 and b"LDS" in shim.swa2_model_message()
     # a slab one row short: the last row's copy must be caught
-    rc = shim.swa2_model(64, 4, 1, 16, 16, 3, 3, 128, 1, 16 * 16 * 128 - 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
+    rc = shim.swa2_model(64, 4, 1, 16, 16, 3, 3, 1, 128, 1, 16 * 16 * 128 - 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
     assert rc == 1 and b"global" in shim.swa2_model_message()

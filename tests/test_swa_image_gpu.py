@@ -41,10 +41,10 @@ CASES = [
     (2, 2, 16, 16, 4, 4, 1, 1, 32, 32, torch.float16, True),     # the reference demo: 4 x 4 pixel tiles, tile mode
     (1, 2, 4, 6, 8, 8, 1, 2, 64, 64, torch.bfloat16, True),      # 64-token tiles, tile mode
     (1, 1, 3, 4, 4, 12, 2, 1, 64, 128, torch.bfloat16, True),    # 48-token tiles, distinct head dims
-    (1, 2, 9, 7, 2, 2, 1, 1, 64, 64, torch.bfloat16, True),      # 4-token tiles: generic kernels
+    (1, 2, 9, 7, 2, 2, 1, 1, 64, 64, torch.bfloat16, False),     # 4-token tiles: generic kernels here, streaming kernels in token layout
     (1, 1, 5, 4, 2, 3, 1, 2, 32, 32, torch.float32, True),       # 6-token tiles, fp32 tensors
     (2, 2, 12, 20, 1, 1, 3, 2, 64, 64, torch.bfloat16, True),    # single-pixel tiles: a plain strided view, token-grid kernels
-    (1, 3, 10, 6, 1, 5, 2, 1, 128, 128, torch.bfloat16, True),   # tiles of one pixel row
+    (1, 3, 10, 6, 1, 5, 2, 1, 128, 128, torch.bfloat16, False),  # tiles of one pixel row (5 tokens): generic here, streaming in token layout
 ]
 
 

@@ -69,3 +69,36 @@ def test_tile_mode_matches_generic_kernels_bitwise_close():
         outs.append((o.float(), qg.grad.float(), kg.grad.float(), vg.grad.float()))
     for a, b in zip(*outs):
         assert (a - b).abs().max().item() <= 2e-2 * max(1.0, b.abs().max().item())
+
+
+# tiles of fewer than 16 tokens (the reference's small-tile regime, src/tiled_swa.py:611: b_size < 16): the streaming
+# token-grid kernels on the grid of token slots, a token's window given by its tile
+SMALL = [
+    # B, H, th, tw, S, WR, WC, d, dtype
+    (1, 2, 9, 11, 4, 1, 1, 64, torch.bfloat16),      # 2 x 2-pixel tiles, 3 x 3 tile window
+    (1, 2, 7, 5, 9, 1, 1, 128, torch.bfloat16),      # 3 x 3-pixel tiles
+    (2, 1, 12, 6, 2, 3, 2, 64, torch.float16),
+    (1, 1, 5, 9, 3, 0, 2, 128, torch.float16),       # window of one row
+    (1, 2, 6, 4, 8, 2, 1, 64, torch.bfloat16),
+    (1, 1, 4, 3, 15, 1, 1, 64, torch.bfloat16),      # 45-slot windows: two column passes
+    (1, 1, 3, 2, 12, 4, 4, 128, torch.bfloat16),     # window larger than the grid
+    (1, 2, 20, 1, 5, 2, 0, 64, torch.bfloat16),      # one tile per row
+]
+
+
+@pytest.mark.parametrize("B,H,th,tw,S,WR,WC,d,dtype", SMALL)
+def test_small_tiles_forward_backward(B, H, th, tw, S, WR, WC, d, dtype):
+    from dl_templates_amd import _lib
+    sw = _swa()
+    N = th * tw * S
+    q, k, v, do = orc.make_qkv(N + d + S, B, H, N, N, d, d, dtype)
+    scale = 1 / math.sqrt(d)
+    o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), S, th, tw, WR, WC, scale)
+    qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    o = sw.TiledSwa.apply(qg, kg, vg, S, th, tw, WR, WC, scale)
+    assert _lib.KERNEL_FAMILIES[_lib.load().dlt_last_kernel_family()] == "streaming"
+    o.backward(do.cuda())
+    assert _lib.KERNEL_FAMILIES[_lib.load().dlt_last_kernel_family()] == "streaming"
+    assert (o.float().cpu() - o_w).abs().max().item() <= FWD_TOL
+    errs = (_rel(qg.grad, dq_w), _rel(kg.grad, dk_w), _rel(vg.grad, dv_w))
+    assert max(errs) <= GRAD_TOL, errs
