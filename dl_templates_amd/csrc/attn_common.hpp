@@ -56,6 +56,17 @@ template <typename CT> DLT_DEV float unpack_hi(unsigned int w) {
   return (float)__builtin_bit_cast(CT, (unsigned short)(w >> 16));
 }
 
+// c + a.lo * b.lo + a.hi * b.hi for dwords of two 16-bit values (one vector instruction, fp32 accumulation)
+template <typename CT> DLT_DEV float dot2_acc(unsigned int a, unsigned int b, float c);
+template <> DLT_DEV float dot2_acc<bf16_t>(unsigned int a, unsigned int b, float c) {
+  typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
+}
+template <> DLT_DEV float dot2_acc<f16_t>(unsigned int a, unsigned int b, float c) {
+  typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
+}
+
 DLT_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 DLT_DEV float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 DLT_DEV float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }

@@ -320,11 +320,12 @@ bool swa2_compose_ok(const AttnProblem& p, const Swa1Class& c) {
   return (c.D == 64 || c.D == 128) && p.dk == c.D && p.dv == c.D && (int64_t)p.B * p.H * p.g.TR * p.g.TC >= 131072;
 }
 
-void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan) {
+void swa2_make_plan(const AttnProblem& p, Swa2Plan& plan, int band = 8) {
   { int c; swa2_split(p, c, plan.npass); }
   plan.S = p.g.S; plan.WCt = p.g.WC;
   dlt_fastdiv_make((uint32_t)p.g.S, plan.m_S, plan.s_S);
-  plan.nblk_r = (p.g.TR + 7) / 8;
+  plan.band = band;
+  plan.nblk_r = (p.g.TR + band - 1) / band;
   plan.nblk_c = (swa2_slots(p) + 15) / 16;
   dlt_fastdiv_make((uint32_t)(plan.nblk_r * plan.nblk_c), plan.m_bh, plan.s_bh);
   dlt_fastdiv_make((uint32_t)plan.nblk_c, plan.m_c, plan.s_c);
@@ -359,7 +360,10 @@ int swa2_forward(const AttnProblem& p, const AttnTensors& t, hipStream_t stream)
   if (dlt_route_note(DLT_FAMILY_STREAMING)) return DLT_OK;
   Swa2FwdArgs a;
   a.p = p;
-  swa2_make_plan(p, a.plan);
+  // head dim 128, more than one band of 8 rows: the forward kernel with two stacked patches per wave (bands of 16 rows);
+  // DLT_SWA2_SINGLE_PATCH=1 (read once per process) keeps the one-patch kernel for A/B timing and for its tests
+  static const bool single_patch = [] { const char* e = getenv("DLT_SWA2_SINGLE_PATCH"); return e != nullptr && e[0] == '1'; }();
+  swa2_make_plan(p, a.plan, p.dk == 128 && p.g.TR > 8 && !single_patch ? 16 : 8);
   a.q = t.q; a.k = t.k; a.v = t.v; a.o = t.out_o; a.lse = t.lse;
   for (int i = 0; i < 4; i++) { a.qs[i] = t.qs[i]; a.ks[i] = t.ks[i]; a.vs[i] = t.vs[i]; a.os[i] = t.os[i]; }
   for (int i = 0; i < 3; i++) a.ls[i] = t.ls[i];

@@ -4,7 +4,8 @@
 //
 // A workgroup of 8 waves owns a band of 8 grid rows x 16 grid columns; wave w owns the 4x4 patch at rows
 // 4 (w >> 2), columns 4 (w & 3).  The halo of the band (8 + 2 WR rows x HCW columns, first halo column = c0 - WC)
-// streams through LDS in chunks of 4 halo rows.
+// streams through LDS in chunks of 4 halo rows.  Stacked variant (Swa2Plan::band = 16): a band of 16 grid rows, wave w
+// owns the two 4x4 patches at rows 8 (w >> 2) and 8 (w >> 2) + 4, columns 4 (w & 3): "row group" rg below is then 0 .. 3.
 //
 // Tiles of S tokens (1 < S < 16): a grid row then holds TC = tiles * S token slots ("columns" below are slots), a token
 // in tile t sees the slots of tiles t - WCt .. t + WCt, i.e. S WCt + (x mod S) slots to its left and S WCt + S - 1 - (x mod S)
@@ -52,6 +53,7 @@ struct Swa2Plan {
   int32_t npass;   // column passes: a window of more than NCG column groups is walked in npass slices of NCG groups
   int32_t S, WCt;  // tokens per tile, window half-width in tiles
   uint32_t m_S, s_S;   // division by S
+  int32_t band;    // grid rows of a workgroup's band: 8 (one patch per wave) or 16 (two stacked patches per wave)
 };
 
 struct Swa2Geom {
@@ -80,9 +82,9 @@ DLT_HD Swa2Geom swa2_geom_at(int TR, int TC, int WR, int WC, int H, const Swa2Pl
   G.b = (int)dlt_fastdiv((uint32_t)bh, P.m_h, P.s_h);
   G.h = bh - G.b * H;
   G.TR = TR; G.TC = TC; G.WR = WR; G.WC = WC;
-  G.r0 = 8 * br;
+  G.r0 = P.band * br;
   G.c0 = 16 * (rem - br * P.nblk_c);
-  const int lo = dlt_imax(0, G.WR - G.r0), hi = dlt_imin(7 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
+  const int lo = dlt_imax(0, G.WR - G.r0), hi = dlt_imin(P.band - 1 + 2 * G.WR, G.TR - 1 - G.r0 + G.WR);
   G.ch_first = lo >> 2;
   G.ch_last = hi >> 2;
   return G;

@@ -1,6 +1,7 @@
 // Streaming token-grid kernels: instantiations and launchers for one head dim (DLT_SWA2_D), included by one
 // translation unit per head dim.
 #include "swa2_bwd_kernel.hpp"
+#include "swa2s_fwd_kernel.hpp"
 
 #define DLT_SWA2_CAT_(a, b) a##b
 #define DLT_SWA2_CAT(a, b) DLT_SWA2_CAT_(a, b)
@@ -13,6 +14,11 @@ template <typename TIO, int NCG>
 int swa2_launch_fwd_t(const Swa2FwdArgs& a, int grid, hipStream_t stream) {
   typedef Swa2Cfg<DLT_SWA2_D, NCG> C;
   auto kern = swa2_fwd_kernel<TIO, DLT_SWA2_D, NCG>;
+  if constexpr (DLT_SWA2_D == 128) {
+    if (a.plan.band == 16) kern = swa2s_fwd_kernel<TIO, DLT_SWA2_D, NCG>;   // two stacked patches per wave
+  } else if (a.plan.band != 8) {
+    return dlt_set_error(DLT_ERR_UNSUPPORTED, "streaming token-grid kernels: no instantiation for bands of %d rows", a.plan.band);
+  }
   int rc = swa2_set_lds(kern, C::LDS);
   if (rc != DLT_OK) return rc;
   dlt_timing_before(DLT_K_FWD, stream);

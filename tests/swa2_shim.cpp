@@ -25,7 +25,7 @@ int fail(const char* fmt, int a = 0, int b = 0, int c = 0, int d = 0, int e = 0,
 struct Slot { int tensor, r, c, piece; };   // tensor -1: never written
 
 template <typename C>
-int model(int TR, int TCt, int WR, int WCt, int S, int npass, int sn2, int ls2, long long slab_bytes, long long scal_elems, int lds_bytes, int lds_kv_bytes) {
+int model(int TR, int TCt, int WR, int WCt, int S, int npass, int band, int sn2, int ls2, long long slab_bytes, long long scal_elems, int lds_bytes, int lds_kv_bytes) {
   if (lds_bytes != C::LDS) return fail("launcher asks for %d bytes of LDS, the class needs %d", lds_bytes, C::LDS);
   if (lds_kv_bytes != C::LDS_KV) return fail("launcher asks for %d bytes of LDS (dK/dV), the class needs %d", lds_kv_bytes, C::LDS_KV);
   // token slots per grid row and the largest column extent of a window in slots (tiles of S tokens)
@@ -33,7 +33,9 @@ int model(int TR, int TCt, int WR, int WCt, int S, int npass, int sn2, int ls2, 
   const int ncg_total = (4 + 2 * WC + 3) >> 2;
   if (ncg_total > C::NCG * npass) return fail("window of %d column groups on a class with %d in %d column passes", ncg_total, C::NCG, npass);
   Swa2Plan P;
-  P.nblk_r = (TR + 7) / 8;
+  if (band != 8 && band != 16) return fail("bands of %d rows", band);
+  P.band = band;   // 16: two stacked patches per wave (row groups 0 .. 3)
+  P.nblk_r = (TR + band - 1) / band;
   P.nblk_c = (TC + 15) / 16;
   const int H = 1;
   P.npass = npass; P.S = S; P.WCt = WCt;
@@ -52,8 +54,8 @@ int model(int TR, int TCt, int WR, int WCt, int S, int npass, int sn2, int ls2, 
     if (G.r0 >= TR || G.c0 >= TC) return fail("workgroup %d starts outside the grid (%d, %d)", lin, G.r0, G.c0);
     if (G.ch_first > G.ch_last) return fail("workgroup %d: empty chunk range", lin);
     // ---- windows against the shared geometry routine
-    for (int wave = 0; wave < 8; wave++) {
-      const int pc = wave & 3, rg = wave >> 2;
+    for (int patch = 0; patch < band / 4 * 4; patch++) {
+      const int pc = patch & 3, rg = patch >> 2;
       for (int n = 0; n < 16; n++) {
         const Swa2Win W0 = swa2_window(G, rg, pc, n);
         const int r = G.r0 + 4 * rg + (n >> 2), c = G.c0 + 4 * pc + (n & 3);
@@ -65,7 +67,7 @@ int model(int TR, int TCt, int WR, int WCt, int S, int npass, int sn2, int ls2, 
           const Swa2Geom Gp = swa2_pass_geom(G0, C::NCG, pass);
           const Swa2Win W = swa2_pass_window(W0, C::NCG, pass);
           const int ncg = swa2_pass_ncg(WC, C::NCG, pass);
-          for (int ch = 0; ch <= (7 + 2 * WR) >> 2; ch++)
+          for (int ch = 0; ch <= (band - 1 + 2 * WR) >> 2; ch++)
             for (int hr = 0; hr < 4; hr++) {
               const int hrow = 4 * ch + hr, kr = G.r0 - WR + hrow;
               const bool row_vis = hrow >= W.rlo && hrow <= W.rhi;
@@ -250,10 +252,10 @@ extern "C" {
 // class (checked against the class constants); slab_bytes: bytes of one (batch, head) slab of a streamed tensor;
 // scal_elems: elements of one (batch, head) slab of lse2 / delta.
 // TC, WC: tiles per grid row and window half-width in tiles; S: tokens per tile
-int swa2_model(int D, int NCG, int npass, int TR, int TC, int WR, int WC, int S, int sn2, int ls2, long long slab_bytes, long long scal_elems,
-               int lds_bytes, int lds_kv_bytes) {
+int swa2_model(int D, int NCG, int npass, int band, int TR, int TC, int WR, int WC, int S, int sn2, int ls2, long long slab_bytes,
+               long long scal_elems, int lds_bytes, int lds_kv_bytes) {
   g_msg[0] = 0;
-#define CASE(d, n) if (D == d && NCG == n) return model<Swa2Cfg<d, n>>(TR, TC, WR, WC, S, npass, sn2, ls2, slab_bytes, scal_elems, lds_bytes, lds_kv_bytes);
+#define CASE(d, n) if (D == d && NCG == n) return model<Swa2Cfg<d, n>>(TR, TC, WR, WC, S, npass, band, sn2, ls2, slab_bytes, scal_elems, lds_bytes, lds_kv_bytes);
   CASE(64, 4) CASE(64, 6) CASE(64, 8) CASE(64, 10) CASE(128, 4) CASE(128, 6)
 #undef CASE
   return fail("no class (%d, %d)", D, NCG);

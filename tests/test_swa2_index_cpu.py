@@ -25,7 +25,7 @@ def shim(tmp_path_factory):
     subprocess.run([cxx, "-O2", "-std=c++17", "-Wno-unknown-pragmas", "-shared", "-fPIC", os.path.join(HERE, "swa2_shim.cpp"), "-o", out],
                    check=True)
     lib = ctypes.CDLL(out)
-    lib.swa2_model.argtypes = [ctypes.c_int] * 10 + [ctypes.c_longlong] * 2 + [ctypes.c_int] * 2
+    lib.swa2_model.argtypes = [ctypes.c_int] * 11 + [ctypes.c_longlong] * 2 + [ctypes.c_int] * 2
     lib.swa2_model_message.restype = ctypes.c_char_p
     return lib
 
@@ -40,13 +40,13 @@ def _classes(WC):
     return [(d, n, -(-need // n)) for d, n in ALL if -(-need // n) <= 4]
 
 
-def _run(shim, D, NCG, npass, TR, TC, WR, WC, pad=0, ls2=1, S=1):
-    """TC, WC in tiles of S tokens."""
+def _run(shim, D, NCG, npass, TR, TC, WR, WC, pad=0, ls2=1, S=1, band=8):
+    """TC, WC in tiles of S tokens; band: grid rows per workgroup (16: two stacked patches per wave)."""
     sn2 = 2 * D + pad
     slab = (TR * TC * S - 1) * sn2 + 2 * D
     scal = (TR * TC * S - 1) * ls2 + 1
-    rc = shim.swa2_model(D, NCG, npass, TR, TC, WR, WC, S, sn2, ls2, slab, scal, shim.swa2_class_lds(D, NCG, 0), shim.swa2_class_lds(D, NCG, 1))
-    assert rc == 0, f"D={D} NCG={NCG} x {npass} grid {TR}x{TC} tiles of {S} window ({WR},{WC}) stride {sn2}: {shim.swa2_model_message().decode()}"
+    rc = shim.swa2_model(D, NCG, npass, band, TR, TC, WR, WC, S, sn2, ls2, slab, scal, shim.swa2_class_lds(D, NCG, 0), shim.swa2_class_lds(D, NCG, 1))
+    assert rc == 0, f"D={D} NCG={NCG} x {npass} band {band} grid {TR}x{TC} tiles of {S} window ({WR},{WC}) stride {sn2}: {shim.swa2_model_message().decode()}"
 
 
 # grids of the GPU tests (ragged, one token, narrower than a band, windows wider than the grid) and of the benchmark
@@ -60,6 +60,8 @@ def test_every_class_on_small_and_ragged_grids(shim, TR, TC):
     for WR, WC in WINDOWS:
         for D, NCG, npass in _classes(WC):
             _run(shim, D, NCG, npass, TR, TC, WR, WC)
+            if D == 128:   # the forward kernel with two stacked patches per wave: bands of 16 rows
+                _run(shim, D, NCG, npass, TR, TC, WR, WC, band=16)
 
 
 def test_more_passes_than_needed_change_nothing(shim):
@@ -69,8 +71,11 @@ def test_more_passes_than_needed_change_nothing(shim):
 
 
 def test_benchmark_grids_and_strided_rows(shim):
-    _run(shim, 128, 6, 1, 128, 128, 10, 10)
-    _run(shim, 128, 6, 1, 96, 160, 10, 10)
+    for band in (8, 16):
+        _run(shim, 128, 6, 1, 128, 128, 10, 10, band=band)
+        _run(shim, 128, 6, 1, 96, 160, 10, 10, band=band)
+        _run(shim, 128, 6, 4, 128, 128, 20, 46, band=band)
+        _run(shim, 128, 4, 2, 21, 37, 5, 11, pad=768, ls2=3, band=band)
     _run(shim, 64, 4, 1, 64, 64, 6, 6)
     for D, NCG, npass, WC in [(64, 8, 1, 11), (64, 8, 1, 14), (64, 10, 1, 15), (64, 10, 1, 18), (128, 4, 2, 11), (128, 6, 2, 18),
                               (64, 6, 3, 34), (128, 6, 4, 46)]:
@@ -90,14 +95,16 @@ def test_tiles_of_fewer_than_16_tokens(shim, S):
             npass = -(-need // NCG)
             if npass <= 4:
                 _run(shim, D, NCG, npass, TR, TC, WR, WC, S=S)
+                if D == 128:
+                    _run(shim, D, NCG, npass, TR, TC, WR, WC, S=S, band=16)
 
 
 def test_the_model_notices_a_wrong_launch(shim):
     # a window wider than class x passes, and an LDS size below what the class needs
-    rc = shim.swa2_model(64, 4, 1, 16, 16, 3, 7, 1, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
+    rc = shim.swa2_model(64, 4, 1, 8, 16, 16, 3, 7, 1, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
     assert rc == 1 and b"column groups" in shim.swa2_model_message()
-    rc = shim.swa2_model(64, 6, 1, 16, 16, 3, 7, 1, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 6, 1))
+    rc = shim.swa2_model(64, 6, 1, 8, 16, 16, 3, 7, 1, 128, 1, 16 * 16 * 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 6, 1))
     assert rc == 1 and b"LDS" in shim.swa2_model_message()
     # a slab one row short: the last row's copy must be caught
-    rc = shim.swa2_model(64, 4, 1, 16, 16, 3, 3, 1, 128, 1, 16 * 16 * 128 - 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
+    rc = shim.swa2_model(64, 4, 1, 8, 16, 16, 3, 3, 1, 128, 1, 16 * 16 * 128 - 128, 256, shim.swa2_class_lds(64, 4, 0), shim.swa2_class_lds(64, 4, 1))
     assert rc == 1 and b"global" in shim.swa2_model_message()
