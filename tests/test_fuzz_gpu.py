@@ -61,6 +61,51 @@ def test_random_sliding_window_cases():
         _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
 
 
+def test_random_small_tiles_wide_windows_and_padded_head_dims():
+    """Tiles of 2 ... 15 tokens (the regime of the reference's small-tile kernel, src/tiled_swa.py:15-133, picked at :611),
+    windows of 23 ... 93 columns, head dim 128 on grids of more and fewer than 16 rows, head dims the Python operators pad,
+    two batches, three scales.  The same generator ran 1800 further cases with other seeds without a failure."""
+    from dl_templates_amd import tiled_swa as sw
+    rng = random.Random(11)
+    done = 0
+    while done < 40:
+        kind = rng.choice(["tiles", "tiles", "wide", "wide", "plain128", "pad"])
+        d = dv = rng.choice([64, 128])
+        S = 1
+        if kind == "tiles":
+            S = rng.randint(2, 15)
+            th, tw = rng.randint(1, 20), rng.randint(1, max(1, 60 // S))
+            WR, WC = rng.randint(0, 4), rng.randint(0, max(0, min(3, (44 // S) - 1)))
+        elif kind == "wide":
+            th, tw = rng.randint(1, 40), rng.randint(1, 100)
+            WR, WC = rng.randint(0, 12), rng.randint(11, 46)
+        elif kind == "plain128":
+            d = dv = 128
+            th, tw = rng.randint(1, 50), rng.randint(1, 50)
+            WR, WC = rng.randint(0, 10), rng.randint(0, 10)
+        else:
+            d = rng.choice([40, 48, 72, 80, 96, 112])
+            dv = rng.choice([d, d, 64, 128])
+            S = rng.choice([1, 1, 4, 9])
+            th, tw = rng.randint(1, 16), rng.randint(1, 24 // max(1, S // 3))
+            WR, WC = rng.randint(0, 6), rng.randint(0, 6 if S == 1 else 1)
+        dt = rng.choice([torch.bfloat16, torch.float16])
+        B, H = rng.randint(1, 2), rng.randint(1, 3)
+        N = th * tw * S
+        if N > 3000 or N * (2 * WR + 1) * (2 * WC + 1) * S > 4e6:
+            continue
+        done += 1
+        scale = rng.choice([1 / math.sqrt(d), 0.3, 0.05])
+        tag = f"case {done}: {kind} S={S} grid={th}x{tw} W=({WR},{WC}) d={d}/{dv} {dt} B={B} H={H} scale={scale:.3f}"
+        print(tag, flush=True)
+        q, k, v, do = orc.make_qkv(done * 7 + 1, B, H, N, N, d, dv, dt)
+        qg, kg, vg = (t.cuda().requires_grad_(True) for t in (q, k, v))
+        o_w, dq_w, dk_w, dv_w = orc.tiled_swa_grads(q.float(), k.float(), v.float(), do.float(), S, th, tw, WR, WC, scale)
+        o = sw.TiledSwa.apply(qg, kg, vg, S, th, tw, WR, WC, scale)
+        o.backward(do.cuda())
+        _check(tag, o, o_w, (qg.grad, kg.grad, vg.grad), (dq_w, dk_w, dv_w))
+
+
 def test_random_flash_cases():
     from dl_templates_amd import flash_attn as fa
     rng = random.Random(3)
