@@ -73,8 +73,13 @@ __global__ __launch_bounds__(SWA2_THREADS, 2) void swa2s_fwd_kernel(const Swa2Fw
   pin_loaded(qf);
   __syncthreads();
 
-  auto consume = [&](const int ch, Swa2Lds __restrict__ cur, char* __restrict__ nxt, auto more_tag) {
+  // PM: the patches that see rows of the chunk (bit 0: the upper patch, bit 1: the lower one).  The chunks of a wave come
+  // in the order "upper only" (at most one), "both", "lower only" (at most one); the one-patch bodies issue no product,
+  // mask, exponential or reduction for the other patch.
+  auto consume = [&](const int ch, Swa2Lds __restrict__ cur, char* __restrict__ nxt, auto more_tag, auto pm_tag) {
     constexpr bool more = decltype(more_tag)::value;   // a later chunk exists: its copies are issued between the products
+    constexpr int PM = decltype(pm_tag)::value;
+    constexpr bool P0 = (PM & 1) != 0, P1 = (PM & 2) != 0;
     Swa2Lds sK = cur;
     Swa2Lds sV = sK + C::REGION;
     const char* nrow = swa2_issue_row(G, ch + 1, sbase, srow, wave);
@@ -84,7 +89,7 @@ __global__ __launch_bounds__(SWA2_THREADS, 2) void swa2s_fwd_kernel(const Swa2Fw
     // wherever the own token of patch 1 is inside the grid that of patch 0 is too); a patch row outside the grid is
     // folded into the row test
     const bool row_vis[2] = {(hrow >= W[0].rlo) && (hrow <= W[0].rhi), (hrow >= W[1].rlo) && (hrow <= W[1].rhi) && W[1].cspan >= 0};
-    // ---- scores of the chunk for both patches, one column group (16 keys) at a time
+    // ---- scores of the chunk, one column group (16 keys) at a time
     float t[2][NKB][8];
     float mx[2][4];
 #pragma unroll
@@ -100,8 +105,9 @@ __global__ __launch_bounds__(SWA2_THREADS, 2) void swa2s_fwd_kernel(const Swa2Fw
       mx[p][cg & 3] = fmaxf(fmaxf(mx[p][cg & 3], t[p][kb][h4]), t[p][kb][h4 + 1]);
       mx[p][(cg + 2) & 3] = fmaxf(fmaxf(mx[p][(cg + 2) & 3], t[p][kb][h4 + 2]), t[p][kb][h4 + 3]);
     };
-    // K fragments live in ONE set of registers: piece c of the next group is requested as soon as both products of piece c
-    // of this group are issued (every fragment feeds two products, so one group of read-ahead covers the LDS latency)
+    // K fragments live in ONE set of registers: piece c of the next group is requested as soon as the products of piece c
+    // of this group are issued (with two patches every fragment feeds two products, so one group of read-ahead covers
+    // the LDS latency)
     swa2_read_a<C, 0>(sK, L, ka);
     swa2_for<0, NCG>([&](auto cgc) {
       constexpr int cg = decltype(cgc)::value;
@@ -110,66 +116,65 @@ __global__ __launch_bounds__(SWA2_THREADS, 2) void swa2s_fwd_kernel(const Swa2Fw
       f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < KC; c++) {
-        s0 = Mma<CT>::mfma(ka[c], qf[0][c], s0);
-        s1 = Mma<CT>::mfma(ka[c], qf[1][c], s1);
-        if (c == 1) {
-          if constexpr (cg > 0) mask_max(0, cg - 1, sc[0][(cg - 1) & 1]);
-        }
-        if (c == 3 || c == KC - 1) {
-          if constexpr (cg > 0) { if (c == KC - 1) mask_max(1, cg - 1, sc[1][(cg - 1) & 1]); }
+        if constexpr (P0) s0 = Mma<CT>::mfma(ka[c], qf[0][c], s0);
+        if constexpr (P1) s1 = Mma<CT>::mfma(ka[c], qf[1][c], s1);
+        if constexpr (cg > 0) {
+          if (P0 && c == 1) mask_max(0, cg - 1, sc[0][(cg - 1) & 1]);
+          if (P1 && c == KC - 1) mask_max(1, cg - 1, sc[1][(cg - 1) & 1]);
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (cg + 1 < NCG) ka[c] = swa2_lds16(sK + swa2_read_a_off<C, cg + 1>(L, c));
         __builtin_amdgcn_sched_barrier(0);
       }
-      sc[0][cg & 1] = s0;
-      sc[1][cg & 1] = s1;
+      if constexpr (P0) sc[0][cg & 1] = s0;
+      if constexpr (P1) sc[1][cg & 1] = s1;
     });
-    mask_max(0, NCG - 1, sc[0][(NCG - 1) & 1]);
-    mask_max(1, NCG - 1, sc[1][(NCG - 1) & 1]);
+    if constexpr (P0) mask_max(0, NCG - 1, sc[0][(NCG - 1) & 1]);
+    if constexpr (P1) mask_max(1, NCG - 1, sc[1][(NCG - 1) & 1]);
     // reference maxima move only when some score exceeds them by more than 2^8 after scaling (see swa2_fwd_kernel)
-    const float mloc0 = wave_max4(fmaxf(fmaxf(mx[0][0], mx[0][1]), fmaxf(mx[0][2], mx[0][3])));
-    const float mloc1 = wave_max4(fmaxf(fmaxf(mx[1][0], mx[1][1]), fmaxf(mx[1][2], mx[1][3])));
-    if (__builtin_amdgcn_ballot_w64((mloc0 - m_run[0]) * scale > 8.f)) {
-      keep_branch();
-      const float m_new = fmaxf(m_run[0], mloc0);
-      const float alpha = m_new == -INFINITY ? 1.f : fast_exp2((m_run[0] - m_new) * scale);
-      m_run[0] = m_new;
+    float mloc[2] = {-INFINITY, -INFINITY};
+    if constexpr (P0) mloc[0] = wave_max4(fmaxf(fmaxf(mx[0][0], mx[0][1]), fmaxf(mx[0][2], mx[0][3])));
+    if constexpr (P1) mloc[1] = wave_max4(fmaxf(fmaxf(mx[1][0], mx[1][1]), fmaxf(mx[1][2], mx[1][3])));
+    swa2_for<0, 2>([&](auto pc_) {
+      constexpr int p = decltype(pc_)::value;
+      if constexpr ((PM >> p) & 1) {
+        if (__builtin_amdgcn_ballot_w64((mloc[p] - m_run[p]) * scale > 8.f)) {
+          keep_branch();
+          const float m_new = fmaxf(m_run[p], mloc[p]);
+          // a lane that has not seen a key yet keeps its (zero) accumulators as they are
+          const float alpha = m_new == -INFINITY ? 1.f : fast_exp2((m_run[p] - m_new) * scale);
+          m_run[p] = m_new;
 #pragma unroll
-      for (int d = 0; d < VB; d++) acc[0][d] *= alpha;
-      lsum[0] *= alpha;
-    }
-    if (__builtin_amdgcn_ballot_w64((mloc1 - m_run[1]) * scale > 8.f)) {
-      keep_branch();
-      const float m_new = fmaxf(m_run[1], mloc1);
-      const float alpha = m_new == -INFINITY ? 1.f : fast_exp2((m_run[1] - m_new) * scale);
-      m_run[1] = m_new;
-#pragma unroll
-      for (int d = 0; d < VB; d++) acc[1][d] *= alpha;
-      lsum[1] *= alpha;
-    }
+          for (int d = 0; d < VB; d++) acc[p][d] *= alpha;
+          lsum[p] *= alpha;
+        }
+      }
+    });
     const float neg_m2[2] = {m_run[0] == -INFINITY ? 0.f : -m_run[0] * scale, m_run[1] == -INFINITY ? 0.f : -m_run[1] * scale};
-    // ---- O^T += V^T P^T for both patches, 32 keys at a time: every V^T fragment feeds two products
+    // ---- O^T += V^T P^T, 32 keys at a time: with two patches every V^T fragment feeds two products
     u32x4 va[4];
     u32x4 pb[2][2];
-    auto probs = [&](const int p, const int kb, const int half, u32x4& out) {
-#pragma unroll
-      for (int i = 4 * half; i < 4 * half + 4; i++) t[p][kb][i] = fast_exp2(fmaf(t[p][kb][i], scale, neg_m2[p]));
-      if (half == 0) { out.x = pack2<CT>(t[p][kb][0], t[p][kb][1]); out.y = pack2<CT>(t[p][kb][2], t[p][kb][3]); }
-      else { out.z = pack2<CT>(t[p][kb][4], t[p][kb][5]); out.w = pack2<CT>(t[p][kb][6], t[p][kb][7]); }
-    };
-    // V^T fragments live in one set of registers too: fragment d of the next step is requested behind the two products
-    // of fragment d of this step
+    // V^T fragments live in one set of registers too: fragment d of the next step is requested behind the products of
+    // fragment d of this step
     auto read_v = [&](auto ic, const int d) {
       constexpr int i = decltype(ic)::value, kb = i / NG, grp = i % NG;
       const u32x2 lo = swa2_lds_tr(sV + swa2_read_tr_off<C, kb>(L, 4 * grp + d, 0));
       const u32x2 hi = swa2_lds_tr(sV + swa2_read_tr_off<C, kb>(L, 4 * grp + d, 1));
       va[d].x = lo.x; va[d].y = lo.y; va[d].z = hi.x; va[d].w = hi.y;
     };
+    // probability of element e (0 .. 7) of block kb for the active patches; the pair (e - 1, e) is packed behind odd e
+    auto prob = [&](const int kb, const int e) {
+#pragma unroll
+      for (int p = 0; p < 2; p++)
+        if ((PM >> p) & 1) {
+          t[p][kb][e] = fast_exp2(fmaf(t[p][kb][e], scale, neg_m2[p]));
+          if (e & 1) pb[p][kb & 1][e >> 1] = pack2<CT>(t[p][kb][e - 1], t[p][kb][e]);
+        }
+    };
 #pragma unroll
     for (int d = 0; d < 4; d++) read_v(std::integral_constant<int, 0>{}, d);
 #pragma unroll
-    for (int p = 0; p < 2; p++) { probs(p, 0, 0, pb[p][0]); probs(p, 0, 1, pb[p][0]); }
+    for (int e = 0; e < 8; e++) prob(0, e);
     swa2_for<0, NKB * NG>([&](auto ic) {
       constexpr int i = decltype(ic)::value, kb = i / NG, grp = i % NG;
       if constexpr (more) swa2_issue_one<C, NCG + i>(st, nrow, ndst);
@@ -177,19 +182,13 @@ __global__ __launch_bounds__(SWA2_THREADS, 2) void swa2s_fwd_kernel(const Swa2Fw
       const u32x4 pk0 = pb[0][kb & 1], pk1 = pb[1][kb & 1];
 #pragma unroll
       for (int d = 0; d < 4; d++) {
-        acc[0][4 * grp + d] = Mma<CT>::mfma(va[d], pk0, acc[0][4 * grp + d]);
-        acc[1][4 * grp + d] = Mma<CT>::mfma(va[d], pk1, acc[1][4 * grp + d]);
+        if constexpr (P0) acc[0][4 * grp + d] = Mma<CT>::mfma(va[d], pk0, acc[0][4 * grp + d]);
+        if constexpr (P1) acc[1][4 * grp + d] = Mma<CT>::mfma(va[d], pk1, acc[1][4 * grp + d]);
         if constexpr (kb + 1 < NKB) {
-          // the exponentials of the next 32 keys, EPS elements per patch behind every pair of products
+          // the exponentials of the next 32 keys, EPS elements per patch behind every fragment's products
           constexpr int EPS = 2 / NG;
 #pragma unroll
-          for (int e = (4 * grp + d) * EPS; e < (4 * grp + d + 1) * EPS; e++) {
-#pragma unroll
-            for (int p = 0; p < 2; p++) {
-              t[p][kb + 1][e] = fast_exp2(fmaf(t[p][kb + 1][e], scale, neg_m2[p]));
-              if (e & 1) pb[p][(kb + 1) & 1][e >> 1] = pack2<CT>(t[p][kb + 1][e - 1], t[p][kb + 1][e]);
-            }
-          }
+          for (int e = (4 * grp + d) * EPS; e < (4 * grp + d + 1) * EPS; e++) prob(kb + 1, e);
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (i + 1 < NKB * NG) read_v(std::integral_constant<int, i + 1>{}, d);
@@ -198,34 +197,52 @@ __global__ __launch_bounds__(SWA2_THREADS, 2) void swa2s_fwd_kernel(const Swa2Fw
       if constexpr (grp == NG - 1) {
         // row sums of the rounded probabilities (the values the products above use)
 #pragma unroll
-        for (int j = 0; j < 4; j++) { lsum[0] = dot2_acc<CT>(pk0[j], one2, lsum[0]); lsum[1] = dot2_acc<CT>(pk1[j], one2, lsum[1]); }
+        for (int j = 0; j < 4; j++) {
+          if constexpr (P0) lsum[0] = dot2_acc<CT>(pk0[j], one2, lsum[0]);
+          if constexpr (P1) lsum[1] = dot2_acc<CT>(pk1[j], one2, lsum[1]);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     });
   };
 
-  // chunks that hold visible rows of either patch (contiguous; a patch outside the grid has an empty range)
-  const bool ok0 = W[0].ch_lo <= W[0].ch_hi, ok1 = W[1].ch_lo <= W[1].ch_hi;
-  const int w_lo = ok1 ? dlt_imin(W[0].ch_lo, W[1].ch_lo) : W[0].ch_lo;
-  const int w_hi = ok1 ? dlt_imax(W[0].ch_hi, W[1].ch_hi) : W[0].ch_hi;
-  (void)ok0;
-  const int act_lo = dlt_imax(G.ch_first, w_lo), act_hi = dlt_imin(G.ch_last - 1, w_hi);
+  // Chunk ranges of the two patches (a patch outside the grid has an empty range; the lower patch starts and ends at or
+  // after the upper one, and their ranges touch or overlap): upper only, both, lower only.  One loop per kind, in that
+  // order, and copy-only rounds before and after, keep the accumulators in place (see swa2_fwd_kernel).
+  const bool ok1 = W[1].ch_lo <= W[1].ch_hi;
+  const int a_lo = W[0].ch_lo, a_hi = W[0].ch_hi;
+  const int b_lo = ok1 ? W[1].ch_lo : a_hi + 1, b_hi = ok1 ? W[1].ch_hi : a_hi;
+  const int w_lo = a_lo;
+  const int both_lo = dlt_imax(a_lo, b_lo), both_hi = dlt_imin(a_hi, b_hi);
   auto copy_only = [&](int ch) {
     swa2_issue(st, G, ch + 1, sbase, srow, smem + ((ch + 1) & 1) * C::BUF, wave);
     swa2_wait_copies();
     __syncthreads();
   };
+  auto round = [&](int ch, auto pm_tag) {
+    consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF, smem + ((ch + 1) & 1) * C::BUF, std::true_type{}, pm_tag);
+    swa2_wait_copies();
+    __syncthreads();
+  };
+  typedef std::integral_constant<int, 1> PmUpper;
+  typedef std::integral_constant<int, 2> PmLower;
+  typedef std::integral_constant<int, 3> PmBoth;
   for (int pass = 0;;) {
     int ch = G.ch_first;
-    for (; ch < G.ch_last && ch < act_lo; ch++) copy_only(ch);
-    for (; ch <= act_hi; ch++) {
-      consume(ch, (Swa2Lds)smem + (ch & 1) * C::BUF, smem + ((ch + 1) & 1) * C::BUF, std::true_type{});
-      swa2_wait_copies();
-      __syncthreads();
-    }
+    for (; ch < G.ch_last && ch < w_lo; ch++) copy_only(ch);
+    for (; ch < G.ch_last && ch <= a_hi && ch < both_lo; ch++) round(ch, PmUpper{});
+    for (; ch < G.ch_last && ch <= both_hi; ch++) round(ch, PmBoth{});
+    for (; ch < G.ch_last && ch <= b_hi; ch++) round(ch, PmLower{});
     for (; ch < G.ch_last; ch++) copy_only(ch);
-    if (G.ch_last >= w_lo && G.ch_last <= w_hi)
-      consume(G.ch_last, (Swa2Lds)smem + (G.ch_last & 1) * C::BUF, smem + ((G.ch_last + 1) & 1) * C::BUF, std::false_type{});
+    {
+      const int cl = G.ch_last;
+      const bool in0 = cl >= a_lo && cl <= a_hi, in1 = ok1 && cl >= b_lo && cl <= b_hi;
+      Swa2Lds cur = (Swa2Lds)smem + (cl & 1) * C::BUF;
+      char* nxt = smem + ((cl + 1) & 1) * C::BUF;
+      if (in0 && in1) consume(cl, cur, nxt, std::false_type{}, PmBoth{});
+      else if (in0) consume(cl, cur, nxt, std::false_type{}, PmUpper{});
+      else if (in1) consume(cl, cur, nxt, std::false_type{}, PmLower{});
+    }
     __syncthreads();   // every wave is done with both chunk buffers
     if (++pass >= a.plan.npass) break;
     G = swa2_pass_geom(G0, NCG, pass);
