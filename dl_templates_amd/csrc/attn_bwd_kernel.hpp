@@ -67,7 +67,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const BwdArgs a) {
   for (int off = 1; off < CH; off <<= 1) part += __shfl_xor(part, off);
   if (tok < total && c == 0) {
     const int b = (int)(bh / a.p.H), h = (int)(bh - (int64_t)b * a.p.H);
-    a.delta[b * a.ls[0] + h * a.ls[1] + nn * a.ls[2]] = part;
+    store_stream4(a.delta + (b * a.ls[0] + h * a.ls[1] + nn * a.ls[2]), part);
   }
 }
 

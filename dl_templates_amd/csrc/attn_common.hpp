@@ -149,6 +149,15 @@ DLT_DEV float wave_sum4(float v) {
 // ---- global <-> register moves of 8 consecutive head dims -------------------------------
 template <typename TIO, typename CT> struct Io;
 
+// Stores of results that this kernel does not read again are issued as streaming ("nontemporal") stores: they are
+// written through towards memory while the kernel still runs.  A plain store leaves its line dirty in the L2 of its XCD
+// until the write-back at the end of the kernel, which the next kernel of the stream waits for: measured between two
+// kernels of one stream, 1.1 us when the first writes nothing at its end, 5.0 us after 8 MB, 12.7 us after 26 MB.
+DLT_DEV void store_stream16(void* p, const u32x4& v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p)); }
+DLT_DEV void store_stream8(void* p, const u32x2& v) { __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p)); }
+DLT_DEV void store_stream4(float* p, float v) { __builtin_nontemporal_store(v, p); }
+DLT_DEV void store_stream16f(float* p, float a, float b, float c, float d) { __builtin_nontemporal_store(f32x4{a, b, c, d}, reinterpret_cast<f32x4*>(p)); }
+
 template <typename T> struct Io<T, T> {  // 2-byte element, same compute type
   static DLT_DEV u32x4 load8(const T* p, bool vec, int64_t sd, int nvalid) {
     if (vec) return *reinterpret_cast<const u32x4*>(p);
@@ -164,7 +173,7 @@ template <typename T> struct Io<T, T> {  // 2-byte element, same compute type
     if (vec) {
       u32x4 r;
       r.x = pack2<T>(v[0], v[1]); r.y = pack2<T>(v[2], v[3]); r.z = pack2<T>(v[4], v[5]); r.w = pack2<T>(v[6], v[7]);
-      *reinterpret_cast<u32x4*>(p) = r;
+      store_stream16(p, r);
     } else {
 #pragma unroll
       for (int j = 0; j < 8; j++) if (j < nvalid) p[j * sd] = (T)v[j];
@@ -189,8 +198,8 @@ template <> struct Io<float, bf16_t> {  // fp32 in HBM, bf16 arithmetic
   }
   static DLT_DEV void store8(float* p, const float* v, bool vec, int64_t sd, int nvalid) {
     if (vec) {
-      reinterpret_cast<float4*>(p)[0] = make_float4(v[0], v[1], v[2], v[3]);
-      reinterpret_cast<float4*>(p)[1] = make_float4(v[4], v[5], v[6], v[7]);
+      store_stream16f(p, v[0], v[1], v[2], v[3]);
+      store_stream16f(p + 4, v[4], v[5], v[6], v[7]);
     } else {
 #pragma unroll
       for (int j = 0; j < 8; j++) if (j < nvalid) p[j * sd] = v[j];

@@ -181,7 +181,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const FwdArgs a) {
       for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * inv);
     const int xq = wfirst + 16 * p + n;
     if (g == 0 && xq <= xlast)
-      a.lse[b * a.ls[0] + h * a.ls[1] + ((int64_t)r_own * G.XLq + xq) * a.ls[2]] = m_run[p] + fast_log2(lt);
+      store_stream4(a.lse + (b * a.ls[0] + h * a.ls[1] + ((int64_t)r_own * G.XLq + xq) * a.ls[2]), m_run[p] + fast_log2(lt));
   }
   __syncthreads();
   store_tile<TIO, TL, DV>(sO, PO, ob, tok_addr(a.os, a.p.tm), a.os[3], a.p.dv, a.o_vec != 0, OWN,

@@ -623,7 +623,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_fwd_kernel(co
     for (int d = 0; d < VB; d++)
 #pragma unroll
       for (int i = 0; i < 4; i++) orow[16 * d + 4 * g + i] = (TL)(acc[p][d][i] * inv);
-    if (g == 0 && tq[p] >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]] = m_run[p] * scale + fast_log2(lt);
+    if (g == 0 && tq[p] >= 0) store_stream4(a.lse + (b * a.ls[0] + h * a.ls[1] + tq[p] * a.ls[2]), m_run[p] * scale + fast_log2(lt));
   }
   __syncthreads();
   int tw = tid;   // opaque copy: keeps the tile writer's addresses out of the registers that live across the chunk loop
@@ -712,7 +712,7 @@ __global__ __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) void flashd_bwd_q_kernel(
         for (int j = 0; j < 8; j++) part += fo[j] * fd[j];
       }
       del_n[p] = wave_sum4(part);
-      if (g == 0 && tq >= 0) a.delta_out[off] = del_n[p];
+      if (g == 0 && tq >= 0) store_stream4(a.delta_out + off, del_n[p]);
     } else {
       del_n[p] = tq >= 0 ? a.delta[off] : 0.f;
     }

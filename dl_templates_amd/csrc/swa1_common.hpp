@@ -399,7 +399,7 @@ DLT_DEV void swa1_store_own(char* sW, const f32x4 (&acc)[D / 16], float mul, TIO
         }
         v = pack8<CT>(self);
       }
-      if (ok[it]) *reinterpret_cast<u32x4*>(base + (int64_t)tok[it] * sn + 8 * c) = v;
+      if (ok[it]) store_stream16(base + (int64_t)tok[it] * sn + 8 * c, v);
     }
   } else {
 #pragma unroll

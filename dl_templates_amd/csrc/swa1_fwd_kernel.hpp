@@ -153,8 +153,8 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
     for (int c = 0; c < KC; c++) {
       const int ch = 4 * c + g;
       if (8 * ch < a.p.dk) {
-        *reinterpret_cast<u32x4*>(qr + 8 * ch) = qf[c];
-        *reinterpret_cast<u32x4*>(kr + 8 * ch) = kf_own[c];
+        store_stream16(qr + 8 * ch, qf[c]);
+        store_stream16(kr + 8 * ch, kf_own[c]);
       }
     }
   }
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(256, (D <= 64 ? (CR == 4 ? (NCGMAX <= 4 ? 4 : 3) : 
   const float lt = wave_sum4(ONES ? acc_l[0] : l_run);   // ones product: only lane group 0 is non-zero
   const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
   const int64_t tq = own_token(16 * wave + n);
-  if (g == 0 && tq >= 0) a.lse[b * a.ls[0] + h * a.ls[1] + tq * a.ls[2]] = m_run * scale + fast_log2(lt);
+  if (g == 0 && tq >= 0) store_stream4(a.lse + (b * a.ls[0] + h * a.ls[1] + tq * a.ls[2]), m_run * scale + fast_log2(lt));
   if (a.o_vec != 0) {  // the loop ended with a workgroup barrier: the chunk buffers are free
     swa1_store_own<TIO, CT, D>(smem + wave * 16 * PO, acc, inv, ob, a.os[2], a.p.dv, G, wave, lane, no_rope, false);
     return;

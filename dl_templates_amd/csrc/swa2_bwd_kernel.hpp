@@ -80,7 +80,7 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_bwd_q(D)) void swa2_bwd_q_ke
         part = fmaf(unpack_hi<CT>(of[c][j]), unpack_hi<CT>(dof[c][j]), part);
       }
     del_n = wave_sum4(part);
-    if (g == 0 && tq >= 0) delb[(int64_t)tq * a.ls[2]] = del_n;
+    if (g == 0 && tq >= 0) store_stream4(delb + (int64_t)tq * a.ls[2], del_n);
   }
   const Swa2Win W0 = swa2_window(G0, rg, pc, n);
   Swa2Win W = W0;

@@ -162,7 +162,7 @@ DLT_DEV void swa2_store_own(char* sW, const f32x4 (&acc)[C::VB], float mul, TIO*
     const int row = lane / C::PIECES + RPI * it;
     const u32x4 v = lds_read16(sW + swa2_tile_read_off<C>(row, c));
     const int r = r_p + (row >> 2), col = c_p + (row & 3);
-    if (r < G.TR && col < G.TC) *reinterpret_cast<u32x4*>(base + (int64_t)(r * G.TC + col) * sn + 8 * c) = v;
+    if (r < G.TR && col < G.TC) store_stream16(base + (int64_t)(r * G.TC + col) * sn + 8 * c, v);
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();

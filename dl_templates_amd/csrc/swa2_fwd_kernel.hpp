@@ -199,6 +199,6 @@ __global__ __launch_bounds__(SWA2_THREADS, swa2_occ_fwd(D)) void swa2_fwd_kernel
   // ---- epilogue (the loop ended with a barrier: the chunk buffers are free)
   const float lt = wave_sum4(acc_l[0]);   // only row 0 of the ones operand is set: the other lane groups hold zeros
   const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
-  if (g == 0 && tq >= 0) lseb[(int64_t)tq * ls2] = m_run * scale + fast_log2(lt);
+  if (g == 0 && tq >= 0) store_stream4(lseb + (int64_t)tq * ls2, m_run * scale + fast_log2(lt));
   swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, acc, inv, ob, os2, G, r_p, c_p, lane);
 }

@@ -260,7 +260,7 @@ __global__ __launch_bounds__(SWA2_THREADS, 2) void swa2s_fwd_kernel(const Swa2Fw
   for (int p = 0; p < 2; p++) {
     const float lt = wave_sum4(lsum[p]);
     const float inv = lt > 0.f ? fast_rcp(lt) : 0.f;
-    if (g == 0 && tq[p] >= 0) lseb[(int64_t)tq[p] * ls2] = m_run[p] * scale + fast_log2(lt);
+    if (g == 0 && tq[p] >= 0) store_stream4(lseb + (int64_t)tq[p] * ls2, m_run[p] * scale + fast_log2(lt));
     swa2_store_own<C, TIO, CT>(smem + wave * C::TILE, acc[p], inv, ob, os2, G, r_p[p], c_p, lane);
   }
 }

@@ -112,7 +112,7 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_bwd_q_kernel(const SwamBwdA
       for (int j = 0; j < 8; j++) part += fo[j] * fd[j];
     }
     const float del = wave_sum4(part);
-    if (g == 0 && w.tok >= 0) delb[(int64_t)w.tok * ls2] = del;
+    if (g == 0 && w.tok >= 0) store_stream4(delb + (int64_t)w.tok * ls2, del);
     return del;
   };
   // rotary indices of the two tile rows a lane stores in step s

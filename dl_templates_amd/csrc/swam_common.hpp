@@ -319,5 +319,5 @@ template <typename TIO>
 DLT_DEV void swam_store_rows(TIO* base, int64_t sn, const int (&tok)[2], int lane, const u32x4 (&v)[2]) {
 #pragma unroll
   for (int it = 0; it < 2; it++)
-    if (tok[it] >= 0) *reinterpret_cast<u32x4*>(base + (int64_t)tok[it] * sn + 8 * (lane & 7)) = v[it];
+    if (tok[it] >= 0) store_stream16(base + (int64_t)tok[it] * sn + 8 * (lane & 7), v[it]);
 }

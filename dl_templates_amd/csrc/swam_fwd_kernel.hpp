@@ -122,18 +122,18 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
     swam_rotate_pair<CT>(it.v[0], it.v[1], tb, false);
     if (save_rot && st.own_col && it.row >= G.r0 && it.row < G.r0 + band && it.row < G.TR) {
       char* p = krb + ((uint32_t)((it.row * G.TC + st.cc) * sn2kr) + 32 * st.qd);
-      *reinterpret_cast<u32x4*>(p) = it.v[0];
-      *reinterpret_cast<u32x4*>(p + 16) = it.v[1];
-      *reinterpret_cast<u32x4*>(p + 64) = it.v[2];
-      *reinterpret_cast<u32x4*>(p + 80) = it.v[3];
+      store_stream16(p, it.v[0]);
+      store_stream16(p + 16, it.v[1]);
+      store_stream16(p + 64, it.v[2]);
+      store_stream16(p + 80, it.v[3]);
     }
   };
   auto rotate_q = [&](SwamOwn& w, const SwamTab& tb) {
     swam_own_rotate<CT>(w, tb, g, false);
     if (save_rot && w.tok >= 0) {
       TIO* qr = qrb + (int64_t)w.tok * qrs2;
-      *reinterpret_cast<u32x4*>(qr + 8 * g) = w.f[0];
-      *reinterpret_cast<u32x4*>(qr + 32 + 8 * g) = w.f[1];
+      store_stream16(qr + 8 * g, w.f[0]);
+      store_stream16(qr + 32 + 8 * g, w.f[1]);
     }
   };
   auto commit_chunk = [&](const SwamItem& it, int c) {
@@ -332,7 +332,7 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
     return w;
   };
   auto store_o = [&](const OutRows& w, const SwamFwdOut& r) {
-    if (g == 0 && qo.tok >= 0) lseb[(int64_t)qo.tok * ls2] = r.lse2;
+    if (g == 0 && qo.tok >= 0) store_stream4(lseb + (int64_t)qo.tok * ls2, r.lse2);
     int ln = lane;
     asm volatile("" : "+v"(ln));
     swam_store_rows<TIO>(ob, os2, w.tok, ln, w.v);
