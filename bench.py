@@ -530,7 +530,10 @@ def main():
     value = flops_step / (ms_step * 1e-3) / 1e12
 
     kflops = wl.kernel_flops()
-    dom = max((k for k in kb if k in kflops), key=lambda k: kb[k]["avg_ms"])
+    # the dominant kernel: the longest one; kernels within 3 % of it (run-to-run noise) count as equally long, and among
+    # those the one that does the most algorithmic work stands for the step
+    longest = max(kb[k]["avg_ms"] for k in kb if k in kflops)
+    dom = max((k for k in kb if k in kflops and kb[k]["avg_ms"] >= 0.97 * longest), key=lambda k: kflops[k])
     # A pair of HIP events around a launch adds the markers' own cost to every kernel: the kernels of a step, bracketed,
     # sum to more than the step takes back to back without markers.  That excess, spread evenly over the step's launches,
     # is taken off again, so that `avg_launch_ms` is the kernel's share of the un-instrumented step (what rocprofv3's
