@@ -184,7 +184,21 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
         commit_chunk(it[c], c);
       }
     }
-    if (ROT) {
+    if (ROT && TL) {
+      // the tables are in LDS: chunk by chunk as the loads return, the K items rotated on their way
+#pragma unroll
+      for (int c = 0; c < SWAM_NSLOT; c++) {
+        swam_pin(it[c]);
+        if ((c & 1) == kpar) {
+          swam_tab_get<true>(tb[0], idk[c >> 1], st.qd, rope, tabs);
+          rotate_k(it[c], tb[0]);
+        }
+        commit_chunk(it[c], c);
+      }
+      swam_own_pin(qo, ROT);
+      swam_tab_get<true>(tbq, idq, g >> 1, rope, tabs);
+      rotate_q(qo, tbq);
+    } else if (ROT) {
       // V chunks need no rotation and are written as they arrive; the K chunks wait for their table rows, which were
       // requested last (static register indexing: the K items of this half are chunks kpar, kpar + 2, kpar + 4)
       if (kpar == 0) {
@@ -198,12 +212,6 @@ __global__ __launch_bounds__(SWAM_THREADS) void swam_fwd_kernel(const SwamFwdArg
 #pragma unroll
       for (int c = 0; c < SWAM_NSLOT; c++) swam_pin(it[c]);
       swam_own_pin(qo, ROT);
-      if (TL) {
-#pragma unroll
-        for (int i = 0; i < 3; i++)
-          if (kpar + 2 * i < SWAM_NSLOT) swam_tab_get<true>(tb[i], idk[i], st.qd, rope, tabs);
-        swam_tab_get<true>(tbq, idq, g >> 1, rope, tabs);
-      }
       if (kpar == 0) {
         rotate_k(it[0], tb[0]); commit_chunk(it[0], 0);
         rotate_k(it[2], tb[1]); commit_chunk(it[2], 2);
